@@ -1,0 +1,219 @@
+"""Pins for oracle.stream (restating context_manager.py).
+
+The reference holds no tests or fixtures for this path, so the stateful oracle
+is pinned against an independent derivation in absolute positions
+(oracle.absolute), closed forms, invariances and textbook special cases.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle.absolute import run_absolute, block_boundaries
+from oracle.rope import RopeOracle
+from oracle.stream import StreamOracle, UnitCacheModel
+
+GEOM = dict(n_init=4, n_local=32, block_size=8, max_cached_block=4, topk=2, exc_block_size=16, repr_topk=2)
+
+
+def _stream(T, H=4, Hkv=2, D=16, seed=0, B=1):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(B, H, T, D, generator=g), torch.randn(B, Hkv, T, D, generator=g),
+            torch.randn(B, Hkv, T, D, generator=g))
+
+
+def _run(q, k, v, calls, base=10000, **over):
+    kw = dict(GEOM, **over)
+    cm = StreamOracle(RopeOracle(q.shape[-1], base=base), **kw)
+    outs, pos = [], 0
+    for L in calls:
+        outs.append(cm.append(q[:, :, pos:pos + L], k[:, :, pos:pos + L], v[:, :, pos:pos + L]))
+        pos += L
+    return torch.cat(outs, dim=-2), cm
+
+
+@pytest.mark.parametrize("calls", [[200], [64, 64, 72], [16] * 12 + [8], [5, 1, 1, 40, 1, 90, 33, 29], [1] * 70])
+def test_matches_absolute_position_derivation(calls):
+    T = sum(calls)
+    q, k, v = _stream(T, seed=len(calls))
+    out, cm = _run(q, k, v, calls)
+    kw = {a: GEOM[a] for a in ("n_init", "n_local", "block_size", "topk", "exc_block_size", "repr_topk")}
+    ref = run_absolute(q[0], k[0], v[0], calls, **kw)
+    assert [b["selected"][0] for b in cm.block_trace] == ref["selected"]
+    assert torch.allclose(out[0].double(), ref["out"], atol=2e-4), float((out[0].double() - ref["out"]).abs().max())
+    for mine, theirs in zip(cm.reps[0], ref["reps"]):
+        assert torch.allclose(mine.double(), theirs, atol=1e-5)
+    assert cm.length == T == cm.size()
+
+
+def test_geometry_without_gqa_and_odd_sizes():
+    calls = [37, 50, 3, 61]
+    q, k, v = _stream(sum(calls), H=3, Hkv=3, D=8, seed=7)
+    over = dict(n_init=3, n_local=20, block_size=5, topk=3, exc_block_size=7, repr_topk=1, max_cached_block=3)
+    out, cm = _run(q, k, v, calls, **over)
+    kw = {a: over[a] for a in ("n_init", "n_local", "block_size", "topk", "exc_block_size", "repr_topk")}
+    ref = run_absolute(q[0], k[0], v[0], calls, **kw)
+    assert [b["selected"][0] for b in cm.block_trace] == ref["selected"]
+    assert torch.allclose(out[0].double(), ref["out"], atol=2e-4)
+
+
+def test_closed_forms_for_init_units_and_lengths():
+    T = 333
+    q, k, v = _stream(T, seed=3)
+    _, cm = _run(q, k, v, [T])
+    n_init, n_local, bs, exc, topk = (GEOM[x] for x in ("n_init", "n_local", "block_size", "exc_block_size", "topk"))
+    assert torch.equal(cm.init_k, k[:, :, :n_init])
+    assert cm.n_units == (T - n_init - n_local) // bs == len(cm.units[0])
+    for u, (uk, uv) in enumerate(cm.units[0]):
+        assert torch.equal(uk, k[0, :, n_init + u * bs:n_init + (u + 1) * bs])
+        assert torch.equal(uv, v[0, :, n_init + u * bs:n_init + (u + 1) * bs])
+    assert torch.equal(cm.win_k, k[:, :, -n_local:])
+    assert n_local <= cm.rem_k.shape[-2] < n_local + bs
+    assert torch.equal(cm.rem_k, k[:, :, n_init + cm.n_units * bs:])
+    for (b0, b1), tr in zip(block_boundaries([T], exc), cm.block_trace):
+        assert tr["n_units"] == max(0, (b0 - n_init - n_local) // bs)
+        assert tr["init_len"] == min(n_init, max(b0 - n_local, 0))
+        assert tr["local_len"] == b1 - max(b0 - n_local, 0)
+        assert tr["global_len"] <= topk * bs + n_init + exc + bs - 1
+        assert tr["global_len"] == len(tr["selected"][0]) * bs + tr["init_len"] + tr["overflow"]
+
+
+def test_invariant_under_exc_aligned_call_splitting():
+    T = 256
+    q, k, v = _stream(T, seed=5)
+    one, cm1 = _run(q, k, v, [T])
+    two, _ = _run(q, k, v, [128, 128])
+    many, cm3 = _run(q, k, v, [16] * 16)
+    assert torch.allclose(one, two, atol=1e-5) and torch.allclose(one, many, atol=1e-5)
+    assert [b["selected"] for b in cm1.block_trace] == [b["selected"] for b in cm3.block_trace]
+
+
+def test_stream_inside_window_is_causal_sdpa_with_standard_rope():
+    T = 30
+    q, k, v = _stream(T, seed=6)
+    out, cm = _run(q, k, v, [T], exc_block_size=32)
+    rope = RopeOracle(16)
+    qr, kr = rope.rotate(q, range(T)), rope.rotate(k, range(T))
+    want = F.scaled_dot_product_attention(qr, kr.repeat_interleave(2, 1), v.repeat_interleave(2, 1), is_causal=True)
+    assert torch.allclose(out, want, atol=1e-5)
+    assert cm.n_units == 0 and cm.init_k.shape[-2] == 0
+
+
+def test_large_topk_attends_every_past_token():
+    """topk >= #units: every token outside the window is attended at the fixed distance."""
+    T = 120
+    q, k, v = _stream(T, H=2, Hkv=2, D=8, seed=8)
+    out, cm = _run(q, k, v, [T], topk=64, max_cached_block=64, exc_block_size=1, n_local=16, n_init=4)
+    rope = RopeOracle(8)
+    i = T - 1
+    ql = rope.rotate(q[0, :, i:i + 1], [15])
+    kl = rope.rotate(k[0, :, i - 15:i + 1], range(16))
+    qg = rope.rotate(q[0, :, i:i + 1], [15])
+    cursor = 4 + cm.block_trace[-1]["n_units"] * 8
+    old = list(range(0, i - 15))
+    assert cursor <= i - 15
+    logits = torch.cat((ql @ kl.transpose(-1, -2), qg @ k[0, :, old].transpose(-1, -2)), dim=-1) / 8 ** 0.5
+    p = torch.softmax(logits, dim=-1)
+    want = p[..., :16] @ v[0, :, i - 15:i + 1] + p[..., 16:] @ v[0, :, old]
+    assert torch.allclose(out[0, :, i:i + 1], want, atol=1e-5)
+
+
+def test_early_queries_double_count_overflow_tokens():
+    """Overflow tokens sit in the global stage of every query of the block and are
+    still inside the local window of the block's early queries."""
+    T = 32 + 16
+    q, k, v = _stream(T, H=1, Hkv=1, D=8, seed=9)
+    out, cm = _run(q, k, v, [32, 16], n_init=0, topk=1, max_cached_block=1, block_size=64)
+    tr = cm.block_trace[-1]
+    assert tr["overflow"] == 16 and tr["n_units"] == 0
+    rope = RopeOracle(8)
+    i = 32                                           # first query of the second block
+    ql = rope.rotate(q[0, :, i:i + 1], [31])
+    kl = rope.rotate(k[0, :, 1:33], range(32))
+    logits = torch.cat((ql @ kl.transpose(-1, -2), ql @ k[0, :, 0:16].transpose(-1, -2)), dim=-1) / 8 ** 0.5
+    p = torch.softmax(logits, dim=-1)
+    want = p[..., :32] @ v[0, :, 1:33] + p[..., 32:] @ v[0, :, 0:16]
+    assert torch.allclose(out[0, :, i:i + 1], want, atol=1e-5)
+
+
+def test_cache_policy_and_capacity_never_change_results():
+    T = 300
+    q, k, v = _stream(T, seed=10)
+    ref, _ = _run(q, k, v, [T])
+    for over in (dict(max_cached_block=2), dict(max_cached_block=16),
+                 dict(cache_strategy="lru-s", score_decay=0.5), dict(cache_strategy="fifo")):
+        got, _ = _run(q, k, v, [T], **over)
+        assert torch.equal(ref, got), over
+
+
+def test_batch_rows_are_independent_and_perhead_splits_heads():
+    T = 150
+    q, k, v = _stream(T, seed=11, B=2)
+    both, _ = _run(q, k, v, [T])
+    for b in range(2):
+        single, _ = _run(q[b:b + 1], k[b:b + 1], v[b:b + 1], [T])
+        assert torch.allclose(both[b:b + 1], single, atol=1e-6)
+    ph, cm = _run(q[:1], k[:1], v[:1], [T], perhead=True)
+    assert ph.shape == (1, 4, T, 16) and cm.B == 4 and cm.H == 1
+    h2, _ = _run(q[:1, 2:3], k[:1, 1:2], v[:1, 1:2], [T])
+    assert torch.allclose(ph[:, 2:3], h2, atol=1e-6)
+
+
+def test_representative_special_cases():
+    T = 200
+    q, k, v = _stream(T, seed=12)
+    # repr_topk == block_size: representative is the plain mean of the unit's keys
+    _, cm = _run(q, k, v, [T], repr_topk=8)
+    want = k[0, :, 4:12].mean(dim=1).repeat_interleave(2, dim=0).reshape(-1)
+    assert torch.allclose(cm.reps[0][0], want, atol=1e-6)
+    # repr_topk == 1: representative is the single best-scored key per query head
+    _, cm = _run(q, k, v, [T], repr_topk=1)
+    tr = cm.unit_trace[0]
+    best = tr["score"].argmax(dim=-1)
+    for h in range(4):
+        assert torch.equal(cm.reps[0][0].reshape(4, 16)[h], k[0, h // 2, 4 + int(best[h])])
+
+
+def test_scores_are_probability_mass():
+    """Every query spreads mass 1 over local+global keys, so the local column sums of a
+    block whose global stage is empty add up to the number of queries."""
+    T = 24
+    q, k, v = _stream(T, seed=13)
+    _, cm = _run(q, k, v, [T], exc_block_size=8)
+    assert torch.allclose(cm.rem_score.sum(-1), torch.full((1, 4), float(T)), atol=1e-4)
+
+
+def test_hooks_override_choices():
+    T = 200
+    q, k, v = _stream(T, seed=14)
+    forced = [0, 1]
+    out, cm = _run(q, k, v, [T], topk_hook=lambda blk, u, s: forced)
+    assert all(b["selected"][0] == forced for b in cm.block_trace if b["n_units"] > 2)
+
+
+def test_cache_model_lru_hand_worked():
+    c = UnitCacheModel(3, "lru")
+    c.touch([0, 1])          # stamps 0:1 1:1
+    c.touch([2])             # 2:2
+    c.touch([0])             # 0:3
+    c.touch([3])             # must evict one: lowest stamp is unit 1
+    assert c.events[-1]["evicted"] == [1] and set(c.cached) == {0, 2, 3}
+    c.touch([1, 4])          # two misses, capacity 3 -> evict 2 (stamp 2) then 0 (stamp 3)
+    assert c.events[-1]["evicted"] == [2, 0] and set(c.cached) == {3, 1, 4}
+    c.touch([3, 1])          # hits only
+    assert c.events[-1] == dict(selected=[1, 3], misses=[], evicted=[])
+
+
+def test_cache_model_ties_break_in_insertion_order_and_selected_are_kept():
+    c = UnitCacheModel(3, "lru")
+    c.touch([5, 3, 4])       # all stamp 1, insertion order 5,3,4
+    c.touch([9, 3])          # one miss -> evict first unselected in insertion order: 5
+    assert c.events[-1]["evicted"] == [5]
+    f = UnitCacheModel(2, "fifo")
+    f.touch([0]); f.touch([1]); f.touch([0]); f.touch([2])
+    assert f.events[-1]["evicted"] == [0]            # fifo ignores the re-use of unit 0
+    s = UnitCacheModel(2, "lru-s", 0.5)
+    s.touch([0, 1]); s.add_scores([0, 1], [1.0, 4.0])
+    s.touch([2])                                     # evicts the lower-scored unit 0
+    assert s.events[-1]["evicted"] == [0]
+    with pytest.raises(AssertionError):
+        UnitCacheModel(1, "lru").touch([0, 1])
