@@ -1,0 +1,203 @@
+/*
+ * C ABI of libinfllm_hip.so: the gfx950 (MI355X) kernels behind the InfLLM
+ * streaming memory-attention path.
+ *
+ * Conventions
+ *  - every pointer named d_* is a device address, h_* a (pinned) host address;
+ *  - bf16 buffers are passed as `const void*` / `void*`, fp32 as float*;
+ *  - all strides are in ELEMENTS, the innermost (head_dim) axis is contiguous;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *  - every call only enqueues work; buffers are borrowed until that work ends;
+ *  - return value 0 = ok, negative = rejected arguments or a launch error, with
+ *    the message available from infllm_last_error() (thread local);
+ *  - head_dim must be 128; dtype of q/k/v is bf16.
+ *
+ * Each entry point names the part of the reference it replaces (file:line in
+ * thunlp/InfLLM).
+ */
+#ifndef INFLLM_HIP_H
+#define INFLLM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define INFLLM_ABI_VERSION 1
+#define INFLLM_HEAD_DIM 128
+#define INFLLM_KEY_TILE 64
+
+/* Library identity; no counterpart in the reference (a pure-Python package). */
+int infllm_version(void);
+const char *infllm_last_error(void);
+
+/* ---------------------------------------------------------------------------
+ * Prologue: RoPE + staging of new tokens.
+ * Replaces RotaryEmbeddingESM.forward / apply_rotary_pos_emb_one_angle
+ * (inf_llm/attention/rope.py:89-112) and the torch.cat of the local window and
+ * the remainder (inf_llm/attention/context_manager.py:719-747).
+ *
+ * For the n new tokens at absolute stream positions pos0 .. pos0+n-1:
+ *   ring_k_raw / ring_v  <- k, v                 (row  pos % ring_cap)
+ *   ring_k_rot           <- RoPE(k, angle pos)
+ *   q_loc                <- RoPE(q, angle pos)
+ *   q_glb                <- RoPE(q, angle glb_pos)      (glb_pos = n_local - 1)
+ *   ring_score rows of the new tokens <- 0
+ * The relative rotation between q_loc[i] and ring_k_rot[j] is exactly
+ * (pos_i - pos_j) * inv_freq, which is what the reference's window-relative
+ * tables produce.  Angles are formed in fp64 (pos * distance_scale * inv_freq)
+ * so that positions of 10^6 and beyond keep full precision.
+ * q: [B,H,n,128], k/v: [B,Hkv,n,128]; rings: [B,Hkv,ring_cap,128];
+ * q_loc/q_glb: [B,H,n,128] contiguous; ring_score: fp32 [B,H,ring_cap].
+ */
+typedef struct {
+    const void *d_q, *d_k, *d_v;
+    int64_t q_sb, q_sh, q_sl;      /* strides of q */
+    int64_t k_sb, k_sh, k_sl;      /* strides of k */
+    int64_t v_sb, v_sh, v_sl;      /* strides of v */
+    int32_t B, H, Hkv, n;
+    int64_t pos0;
+    int64_t glb_pos;
+    const float *d_inv_freq;       /* [64] fp32, as the reference computes it */
+    double distance_scale;
+    void *d_ring_k_raw, *d_ring_k_rot, *d_ring_v;
+    float *d_ring_score;
+    int64_t ring_cap;
+    void *d_q_loc, *d_q_glb;
+} infllm_ingest_args;
+int infllm_ingest(const infllm_ingest_args *a, void *stream);
+
+/* Mean of q_glb over each execution block (context_manager.py:373-375):
+ * q_glb [B,H,n,128] contiguous -> d_qbar fp32 [B, n_blocks, H*128],
+ * block j covers rows [j*exc, min((j+1)*exc, n)). */
+int infllm_block_mean(const void *d_q_glb, int32_t B, int32_t H, int32_t n, int32_t exc,
+                      float *d_qbar, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * One stage of the multi-stage attention (bf16 MFMA flash kernel).
+ * Replaces MultiStageDotProductionAttention.append
+ * (inf_llm/attention/dot_production_attention/torch_impl.py:39-96,
+ *  triton_impl.py:488-556) for one stage; stages are joined by
+ * infllm_attn_merge.  Keys come either from a "linear" source (a tensor or a
+ * ring: key index j lives in row j % cap) with the reference's mask
+ *      dist = i - j + offset;  window: 0 <= dist < size;  complement: dist >= size
+ * or from a page table of 64-key tiles (memory units, init tokens, overflow
+ * remainder: context_manager.py:386-451), all keys of which are visible.
+ * Output: per split s, un-merged partial results
+ *      o_part [nsplit,B,H,Lq,128] fp32 (normalised by the split's own sum)
+ *      lse_part [nsplit,B,H,Lq]   fp32 (base-2 log-sum-exp of scaled logits)
+ */
+typedef struct {
+    const void *k;            /* device address of key row 0 of kv head 0 */
+    const void *v;
+    int64_t head_stride;      /* elements between kv heads */
+    int32_t n_valid;          /* 1..64 rows */
+    int32_t reserved;
+} infllm_page;
+
+enum { INFLLM_MASK_NONE = 0, INFLLM_MASK_WINDOW = 1, INFLLM_MASK_COMPLEMENT = 2 };
+
+typedef struct {
+    const void *d_q;               /* [B,H,Lq,128] */
+    int64_t q_sb, q_sh, q_sl;
+    int32_t B, H, Hkv, Lq;
+    /* linear source (d_pages == NULL) */
+    const void *d_k, *d_v;
+    int64_t k_sb, k_sh, k_sl, v_sb, v_sh, v_sl;
+    int64_t cap;                   /* rows of the ring; >= j_hi for a plain tensor */
+    int64_t j_lo, j_hi;            /* key index range held by the source */
+    int32_t mask;                  /* INFLLM_MASK_* */
+    int32_t reserved;
+    int64_t offset, window;
+    /* paged source (d_pages != NULL): [B, n_pages] */
+    const infllm_page *d_pages;
+    int32_t n_pages;
+    int32_t nsplit;
+    float softmax_scale;           /* 1/sqrt(128) */
+    float *d_o_part;
+    float *d_lse_part;
+} infllm_attn_args;
+int infllm_attn_stage(const infllm_attn_args *a, void *stream);
+
+/* Joint softmax across stages/splits (torch_impl.py:15-36):
+ * o = sum_p 2^(lse_p - LSE) o_p, LSE = log2 sum_p 2^lse_p.
+ * d_o_part [P,B,H,Lq,128], d_lse_part [P,B,H,Lq] -> d_out bf16 [B,H,Lq,128]
+ * (strides given), d_lse fp32 [B,H,Lq]. */
+int infllm_attn_merge(const float *d_o_part, const float *d_lse_part, int32_t P,
+                      int32_t B, int32_t H, int32_t Lq,
+                      void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
+                      float *d_lse, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Column sums of the final probabilities of one linear stage
+ * (torch_impl.py:27-28; triton_impl.py:232-335):
+ *   score[b,h,j] (+)= sum_i 2^(scale*log2e*q_i.k_j - lse[b,h,i]) * visible(i,j)
+ * for j in [j_lo, j_hi); score row index is j % score_cap.
+ */
+typedef struct {
+    const void *d_q;
+    int64_t q_sb, q_sh, q_sl;
+    int32_t B, H, Hkv, Lq;
+    const void *d_k;
+    int64_t k_sb, k_sh, k_sl;
+    int64_t cap;
+    int64_t j_lo, j_hi;
+    int32_t mask;
+    int32_t accumulate;            /* 1: add to d_score, 0: overwrite */
+    int64_t offset, window;
+    const float *d_lse;            /* [B,H,Lq] from infllm_attn_merge */
+    float softmax_scale;
+    int32_t reserved;
+    float *d_score;                /* fp32 [B,H,score_cap] */
+    int64_t score_sb, score_sh, score_cap;
+} infllm_score_args;
+int infllm_local_score(const infllm_score_args *a, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Retrieval: unit scores + top-k.
+ * Replaces VectorTensor.get_topk and calc_block_topk
+ * (context_manager.py:159-163, 366-383).
+ *   scores[n] = sum_c reps[n,c] * qbar[c]   (bf16 reps, fp32 qbar, fp32 out)
+ *   idx[0..k)  = indices of the k largest scores, ascending index order;
+ *                ties at the boundary go to the lower index.
+ * reps [N,C] bf16 row stride rep_stride; C = H*128.  k <= 1024.
+ */
+int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C,
+                      const float *d_qbar, int32_t k,
+                      float *d_scores, int32_t *d_idx, void *stream);
+
+/* Representative key of carved units.
+ * Replaces get_block_k + mean (context_manager.py:268-277, 664-670).
+ * For unit u (0 <= u < n_units) made of the tokens at ring rows
+ * (t0 + u*bs + r) % ring_cap, r < bs:
+ *   per query head h: the repr_topk highest ring_score[b,h,row] (ties -> lower r),
+ *   rep[b, u, h*128 + d] = mean of those rows of ring_k_raw[b, h / (H/Hkv)].
+ * d_rep_out: bf16 [B] rows at d_rep_out + b*rep_sb + u*rep_su; d_idx_out (optional,
+ * may be NULL): int32 [B,n_units,H,repr_topk] chosen r's in descending score order.
+ */
+int infllm_repr_keys(const float *d_ring_score, const void *d_ring_k_raw, int64_t ring_cap,
+                     int32_t B, int32_t H, int32_t Hkv, int64_t t0, int32_t bs,
+                     int32_t n_units, int32_t repr_topk,
+                     void *d_rep_out, int64_t rep_sb, int64_t rep_su,
+                     int32_t *d_idx_out, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Unit cache traffic.  Replaces MemoryUnit.__init__/load
+ * (context_manager.py:39-45, 76-91).
+ * infllm_gather_rows: ring rows (t0 + r) % ring_cap, r < n, of every kv head ->
+ *   out[b*out_sb + (r / unit_rows)*out_su + h*out_sh + (r % unit_rows)*128 ...] (device);
+ *   with unit_rows = n this is a plain [B,Hkv,n,128] copy.  Used to carve units and
+ *   init tokens out of the ring.
+ * infllm_copy_async: hipMemcpyAsync of nbytes, kind 1 = host->device,
+ *   2 = device->host, 3 = device->device, on `stream`.
+ */
+int infllm_gather_rows(const void *d_ring, int64_t ring_cap, int32_t B, int32_t Hkv,
+                       int64_t t0, int32_t n, int32_t unit_rows, void *d_out, int64_t out_sb,
+                       int64_t out_su, int64_t out_sh, void *stream);
+int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int32_t kind, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INFLLM_HIP_H */

@@ -1,0 +1,111 @@
+"""ctypes binding of libinfllm_hip.so (the C ABI declared in include/infllm_hip.h).
+
+The library is the only compute path of this package: if it is missing or does
+not export the expected symbols, loading raises - there is no fallback.
+"""
+import ctypes as C
+import os
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libinfllm_hip.so")
+ABI_VERSION = 1
+
+c_i32, c_i64, c_f32, c_f64, c_vp = C.c_int32, C.c_int64, C.c_float, C.c_double, C.c_void_p
+
+
+class IngestArgs(C.Structure):
+    _fields_ = [
+        ("d_q", c_vp), ("d_k", c_vp), ("d_v", c_vp),
+        ("q_sb", c_i64), ("q_sh", c_i64), ("q_sl", c_i64),
+        ("k_sb", c_i64), ("k_sh", c_i64), ("k_sl", c_i64),
+        ("v_sb", c_i64), ("v_sh", c_i64), ("v_sl", c_i64),
+        ("B", c_i32), ("H", c_i32), ("Hkv", c_i32), ("n", c_i32),
+        ("pos0", c_i64), ("glb_pos", c_i64),
+        ("d_inv_freq", c_vp), ("distance_scale", c_f64),
+        ("d_ring_k_raw", c_vp), ("d_ring_k_rot", c_vp), ("d_ring_v", c_vp),
+        ("d_ring_score", c_vp), ("ring_cap", c_i64),
+        ("d_q_loc", c_vp), ("d_q_glb", c_vp),
+    ]
+
+
+class Page(C.Structure):
+    _fields_ = [("k", c_vp), ("v", c_vp), ("head_stride", c_i64), ("n_valid", c_i32), ("reserved", c_i32)]
+
+
+class AttnArgs(C.Structure):
+    _fields_ = [
+        ("d_q", c_vp), ("q_sb", c_i64), ("q_sh", c_i64), ("q_sl", c_i64),
+        ("B", c_i32), ("H", c_i32), ("Hkv", c_i32), ("Lq", c_i32),
+        ("d_k", c_vp), ("d_v", c_vp),
+        ("k_sb", c_i64), ("k_sh", c_i64), ("k_sl", c_i64),
+        ("v_sb", c_i64), ("v_sh", c_i64), ("v_sl", c_i64),
+        ("cap", c_i64), ("j_lo", c_i64), ("j_hi", c_i64),
+        ("mask", c_i32), ("reserved", c_i32),
+        ("offset", c_i64), ("window", c_i64),
+        ("d_pages", c_vp), ("n_pages", c_i32), ("nsplit", c_i32),
+        ("softmax_scale", c_f32),
+        ("d_o_part", c_vp), ("d_lse_part", c_vp),
+    ]
+
+
+class ScoreArgs(C.Structure):
+    _fields_ = [
+        ("d_q", c_vp), ("q_sb", c_i64), ("q_sh", c_i64), ("q_sl", c_i64),
+        ("B", c_i32), ("H", c_i32), ("Hkv", c_i32), ("Lq", c_i32),
+        ("d_k", c_vp), ("k_sb", c_i64), ("k_sh", c_i64), ("k_sl", c_i64),
+        ("cap", c_i64), ("j_lo", c_i64), ("j_hi", c_i64),
+        ("mask", c_i32), ("accumulate", c_i32),
+        ("offset", c_i64), ("window", c_i64),
+        ("d_lse", c_vp), ("softmax_scale", c_f32), ("reserved", c_i32),
+        ("d_score", c_vp), ("score_sb", c_i64), ("score_sh", c_i64), ("score_cap", c_i64),
+    ]
+
+
+# name -> (restype, argtypes); every symbol include/infllm_hip.h declares
+SYMBOLS = {
+    "infllm_version": (c_i32, []),
+    "infllm_last_error": (C.c_char_p, []),
+    "infllm_ingest": (c_i32, [C.POINTER(IngestArgs), c_vp]),
+    "infllm_block_mean": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
+    "infllm_attn_stage": (c_i32, [C.POINTER(AttnArgs), c_vp]),
+    "infllm_attn_merge": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
+    "infllm_local_score": (c_i32, [C.POINTER(ScoreArgs), c_vp]),
+    "infllm_score_topk": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_vp, c_i32, c_vp, c_vp, c_vp]),
+    "infllm_repr_keys": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i64, c_i32, c_i32, c_i32,
+                                 c_vp, c_i64, c_i64, c_vp, c_vp]),
+    "infllm_gather_rows": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i64, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp]),
+    "infllm_copy_async": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_vp]),
+}
+
+_lib = None
+
+
+class InfLLMHipError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the shared library once; raise if it is absent or incomplete."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise InfLLMHipError(
+            f"{LIB_PATH} is missing: build it with `python -m infllm_amd.build` "
+            "(hipcc --offload-arch=gfx950); this package has no other compute path")
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SYMBOLS.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as e:
+            raise InfLLMHipError(f"{LIB_PATH} does not export {name}") from e
+        fn.restype, fn.argtypes = restype, argtypes
+    if lib.infllm_version() != ABI_VERSION:
+        raise InfLLMHipError(f"ABI version {lib.infllm_version()} != expected {ABI_VERSION}; rebuild the library")
+    _lib = lib
+    return lib
+
+
+def check(status, what):
+    if status != 0:
+        msg = load().infllm_last_error()
+        raise InfLLMHipError(f"{what} failed ({status}): {msg.decode() if msg else ''}")

@@ -1,0 +1,360 @@
+// Multi-stage attention for gfx950: one flash-style MFMA kernel per stage, and the
+// merge that realises the joint softmax across stages
+// (inf_llm/attention/dot_production_attention/torch_impl.py:15-96).
+//
+// Work split.  For one kv head the query heads that share it (GQA) are laid out as
+// "wave tasks" (query tile of 32 rows, head-in-group); a workgroup of 4 waves takes 4
+// consecutive tasks ordered tile-major/head-minor, so with 4 query heads per kv head
+// the 4 waves hold the same 32 queries of the 4 heads and walk the same keys.
+// K and V tiles of 64 keys are staged through LDS once per workgroup.
+//
+// MFMA formulation (v_mfma_f32_32x32x16_bf16), all operands read as 16-byte vectors:
+//   S^T[key, query] = K[key, :] . Q[query, :]       A = K rows (LDS), B = Q (registers)
+//   O^T[d, query]  += V^T[d, key] . P^T[key, query]  A = V^T rows (LDS), B = P (registers)
+// A lane owns ONE query column, so the running max / sum / rescale are per-lane scalars
+// and P never leaves registers.  MFMA row r of a 32-key sub-tile is bound to key
+// pi(r) = 16*(r>>4) + 8*((r>>2)&1) + 4*((r>>3)&1) + (r&3); with that binding the 16
+// accumulator registers of a lane are two runs of 8 consecutive keys, which is exactly
+// the k-slice the second MFMA wants from the lane.  V is transposed on its way into LDS.
+#include "common.h"
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * kWave;
+constexpr int kQTile = 32;                 // queries per wave
+constexpr int kKPad = kD + 8;              // LDS row of K  (bf16 elements)
+constexpr int kVPad = kTile + 8;           // LDS row of V^T (bf16 elements)
+
+struct StageRange {
+    int64_t lo, hi;   // key index range [lo, hi) visible to a span of queries
+};
+
+// keys visible to queries [i0, i1] under the stage mask, clipped to the source range
+__device__ __forceinline__ StageRange visible_range(const infllm_attn_args &a, int64_t i0, int64_t i1) {
+    StageRange r{a.j_lo, a.j_hi};
+    if (a.mask == INFLLM_MASK_WINDOW) {
+        r.lo = max(r.lo, i0 + a.offset - a.window + 1);
+        r.hi = min(r.hi, i1 + a.offset + 1);
+    } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
+        r.hi = min(r.hi, i1 + a.offset - a.window + 1);
+    }
+    return r;
+}
+
+__device__ __forceinline__ int floordiv64(int64_t x) { return (int)(x >> 6); }   // arithmetic shift = floor
+
+template <bool PAGED>
+__global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a) {
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[kTile][kKPad];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt[kD][kVPad];
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 31, grp = lane >> 5;
+    const int G = a.H / a.Hkv;
+    const int b = blockIdx.y / a.Hkv, g = blockIdx.y % a.Hkv;
+    const int split = blockIdx.z;
+    const int n_qtiles = (a.Lq + kQTile - 1) / kQTile;
+    const int n_tasks = n_qtiles * G;
+
+    // ---- this wave's task and the tiles it needs
+    const int task = blockIdx.x * kWaves + wave;
+    const bool live = task < n_tasks;
+    const int qt = live ? task / G : 0, hg = live ? task % G : 0;
+    const int h = g * G + hg;
+    const int i0 = qt * kQTile, i1 = min(i0 + kQTile, a.Lq) - 1;
+
+    int w_t0, w_t1;                      // this wave's tile range
+    if (PAGED) {
+        w_t0 = 0;
+        w_t1 = live ? a.n_pages : 0;
+    } else {
+        StageRange r = visible_range(a, i0, i1);
+        if (!live || r.hi <= r.lo) {
+            w_t0 = w_t1 = 0;
+        } else {
+            w_t0 = floordiv64(r.lo);
+            w_t1 = floordiv64(r.hi - 1) + 1;
+        }
+    }
+    // ---- workgroup range = union over its waves; the split takes a contiguous share of it
+    __shared__ int wg_lo[kWaves], wg_hi[kWaves];
+    if (lane == 0) {
+        wg_lo[wave] = w_t1 > w_t0 ? w_t0 : INT32_MAX;
+        wg_hi[wave] = w_t1 > w_t0 ? w_t1 : INT32_MIN;
+    }
+    __syncthreads();
+    int g_t0 = min(min(wg_lo[0], wg_lo[1]), min(wg_lo[2], wg_lo[3]));
+    int g_t1 = max(max(wg_hi[0], wg_hi[1]), max(wg_hi[2], wg_hi[3]));
+    if (g_t1 <= g_t0) g_t0 = g_t1 = 0;
+    {
+        int64_t n = g_t1 - g_t0;
+        int t_begin = g_t0 + (int)(n * split / a.nsplit);
+        int t_end = g_t0 + (int)(n * (split + 1) / a.nsplit);
+        g_t0 = t_begin;
+        g_t1 = t_end;
+    }
+
+    // ---- Q as the B operand: lane = (query col, k-group)
+    bf16x8 qreg[kD / 16];
+    {
+        const int qi = i0 + col;
+        const bool ok = live && qi < a.Lq;
+        const bf16_t *qrow = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qi * a.q_sl;
+#pragma unroll
+        for (int kk = 0; kk < kD / 16; ++kk) {
+            u32x4 raw = ok ? *(const u32x4 *)(qrow + kk * 16 + grp * 8) : u32x4{0, 0, 0, 0};
+            qreg[kk] = __builtin_bit_cast(bf16x8, raw);
+        }
+    }
+
+    // ---- cooperative tile loads: thread -> (rows, 16-byte chunk)
+    const int ld_chunk = tid & 15;            // 8 head_dim elements
+    const int ld_row = tid >> 4;              // 0..15
+    u32x4 kbuf[4], vbuf[4];                   // K rows ld_row + 16*i ; V rows 4*ld_row + i
+
+    auto load_tile = [&](int t) {
+        const bf16_t *kbase, *vbase;
+        int64_t k_sl, v_sl;
+        int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
+        if (PAGED) {
+            const infllm_page pg = a.d_pages[(int64_t)b * a.n_pages + t];
+            kbase = (const bf16_t *)pg.k + (int64_t)g * pg.head_stride;
+            vbase = (const bf16_t *)pg.v + (int64_t)g * pg.head_stride;
+            k_sl = v_sl = kD;
+            row_lo = 0;
+            row_hi = pg.n_valid;
+        } else {
+            const int64_t j0 = (int64_t)t * kTile;
+            const int64_t r0 = j0 % a.cap;    // cap is a multiple of the tile, so a tile never wraps
+            kbase = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh + r0 * a.k_sl;
+            vbase = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh + r0 * a.v_sl;
+            k_sl = a.k_sl;
+            v_sl = a.v_sl;
+            row_lo = (int)max((int64_t)0, a.j_lo - j0);
+            row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int r = ld_row + 16 * i;
+            kbuf[i] = (r >= row_lo && r < row_hi) ? *(const u32x4 *)(kbase + (int64_t)r * k_sl + ld_chunk * 8)
+                                                 : u32x4{0, 0, 0, 0};
+            int rv = 4 * ld_row + i;
+            vbuf[i] = (rv >= row_lo && rv < row_hi) ? *(const u32x4 *)(vbase + (int64_t)rv * v_sl + ld_chunk * 8)
+                                                   : u32x4{0, 0, 0, 0};
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(u32x4 *)&Ks[ld_row + 16 * i][ld_chunk * 8] = kbuf[i];
+        // 4 keys x 8 dims -> 8 dims x 4 keys
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            u32x2 even, odd;                  // dims 2w and 2w+1 of keys 0..3
+            even[0] = (vbuf[0][w] & 0xffffu) | (vbuf[1][w] << 16);
+            even[1] = (vbuf[2][w] & 0xffffu) | (vbuf[3][w] << 16);
+            odd[0] = (vbuf[0][w] >> 16) | (vbuf[1][w] & 0xffff0000u);
+            odd[1] = (vbuf[2][w] >> 16) | (vbuf[3][w] & 0xffff0000u);
+            *(u32x2 *)&Vt[ld_chunk * 8 + 2 * w][4 * ld_row] = even;
+            *(u32x2 *)&Vt[ld_chunk * 8 + 2 * w + 1][4 * ld_row] = odd;
+        }
+    };
+
+    // ---- running softmax state of this lane's query
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x16 oacc[kD / 32];
+#pragma unroll
+    for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
+
+    const float scale = a.softmax_scale * 1.4426950408889634f;
+    // MFMA row -> key of a 32-key sub-tile
+    const int pi_row = 16 * (col >> 4) + 8 * ((col >> 2) & 1) + 4 * ((col >> 3) & 1) + (col & 3);
+    const int64_t qpos = (int64_t)i0 + col + a.offset;          // query index shifted into key index space
+
+    if (g_t1 > g_t0) load_tile(g_t0);
+    for (int t = g_t0; t < g_t1; ++t) {
+        __syncthreads();                       // previous tile fully consumed
+        store_tile();
+        __syncthreads();
+        if (t + 1 < g_t1) load_tile(t + 1);     // in flight while this tile is computed
+        if (t < w_t0 || t >= w_t1) continue;    // wave-uniform; barriers stay outside
+
+        f32x16 s[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[ks][r] = 0.f;
+            const bf16_t *krow = &Ks[ks * 32 + pi_row][grp * 8];
+#pragma unroll
+            for (int kk = 0; kk < kD / 16; ++kk) {
+                bf16x8 ka = *(const bf16x8 *)(krow + kk * 16);
+                s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[kk], s[ks], 0, 0, 0);
+            }
+        }
+        // ---- mask (only tiles that touch a boundary) and scale
+        bool need_mask;
+        int row_lo = 0, row_hi = kTile;
+        const int64_t j0 = (int64_t)t * kTile;
+        if (PAGED) {
+            row_hi = a.d_pages[(int64_t)b * a.n_pages + t].n_valid;
+            need_mask = row_hi < kTile;
+        } else {
+            row_lo = (int)max((int64_t)0, a.j_lo - j0);
+            row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
+            need_mask = row_lo > 0 || row_hi < kTile;
+            if (a.mask == INFLLM_MASK_WINDOW) {
+                // fully visible iff the oldest query still sees the newest key... check both ends
+                need_mask |= (j0 + kTile - 1 > (int64_t)i0 + a.offset) ||
+                             (j0 < (int64_t)i1 + a.offset - a.window + 1);
+            } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
+                need_mask |= (j0 + kTile - 1 > (int64_t)i0 + a.offset - a.window);
+            }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float x = s[ks][r] * scale;
+                if (need_mask) {
+                    const int ko = ks * 32 + 16 * (r >> 3) + 8 * grp + (r & 7);
+                    bool vis = ko >= row_lo && ko < row_hi;
+                    if (!PAGED) {
+                        const int64_t dist = qpos - (j0 + ko);
+                        if (a.mask == INFLLM_MASK_WINDOW) vis = vis && dist >= 0 && dist < a.window;
+                        if (a.mask == INFLLM_MASK_COMPLEMENT) vis = vis && dist >= a.window;
+                    }
+                    x = vis ? x : -INFINITY;
+                }
+                s[ks][r] = x;
+                tmax = fmaxf(tmax, x);
+            }
+        tmax = fmaxf(tmax, wave_xor32(tmax));
+        const float m_new = fmaxf(m_run, tmax);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        float psum = 0.f;
+        uint32_t pw[2][8];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                float p0 = __builtin_amdgcn_exp2f(s[ks][r] - m_use);
+                float p1 = __builtin_amdgcn_exp2f(s[ks][r + 1] - m_use);
+                psum += p0 + p1;
+                pw[ks][r >> 1] = pack_bf16x2(p0, p1);
+            }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
+
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int mm = 0; mm < 2; ++mm) {
+                u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
+                bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+#pragma unroll
+                for (int dt = 0; dt < kD / 32; ++dt) {
+                    bf16x8 va = *(const bf16x8 *)&Vt[dt * 32 + col][ks * 32 + 16 * mm + 8 * grp];
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, oacc[dt], 0, 0, 0);
+                }
+            }
+    }
+
+    // ---- epilogue: normalised partial + base-2 log-sum-exp
+    if (!live) return;
+    const float l_tot = l_run + wave_xor32(l_run);
+    const int qi = i0 + col;
+    if (qi >= a.Lq) return;
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int64_t row = (((int64_t)split * a.B + b) * a.H + h) * a.Lq + qi;
+    float *orow = a.d_o_part + row * kD;
+#pragma unroll
+    for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 o4{oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv, oacc[dt][4 * q4 + 2] * inv,
+                     oacc[dt][4 * q4 + 3] * inv};
+            *(f32x4 *)(orow + dt * 32 + 8 * q4 + 4 * grp) = o4;
+        }
+    if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run + log2f(l_tot) : -INFINITY;
+}
+
+// one thread per (row, 4 dims): P partials -> bf16 output row + final lse
+__global__ __launch_bounds__(256) void attn_merge_kernel(const float *o_part, const float *lse_part, int P, int B, int H,
+                                                         int Lq, bf16_t *out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
+                                                         float *lse_out) {
+    const int64_t rows = (int64_t)B * H * Lq;
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t row = e >> 5;
+    const int c = (int)(e & 31);
+    if (row >= rows) return;
+    float m = -INFINITY;
+    for (int p = 0; p < P; ++p) m = fmaxf(m, lse_part[p * rows + row]);
+    f32x4 acc{0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    if (m > -INFINITY) {
+        for (int p = 0; p < P; ++p) {
+            float w = __builtin_amdgcn_exp2f(lse_part[p * rows + row] - m);
+            if (w > 0.f) {
+                f32x4 o = *(const f32x4 *)(o_part + (p * rows + row) * kD + c * 4);
+                acc += o * w;
+                den += w;
+            }
+        }
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    const int i = (int)(row % Lq), h = (int)((row / Lq) % H), b = (int)(row / ((int64_t)Lq * H));
+    u32x2 packed{pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv)};
+    *(u32x2 *)(out + (int64_t)b * o_sb + (int64_t)h * o_sh + (int64_t)i * o_sl + c * 4) = packed;
+    if (c == 0 && lse_out) lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
+}
+
+}  // namespace
+
+extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
+    INFLLM_REQUIRE(a != nullptr, "attn_stage: null argument block");
+    INFLLM_REQUIRE(a->d_q && a->d_o_part && a->d_lse_part, "attn_stage: null q / output pointer");
+    INFLLM_REQUIRE(a->B > 0 && a->H > 0 && a->Hkv > 0 && a->H % a->Hkv == 0 && a->Lq > 0,
+                   "attn_stage: bad geometry B=%d H=%d Hkv=%d Lq=%d", a->B, a->H, a->Hkv, a->Lq);
+    INFLLM_REQUIRE(a->nsplit >= 1 && a->nsplit <= 64, "attn_stage: nsplit %d out of range", a->nsplit);
+    INFLLM_REQUIRE((a->q_sl % 8 | a->q_sh % 8 | a->q_sb % 8) == 0, "attn_stage: q strides must be multiples of 8");
+    const int G = a->H / a->Hkv;
+    const int n_tasks = ((a->Lq + kQTile - 1) / kQTile) * G;
+    dim3 grid((n_tasks + kWaves - 1) / kWaves, a->B * a->Hkv, a->nsplit);
+    if (a->d_pages) {
+        INFLLM_REQUIRE(a->n_pages >= 0, "attn_stage: negative page count");
+        hipLaunchKernelGGL(attn_stage_kernel<true>, grid, dim3(kThreads), 0, (hipStream_t)stream, *a);
+    } else {
+        INFLLM_REQUIRE(a->j_hi <= a->j_lo || (a->d_k && a->d_v), "attn_stage: null k / v pointer");
+        INFLLM_REQUIRE(a->cap > 0 && a->cap % kTile == 0, "attn_stage: cap %lld is not a positive multiple of %d",
+                       (long long)a->cap, kTile);
+        INFLLM_REQUIRE(a->j_lo >= 0 && a->j_hi - a->j_lo <= a->cap, "attn_stage: key range [%lld,%lld) exceeds cap %lld",
+                       (long long)a->j_lo, (long long)a->j_hi, (long long)a->cap);
+        INFLLM_REQUIRE(a->mask >= 0 && a->mask <= 2, "attn_stage: unknown mask %d", a->mask);
+        INFLLM_REQUIRE((a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8 | a->v_sl % 8 | a->v_sh % 8 | a->v_sb % 8) == 0,
+                       "attn_stage: k/v strides must be multiples of 8");
+        hipLaunchKernelGGL(attn_stage_kernel<false>, grid, dim3(kThreads), 0, (hipStream_t)stream, *a);
+    }
+    INFLLM_CHECK_LAUNCH("attn_stage");
+    return 0;
+}
+
+extern "C" int infllm_attn_merge(const float *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
+                                 int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
+                                 void *stream) {
+    INFLLM_REQUIRE(d_o_part && d_lse_part && d_out, "attn_merge: null pointer");
+    INFLLM_REQUIRE(P >= 1 && B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes P=%d B=%d H=%d Lq=%d", P, B, H, Lq);
+    INFLLM_REQUIRE((o_sl % 4 | o_sh % 4 | o_sb % 4) == 0, "attn_merge: output strides must be multiples of 4");
+    const int64_t threads = (int64_t)B * H * Lq * 32;
+    hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
+    INFLLM_CHECK_LAUNCH("attn_merge");
+    return 0;
+}

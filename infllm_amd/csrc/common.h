@@ -1,0 +1,52 @@
+// Shared helpers for the gfx950 kernels of libinfllm_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/infllm_hip.h"
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kD = INFLLM_HEAD_DIM;       // head_dim
+constexpr int kTile = INFLLM_KEY_TILE;    // keys per tile
+constexpr int kWave = 64;
+
+// thread-local error text, returned by infllm_last_error()
+char *infllm_err_buf();
+int infllm_fail(int code, const char *fmt, ...);
+
+#define INFLLM_REQUIRE(cond, ...)                      \
+    do {                                               \
+        if (!(cond)) return infllm_fail(-1, __VA_ARGS__); \
+    } while (0)
+
+#define INFLLM_CHECK_LAUNCH(name)                                                     \
+    do {                                                                              \
+        hipError_t e_ = hipGetLastError();                                            \
+        if (e_ != hipSuccess) return infllm_fail(-2, "%s: %s", name, hipGetErrorString(e_)); \
+    } while (0)
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) {
+    return __uint_as_float(bits16 << 16);
+}
+// round-to-nearest-even fp32 -> bf16 bits (inputs are finite here; NaN kept quiet)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+__device__ __forceinline__ float wave_xor32(float x) {
+    return __shfl_xor(x, 32, 64);
+}

@@ -1,0 +1,210 @@
+// Retrieval side of the streaming path: unit scores, top-k selection and the
+// representative key of a carved unit
+// (inf_llm/attention/context_manager.py:159-163, 268-277, 366-383, 664-670).
+// All three are memory-bound; reductions are wavefront-wide with a fixed order, so the
+// outputs are deterministic.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+// ---------------------------------------------------------------- unit scores (GEMV)
+// one wave per representative row; the mean query sits in LDS as fp32
+__global__ __launch_bounds__(256) void unit_scores_kernel(const bf16_t *reps, int64_t rep_stride, int N, int C,
+                                                          const float *qbar, float *scores) {
+    extern __shared__ float qs[];
+    for (int e = threadIdx.x; e < C; e += 256) qs[e] = qbar[e];
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int wave_global = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int n_waves = gridDim.x * 4;
+    const int chunks = C / 8;
+    for (int n = wave_global; n < N; n += n_waves) {
+        const bf16_t *row = reps + (int64_t)n * rep_stride;
+        float acc = 0.f;
+        for (int c = lane; c < chunks; c += 64) {
+            u32x4 w = *(const u32x4 *)(row + c * 8);
+            const float *qv = qs + c * 8;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc += bf16_bits_to_f32(w[i] & 0xffffu) * qv[2 * i];
+                acc += bf16_bits_to_f32(w[i] >> 16) * qv[2 * i + 1];
+            }
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) scores[n] = acc;
+    }
+}
+
+// ---------------------------------------------------------------- top-k (radix select)
+constexpr int kSelThreads = 1024;
+
+__device__ __forceinline__ uint32_t order_key(float f) {
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);       // larger float <=> larger key
+}
+
+// exclusive scan of one int per thread over the workgroup; returns the total in *total
+__device__ int block_exclusive_scan(int v, int *wave_tot, int *total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        int n = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += n;
+    }
+    __syncthreads();                      // wave_tot free to overwrite
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    int base = 0, tot = 0;
+    for (int w = 0; w < kSelThreads / 64; ++w) {
+        int t = wave_tot[w];
+        if (w < wave) base += t;
+        tot += t;
+    }
+    *total = tot;
+    return base + incl - v;
+}
+
+__global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, int N, int k, int32_t *idx_out) {
+    __shared__ int hist[256];
+    __shared__ int wave_tot[kSelThreads / 64];
+    __shared__ uint32_t sh_prefix;
+    __shared__ int sh_need;
+    const int tid = threadIdx.x;
+
+    // ---- find the k-th largest key, 8 bits per pass from the top
+    uint32_t prefix = 0, pmask = 0;
+    int need = k;                          // how many of the keys matching `prefix` are still wanted
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        for (int n = tid; n < N; n += kSelThreads) {
+            uint32_t key = order_key(scores[n]);
+            if ((key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            int remaining = need, d = 255;
+            for (; d > 0; --d) {
+                if (hist[d] >= remaining) break;
+                remaining -= hist[d];
+            }
+            sh_prefix = prefix | ((uint32_t)d << shift);
+            sh_need = remaining;
+        }
+        __syncthreads();
+        prefix = sh_prefix;
+        need = sh_need;
+        pmask |= 255u << shift;
+        __syncthreads();
+    }
+    // prefix = key of the k-th largest; take all keys above it and the first `need` equal to it
+    int out_base = 0, eq_base = 0;
+    for (int n0 = 0; n0 < N; n0 += kSelThreads) {
+        const int n = n0 + tid;
+        uint32_t key = n < N ? order_key(scores[n]) : 0u;
+        const int is_eq = (n < N && key == prefix) ? 1 : 0;
+        int tot_eq, tot_sel;
+        const int eq_rank = eq_base + block_exclusive_scan(is_eq, wave_tot, &tot_eq);
+        const int sel = (n < N && (key > prefix || (is_eq && eq_rank < need))) ? 1 : 0;
+        const int pos = out_base + block_exclusive_scan(sel, wave_tot, &tot_sel);
+        if (sel && pos < k) idx_out[pos] = n;
+        eq_base += tot_eq;
+        out_base += tot_sel;
+    }
+}
+
+// ---------------------------------------------------------------- representative keys
+constexpr int kMaxUnit = 2048;             // largest supported unit (block_size)
+
+// one wave per (query head, unit, batch row)
+__global__ __launch_bounds__(64) void repr_keys_kernel(const float *ring_score, const bf16_t *ring_k, int64_t ring_cap,
+                                                       int H, int Hkv, int64_t t0, int bs, int repr_topk, bf16_t *rep_out,
+                                                       int64_t rep_sb, int64_t rep_su, int32_t *idx_out) {
+    __shared__ float sc[kMaxUnit];
+    const int h = blockIdx.x, u = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
+    const int n_units = gridDim.y;
+    const int g = h / (H / Hkv);
+    const int64_t first = t0 + (int64_t)u * bs;
+    const float *srow = ring_score + ((int64_t)b * H + h) * ring_cap;
+    for (int r = lane; r < bs; r += 64) sc[r] = srow[(first + r) % ring_cap];
+    __syncthreads();
+    const bf16_t *kbase = ring_k + ((int64_t)b * Hkv + g) * ring_cap * kD;
+    float a0 = 0.f, a1 = 0.f;
+    for (int it = 0; it < repr_topk; ++it) {
+        float best = -INFINITY;
+        int best_r = INT32_MAX;
+        for (int r = lane; r < bs; r += 64) {
+            float x = sc[r];
+            if (x > best || (x == best && r < best_r)) {     // NaN never wins
+                best = x;
+                best_r = r;
+            }
+        }
+        if (best_r == INT32_MAX && lane < bs) best_r = lane;   // all -inf / NaN: still pick a valid row
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            float ob = __shfl_xor(best, o, 64);
+            int orr = __shfl_xor(best_r, o, 64);
+            if (ob > best || (ob == best && orr < best_r) || best_r == INT32_MAX) {
+                best = ob;
+                best_r = orr;
+            }
+        }
+        if (lane == 0) {
+            sc[best_r] = -INFINITY;
+            if (idx_out) idx_out[(((int64_t)b * n_units + u) * H + h) * repr_topk + it] = best_r;
+        }
+        uint32_t w = *(const uint32_t *)(kbase + ((first + best_r) % ring_cap) * kD + lane * 2);
+        a0 += bf16_bits_to_f32(w & 0xffffu);
+        a1 += bf16_bits_to_f32(w >> 16);
+        __syncthreads();
+    }
+    const float inv = 1.f / (float)repr_topk;
+    *(uint32_t *)(rep_out + (int64_t)b * rep_sb + (int64_t)u * rep_su + (int64_t)h * kD + lane * 2) =
+        pack_bf16x2(a0 * inv, a1 * inv);
+}
+
+}  // namespace
+
+extern "C" int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbar,
+                                 int32_t k, float *d_scores, int32_t *d_idx, void *stream) {
+    INFLLM_REQUIRE(d_reps && d_qbar && d_scores, "score_topk: null pointer");
+    INFLLM_REQUIRE(N > 0 && C > 0 && C % 8 == 0 && C <= 16384, "score_topk: bad sizes N=%d C=%d", N, C);
+    INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "score_topk: row stride %lld", (long long)rep_stride);
+    INFLLM_REQUIRE(k >= 0 && k <= N && k <= 1024, "score_topk: k=%d with N=%d", k, N);
+    INFLLM_REQUIRE(k == 0 || d_idx, "score_topk: null index output");
+    const int wgs = N < 4 * 2048 ? (N + 3) / 4 : 2048;
+    hipLaunchKernelGGL(unit_scores_kernel, dim3(wgs), dim3(256), (size_t)C * sizeof(float), (hipStream_t)stream,
+                       (const bf16_t *)d_reps, rep_stride, N, C, d_qbar, d_scores);
+    INFLLM_CHECK_LAUNCH("unit_scores");
+    if (k > 0) {
+        hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, (hipStream_t)stream, d_scores, N, k, d_idx);
+        INFLLM_CHECK_LAUNCH("topk");
+    }
+    return 0;
+}
+
+extern "C" int infllm_repr_keys(const float *d_ring_score, const void *d_ring_k_raw, int64_t ring_cap, int32_t B, int32_t H,
+                                int32_t Hkv, int64_t t0, int32_t bs, int32_t n_units, int32_t repr_topk, void *d_rep_out,
+                                int64_t rep_sb, int64_t rep_su, int32_t *d_idx_out, void *stream) {
+    INFLLM_REQUIRE(d_ring_score && d_ring_k_raw && d_rep_out, "repr_keys: null pointer");
+    INFLLM_REQUIRE(B > 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "repr_keys: bad geometry B=%d H=%d Hkv=%d", B, H, Hkv);
+    INFLLM_REQUIRE(bs > 0 && bs <= kMaxUnit, "repr_keys: unit size %d not in 1..%d", bs, kMaxUnit);
+    INFLLM_REQUIRE(repr_topk > 0 && repr_topk <= bs, "repr_keys: repr_topk %d not in 1..%d", repr_topk, bs);
+    INFLLM_REQUIRE(n_units >= 0 && t0 >= 0 && (int64_t)n_units * bs <= ring_cap, "repr_keys: %d units do not fit the ring",
+                   n_units);
+    INFLLM_REQUIRE(rep_sb % 2 == 0 && rep_su % 2 == 0, "repr_keys: output strides must be even");
+    if (n_units == 0) return 0;
+    hipLaunchKernelGGL(repr_keys_kernel, dim3(H, n_units, B), dim3(64), 0, (hipStream_t)stream, d_ring_score,
+                       (const bf16_t *)d_ring_k_raw, ring_cap, H, Hkv, t0, bs, repr_topk, (bf16_t *)d_rep_out, rep_sb,
+                       rep_su, d_idx_out);
+    INFLLM_CHECK_LAUNCH("repr_keys");
+    return 0;
+}

@@ -1,0 +1,160 @@
+"""Torch-tensor wrappers over the C ABI (include/infllm_hip.h).
+
+torch is used for device memory and streams only; every computation below is a
+call into libinfllm_hip.so on the current stream.
+"""
+import math
+
+import torch
+
+from . import _lib
+from ._lib import AttnArgs, IngestArgs, Page, ScoreArgs, check
+
+HEAD_DIM = 128
+KEY_TILE = 64
+MASK_NONE, MASK_WINDOW, MASK_COMPLEMENT = 0, 1, 2
+NO_WRAP = 1 << 40          # "cap" of a plain tensor source (a multiple of the key tile)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _bf16_4d(t, name):
+    _need(t.is_cuda, f"{name} must be a GPU tensor")
+    _need(t.dtype == torch.bfloat16, f"{name} must be bfloat16 (the HIP path computes in bf16), got {t.dtype}")
+    _need(t.dim() == 4 and t.shape[-1] == HEAD_DIM, f"{name} must be [B, heads, len, {HEAD_DIM}], got {tuple(t.shape)}")
+    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]):
+        t = t.contiguous()
+    return t
+
+
+def ingest(q, k, v, pos0, glb_pos, inv_freq, distance_scale, ring_k_raw, ring_k_rot, ring_v, ring_score, q_loc, q_glb):
+    """RoPE + staging of the new tokens; see infllm_ingest."""
+    q, k, v = _bf16_4d(q, "q"), _bf16_4d(k, "k"), _bf16_4d(v, "v")
+    B, H, n, _ = q.shape
+    Hkv = k.shape[1]
+    _need(k.shape == v.shape == (B, Hkv, n, HEAD_DIM), "k/v shape mismatch")
+    cap = ring_k_raw.shape[2]
+    for r in (ring_k_raw, ring_k_rot, ring_v):
+        _need(r.is_contiguous() and r.shape == (B, Hkv, cap, HEAD_DIM) and r.dtype == torch.bfloat16, "bad ring")
+    _need(ring_score.is_contiguous() and ring_score.shape == (B, H, cap) and ring_score.dtype == torch.float32, "bad score ring")
+    for o in (q_loc, q_glb):
+        _need(o.is_contiguous() and o.dtype == torch.bfloat16 and o.numel() >= B * H * n * HEAD_DIM, "bad q workspace")
+    _need(inv_freq.dtype == torch.float32 and inv_freq.numel() == HEAD_DIM // 2 and inv_freq.is_cuda, "bad inv_freq")
+    a = IngestArgs(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                   q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                   v.stride(0), v.stride(1), v.stride(2), B, H, Hkv, n, pos0, glb_pos,
+                   inv_freq.data_ptr(), float(distance_scale),
+                   ring_k_raw.data_ptr(), ring_k_rot.data_ptr(), ring_v.data_ptr(), ring_score.data_ptr(), cap,
+                   q_loc.data_ptr(), q_glb.data_ptr())
+    check(_lib.load().infllm_ingest(a, _stream()), "infllm_ingest")
+
+
+def block_mean(q_glb, B, H, n, exc, qbar):
+    check(_lib.load().infllm_block_mean(q_glb.data_ptr(), B, H, n, exc, qbar.data_ptr(), _stream()), "infllm_block_mean")
+
+
+def attn_stage_linear(q, k, v, o_part, lse_part, *, cap=None, j_lo=0, j_hi=None, mask=MASK_NONE, offset=0, window=0,
+                      nsplit=1, softmax_scale=None):
+    """One stage over a linear key source.  q [B,H,Lq,D]; k/v [B,Hkv,rows,D] (rows = ring rows)."""
+    B, H, Lq, D = q.shape
+    Hkv = k.shape[1]
+    if cap is None:
+        cap = NO_WRAP
+    if j_hi is None:
+        j_hi = k.shape[2]
+    a = AttnArgs()
+    a.d_q, a.q_sb, a.q_sh, a.q_sl = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    a.B, a.H, a.Hkv, a.Lq = B, H, Hkv, Lq
+    a.d_k, a.d_v = k.data_ptr(), v.data_ptr()
+    a.k_sb, a.k_sh, a.k_sl = k.stride(0), k.stride(1), k.stride(2)
+    a.v_sb, a.v_sh, a.v_sl = v.stride(0), v.stride(1), v.stride(2)
+    a.cap, a.j_lo, a.j_hi = cap, j_lo, j_hi
+    a.mask, a.offset, a.window = mask, offset, window
+    a.d_pages, a.n_pages, a.nsplit = None, 0, nsplit
+    a.softmax_scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    a.d_o_part, a.d_lse_part = o_part.data_ptr(), lse_part.data_ptr()
+    check(_lib.load().infllm_attn_stage(a, _stream()), "infllm_attn_stage")
+
+
+def attn_stage_paged(q, pages_dev, n_pages, Hkv, o_part, lse_part, *, nsplit=1, softmax_scale=None):
+    """One stage over a device page table [B, n_pages] of infllm_page entries."""
+    B, H, Lq, D = q.shape
+    a = AttnArgs()
+    a.d_q, a.q_sb, a.q_sh, a.q_sl = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    a.B, a.H, a.Hkv, a.Lq = B, H, Hkv, Lq
+    a.d_pages, a.n_pages, a.nsplit = pages_dev.data_ptr(), n_pages, nsplit
+    a.cap = KEY_TILE
+    a.softmax_scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    a.d_o_part, a.d_lse_part = o_part.data_ptr(), lse_part.data_ptr()
+    check(_lib.load().infllm_attn_stage(a, _stream()), "infllm_attn_stage")
+
+
+def attn_merge(o_part, lse_part, P, out, lse):
+    """Join P partials: out bf16 [B,H,Lq,D] (any strides with contiguous rows), lse fp32 [B,H,Lq]."""
+    B, H, Lq, D = out.shape
+    _need(out.stride(-1) == 1 and out.dtype == torch.bfloat16, "bad merge output")
+    check(_lib.load().infllm_attn_merge(o_part.data_ptr(), lse_part.data_ptr(), P, B, H, Lq,
+                                        out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+                                        lse.data_ptr() if lse is not None else None, _stream()), "infllm_attn_merge")
+
+
+def local_score(q, k, lse, score, *, cap=None, j_lo=0, j_hi=None, mask=MASK_NONE, offset=0, window=0,
+                accumulate=True, score_cap=None, softmax_scale=None):
+    """score[b,h,j % score_cap] (+)= column sums of the stage's final probabilities."""
+    B, H, Lq, D = q.shape
+    a = ScoreArgs()
+    a.d_q, a.q_sb, a.q_sh, a.q_sl = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
+    a.B, a.H, a.Hkv, a.Lq = B, H, k.shape[1], Lq
+    a.d_k, a.k_sb, a.k_sh, a.k_sl = k.data_ptr(), k.stride(0), k.stride(1), k.stride(2)
+    a.cap = cap if cap is not None else NO_WRAP
+    a.j_lo, a.j_hi = j_lo, (j_hi if j_hi is not None else k.shape[2])
+    a.mask, a.accumulate, a.offset, a.window = mask, int(accumulate), offset, window
+    a.d_lse = lse.data_ptr()
+    a.softmax_scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
+    a.d_score, a.score_sb, a.score_sh = score.data_ptr(), score.stride(0), score.stride(1)
+    a.score_cap = score_cap if score_cap is not None else NO_WRAP
+    check(_lib.load().infllm_local_score(a, _stream()), "infllm_local_score")
+
+
+def score_topk(reps, n, qbar, k, scores, idx):
+    """scores[:n] = reps[:n] @ qbar; idx[:k] = ascending indices of the k largest."""
+    check(_lib.load().infllm_score_topk(reps.data_ptr(), reps.stride(0), n, reps.shape[1], qbar.data_ptr(), k,
+                                        scores.data_ptr(), idx.data_ptr() if idx is not None else None, _stream()),
+          "infllm_score_topk")
+
+
+def repr_keys(ring_score, ring_k_raw, t0, bs, n_units, repr_topk, rep_out, rep_sb, rep_su, idx_out=None):
+    B, H, cap = ring_score.shape
+    Hkv = ring_k_raw.shape[1]
+    check(_lib.load().infllm_repr_keys(ring_score.data_ptr(), ring_k_raw.data_ptr(), cap, B, H, Hkv, t0, bs, n_units,
+                                       repr_topk, rep_out.data_ptr(), rep_sb, rep_su,
+                                       idx_out.data_ptr() if idx_out is not None else None, _stream()), "infllm_repr_keys")
+
+
+def gather_rows(ring, t0, n, out_ptr, out_sb, out_sh, unit_rows=None, out_su=0):
+    """Ring rows (t0+r) % cap, r < n, of every kv head -> out_ptr + b*out_sb + (r//unit_rows)*out_su + h*out_sh + (r%unit_rows)*D."""
+    B, Hkv, cap, _ = ring.shape
+    check(_lib.load().infllm_gather_rows(ring.data_ptr(), cap, B, Hkv, t0, n, unit_rows if unit_rows else max(n, 1),
+                                         out_ptr, out_sb, out_su, out_sh, _stream()), "infllm_gather_rows")
+
+
+def copy_async(dst, src, nbytes, kind, stream=None):
+    """kind: 1 host->device, 2 device->host, 3 device->device (raw addresses or tensors)."""
+    d = dst.data_ptr() if torch.is_tensor(dst) else dst
+    s = src.data_ptr() if torch.is_tensor(src) else src
+    check(_lib.load().infllm_copy_async(d, s, nbytes, kind, stream if stream is not None else _stream()), "infllm_copy_async")
+
+
+def make_pages(entries):
+    """entries: list of (k_addr, v_addr, head_stride, n_valid) -> ctypes array of infllm_page."""
+    arr = (Page * max(len(entries), 1))()
+    for i, (k, v, hs, n) in enumerate(entries):
+        arr[i].k, arr[i].v, arr[i].head_stride, arr[i].n_valid = k, v, hs, n
+    return arr

@@ -1,0 +1,321 @@
+"""GPU parity of every kernel entry point (called through the C ABI) against the CPU oracle.
+
+Acceptance (floating point): attention outputs within max-abs 2e-2 / mean-abs 2e-3 of
+the fp32 oracle evaluated on the same bf16-rounded inputs; index outputs exact except
+where two candidates' oracle scores are within 1e-3 relative of each other.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.multistage import MultiStageOracle
+from oracle.rope import RopeOracle
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+D = 128
+
+
+def _ops():
+    from infllm_amd import ops
+    return ops
+
+
+def _rand(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).bfloat16()
+
+
+def _check_out(got, want, what=""):
+    err = (got.float().cpu() - want.float()).abs()
+    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (what, float(err.max()), float(err.mean()))
+
+
+# ------------------------------------------------------------------ prologue
+@pytest.mark.parametrize("pos0,n", [(0, 40), (4090, 17), (1_000_003, 33), (2 ** 31 + 5, 8)])
+def test_ingest_matches_rope_oracle(pos0, n):
+    ops = _ops()
+    B, H, Hkv, cap, n_local = 2, 4, 2, 128, 4096
+    q, k, v = _rand((B, H, n, D), 1), _rand((B, Hkv, n, D), 2), _rand((B, Hkv, n, D), 3)
+    rope = RopeOracle(D, base=1e6)
+    dev = "cuda"
+    rk_raw = torch.zeros((B, Hkv, cap, D), dtype=torch.bfloat16, device=dev)
+    rk_rot, rv = torch.zeros_like(rk_raw), torch.zeros_like(rk_raw)
+    rscore = torch.ones((B, H, cap), dtype=torch.float32, device=dev)
+    q_loc = torch.zeros((B, H, n, D), dtype=torch.bfloat16, device=dev)
+    q_glb = torch.zeros_like(q_loc)
+    # strided inputs ([B, n, heads, D] memory order) exercise the stride arguments
+    qd = q.permute(0, 2, 1, 3).contiguous().to(dev).permute(0, 2, 1, 3)
+    ops.ingest(qd, k.to(dev), v.to(dev), pos0, n_local - 1, rope.inv_freq.to(dev), 1.0, rk_raw, rk_rot, rv, rscore, q_loc, q_glb)
+    torch.cuda.synchronize()
+    rows = [(pos0 + i) % cap for i in range(n)]
+    assert torch.equal(rk_raw[:, :, rows].cpu(), k) and torch.equal(rv[:, :, rows].cpu(), v)
+    assert float(rscore[:, :, rows].abs().max()) == 0.0
+    untouched = [r for r in range(cap) if r not in rows]
+    assert float(rscore[:, :, untouched].min()) == 1.0 and float(rk_raw[:, :, untouched].abs().max()) == 0.0
+    # fp64 rotation with the reference's fp32 inverse frequencies
+    inv = rope.inv_freq.double()
+    ang = torch.arange(pos0, pos0 + n, dtype=torch.float64)[:, None] * inv[None, :]
+
+    def rot(x, ang):
+        xd = x.double()
+        lo, hi = xd[..., :64], xd[..., 64:]
+        return torch.cat((lo * ang.cos() - hi * ang.sin(), hi * ang.cos() + lo * ang.sin()), dim=-1)
+
+    for got, src, a in ((q_loc, q, ang), (rk_rot[:, :, rows], k, ang),
+                        (q_glb, q, torch.full((n, 1), float(n_local - 1), dtype=torch.float64) * inv[None, :])):
+        want = rot(src, a)
+        ulp = want.abs().clamp_min(2.0 ** -126) * 2.0 ** -8          # half a bf16 ulp, relative, plus slack
+        assert bool(((got.cpu().double() - want).abs() <= ulp * 1.01 + 1e-6).all())
+    if pos0 + n < 2 ** 20:   # small positions: also equal to the fp32 oracle up to one bf16 rounding
+        want = rope.rotate(q.float(), list(range(pos0, pos0 + n)))
+        assert float((q_loc.cpu().float() - want).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
+
+
+def test_block_mean():
+    ops = _ops()
+    B, H, n, exc = 2, 3, 70, 32
+    x = _rand((B, H, n, D), 4).cuda()
+    qbar = torch.zeros((B, 3, H * D), dtype=torch.float32, device="cuda")
+    ops.block_mean(x, B, H, n, exc, qbar)
+    xf = x.float()
+    for j, (a, b) in enumerate(((0, 32), (32, 64), (64, 70))):
+        want = xf[:, :, a:b].mean(dim=2).reshape(B, H * D)
+        assert torch.allclose(qbar[:, j], want, atol=1e-5)
+
+
+# ----------------------------------------------------------------- attention
+def _oracle_two_stage(q, stages):
+    a = MultiStageOracle(q.shape)
+    for i, (k, v, kw) in enumerate(stages):
+        a.append(q.float(), k.float(), v.float(), end=(i == len(stages) - 1), get_score=True, **kw)
+    return a.get_result()
+
+
+CASES = [
+    # H, Hkv, Lq, Lk, window kwargs
+    (4, 1, 64, 192, dict(sliding_window=128)),
+    (8, 2, 37, 100, dict(sliding_window=50)),
+    (2, 2, 1, 300, dict(sliding_window=256)),
+    (3, 3, 130, 130, dict(sliding_window=1000)),
+    (4, 2, 96, 257, dict()),
+    (4, 1, 50, 200, dict(sliding_window=(170, 64), complement_sliding_window=True)),
+    (6, 1, 33, 90, dict(sliding_window=(40, 30))),
+    (7, 1, 20, 64, dict(sliding_window=16)),
+]
+
+
+@pytest.mark.parametrize("H,Hkv,Lq,Lk,kw", CASES)
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_single_stage_matches_oracle(H, Hkv, Lq, Lk, kw, nsplit):
+    ops = _ops()
+    B = 2
+    q, k, v = _rand((B, H, Lq, D), 10), _rand((B, Hkv, Lk, D), 11), _rand((B, Hkv, Lk, D), 12)
+    want, (want_score,) = _oracle_two_stage(q, [(k, v, kw)])
+    sw = kw.get("sliding_window")
+    if sw is None:
+        mask, offset, window = ops.MASK_NONE, 0, 0
+    else:
+        offset, window = (Lk - Lq, sw) if isinstance(sw, int) else sw
+        mask = ops.MASK_COMPLEMENT if kw.get("complement_sliding_window") else ops.MASK_WINDOW
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o_part = torch.empty((nsplit, B, H, Lq, D), dtype=torch.float32, device="cuda")
+    lse_part = torch.empty((nsplit, B, H, Lq), dtype=torch.float32, device="cuda")
+    ops.attn_stage_linear(qd, kd, vd, o_part, lse_part, j_lo=0, j_hi=Lk, mask=mask, offset=offset, window=window, nsplit=nsplit)
+    out = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty((B, H, Lq), dtype=torch.float32, device="cuda")
+    ops.attn_merge(o_part, lse_part, nsplit, out, lse)
+    _check_out(out, want)
+    # lse is the base-2 log-sum-exp of the scaled visible logits
+    from oracle.multistage import stage_mask, expand_kv
+    logits = (q.float() @ expand_kv(k.float(), H).transpose(-1, -2)) / math.sqrt(D)
+    vis = stage_mask(Lq, Lk, sw, kw.get("complement_sliding_window", False))
+    want_lse = torch.logsumexp(logits.masked_fill(~vis, float("-inf")), dim=-1) / math.log(2.0)
+    has = vis.any(dim=-1)
+    assert torch.allclose(lse.cpu()[..., has], want_lse[..., has], atol=2e-2)
+    assert bool(torch.isinf(lse.cpu()[..., ~has]).all())
+    assert float(out.float().cpu()[:, :, ~has].abs().max() if (~has).any() else 0.0) == 0.0
+    score = torch.full((B, H, Lk), 7.0, dtype=torch.float32, device="cuda")
+    ops.local_score(qd, kd, lse, score, j_lo=0, j_hi=Lk, mask=mask, offset=offset, window=window, accumulate=False)
+    assert torch.allclose(score.cpu(), want_score, atol=2e-2, rtol=2e-2), float((score.cpu() - want_score).abs().max())
+
+
+def test_two_stage_joint_softmax_with_ring_and_pages():
+    """Local stage from a wrapped ring + global stage from a page table, as the stream uses them."""
+    ops = _ops()
+    B, H, Hkv, Lq, n_local, cap = 1, 8, 2, 64, 256, 384
+    b0 = 1000                                  # absolute position of the first query
+    lo, b1 = b0 - n_local, b0 + Lq
+    q = _rand((B, H, Lq, D), 20)
+    k_win, v_win = _rand((B, Hkv, b1 - lo, D), 21), _rand((B, Hkv, b1 - lo, D), 22)
+    n_glob = 64 * 3 + 50
+    k_g, v_g = _rand((B, Hkv, n_glob, D), 23), _rand((B, Hkv, n_glob, D), 24)
+    want, (want_ls, _) = _oracle_two_stage(q, [(k_win, v_win, dict(sliding_window=n_local)), (k_g, v_g, dict())])
+    ring_k = torch.zeros((B, Hkv, cap, D), dtype=torch.bfloat16, device="cuda")
+    ring_v = torch.zeros_like(ring_k)
+    rows = torch.arange(lo, b1) % cap
+    ring_k[:, :, rows] = k_win.cuda()
+    ring_v[:, :, rows] = v_win.cuda()
+    qd = q.cuda()
+    o_part = torch.empty((2, B, H, Lq, D), dtype=torch.float32, device="cuda")
+    lse_part = torch.empty((2, B, H, Lq), dtype=torch.float32, device="cuda")
+    ops.attn_stage_linear(qd, ring_k, ring_v, o_part[0:1], lse_part[0:1], cap=cap, j_lo=lo, j_hi=b1,
+                          mask=ops.MASK_WINDOW, offset=b0, window=n_local)
+    # pages: scattered 64-row tiles inside one pool, the last one partial
+    pool_k = torch.zeros((Hkv, 1024, D), dtype=torch.bfloat16, device="cuda")
+    pool_v = torch.zeros_like(pool_k)
+    starts = [512, 0, 256, 900]
+    ent, pos = [], 0
+    for s in starts:
+        n = min(64, n_glob - pos)
+        pool_k[:, s:s + n] = k_g[0, :, pos:pos + n].cuda()
+        pool_v[:, s:s + n] = v_g[0, :, pos:pos + n].cuda()
+        ent.append((pool_k.data_ptr() + s * D * 2, pool_v.data_ptr() + s * D * 2, 1024 * D, n))
+        pos += n
+    arr = ops.make_pages(ent)
+    import ctypes
+    host = torch.empty((len(ent) * 32,), dtype=torch.uint8)
+    ctypes.memmove(host.data_ptr(), arr, len(ent) * 32)
+    pages = host.cuda()
+    ops.attn_stage_paged(qd, pages, len(ent), Hkv, o_part[1:2], lse_part[1:2])
+    out = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty((B, H, Lq), dtype=torch.float32, device="cuda")
+    ops.attn_merge(o_part, lse_part, 2, out, lse)
+    _check_out(out, want)
+    score = torch.zeros((B, H, cap), dtype=torch.float32, device="cuda")
+    ops.local_score(qd, ring_k, lse, score, cap=cap, j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW, offset=b0, window=n_local,
+                    accumulate=True, score_cap=cap)
+    ops.local_score(qd, ring_k, lse, score, cap=cap, j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW, offset=b0, window=n_local,
+                    accumulate=True, score_cap=cap)
+    assert torch.allclose(score[:, :, rows].cpu(), 2 * want_ls, atol=2e-2, rtol=2e-2)
+
+
+def test_operator_class_protocol():
+    from infllm_amd.attention.dot_production_attention import get_multi_stage_dot_production_attention
+    Attn, flash = get_multi_stage_dot_production_attention(True)
+    assert flash is True
+    B, H, Hkv, Lq = 1, 4, 2, 48
+    q = _rand((B, H, Lq, D), 30)
+    k1, v1 = _rand((B, Hkv, 120, D), 31), _rand((B, Hkv, 120, D), 32)
+    k2, v2 = _rand((B, Hkv, 70, D), 33), _rand((B, Hkv, 70, D), 34)
+    stages = [(k1, v1, dict(sliding_window=64)), (k2, v2, dict(sliding_window=(72, 64), complement_sliding_window=True))]
+    want, (ws1, ws2) = _oracle_two_stage(q, stages)
+    attn = Attn(q.shape, torch.bfloat16, "cuda")
+    attn.append(q.cuda(), k1.cuda(), v1.cuda(), sliding_window=64, get_score=True)
+    attn.append(q.cuda(), k2.cuda(), v2.cuda(), sliding_window=(72, 64), complement_sliding_window=True, end=True)
+    out, (s1, s2) = attn.get_result()
+    _check_out(out, want)
+    assert s2 is None and torch.allclose(s1.cpu(), ws1, atol=2e-2, rtol=2e-2)
+    with pytest.raises(TypeError):
+        Attn(q.shape, torch.float32, "cuda")
+    # empty second stage
+    attn = Attn(q.shape, torch.bfloat16, "cuda")
+    attn.append(q.cuda(), k1.cuda(), v1.cuda(), sliding_window=64)
+    attn.append(q.cuda(), k2.cuda()[:, :, :0], v2.cuda()[:, :, :0], end=True)
+    want1, _ = _oracle_two_stage(q, [(k1, v1, dict(sliding_window=64))])
+    _check_out(attn.get_result()[0], want1)
+
+
+# ----------------------------------------------------------------- retrieval
+@pytest.mark.parametrize("N,k", [(17, 16), (991, 16), (8192, 16), (5000, 64), (40, 1)])
+def test_score_topk_matches_bruteforce(N, k):
+    ops = _ops()
+    C = 32 * D
+    reps = _rand((N, C), 40 + N)
+    qbar = torch.randn(C, generator=torch.Generator().manual_seed(41))
+    scores = torch.empty((N,), dtype=torch.float32, device="cuda")
+    idx = torch.empty((k,), dtype=torch.int32, device="cuda")
+    ops.score_topk(reps.cuda(), N, qbar.cuda(), k, scores, idx)
+    want = reps.double().numpy() @ qbar.double().numpy()
+    got_scores = scores.cpu().double().numpy()
+    assert np.allclose(got_scores, want, rtol=1e-4, atol=1e-3)
+    got = idx.cpu().tolist()
+    assert got == sorted(got) and len(set(got)) == k
+    # exactly the top-k of the kernel's own fp32 scores (ties at the boundary -> lower index) ...
+    order = sorted(range(N), key=lambda i: (-float(scores[i]), i))
+    assert got == sorted(order[:k])
+    # ... and equal to the oracle's set except for candidates within 1e-3 relative of the boundary
+    want_set = set(np.argsort(-want, kind="stable")[:k].tolist())
+    kth = np.sort(want)[-k]
+    for i in set(got) ^ want_set:
+        assert abs(want[i] - kth) <= 1e-3 * abs(kth)
+
+
+def test_topk_with_exact_ties_takes_lowest_indices():
+    ops = _ops()
+    N, C = 300, 128
+    reps = torch.zeros((N, C), dtype=torch.bfloat16)
+    reps[:, 0] = 1.0
+    reps[200:210, 0] = 2.0
+    qbar = torch.zeros(C)
+    qbar[0] = 1.0
+    scores = torch.empty((N,), dtype=torch.float32, device="cuda")
+    idx = torch.empty((16,), dtype=torch.int32, device="cuda")
+    ops.score_topk(reps.cuda(), N, qbar.cuda(), 16, scores, idx)
+    assert idx.cpu().tolist() == [0, 1, 2, 3, 4, 5] + list(range(200, 210))
+    neg = (-reps).cuda()
+    ops.score_topk(neg, N, qbar.cuda(), 4, scores, idx)
+    assert idx.cpu().tolist()[:4] == [0, 1, 2, 3]
+
+
+@pytest.mark.parametrize("bs,r,H,Hkv", [(128, 4, 32, 8), (8, 2, 4, 2), (100, 1, 3, 3), (64, 64, 2, 1)])
+def test_repr_keys_matches_oracle(bs, r, H, Hkv):
+    ops = _ops()
+    B, cap, n_units, t0 = 2, 640, 3, 600            # units wrap around the end of the ring
+    g = torch.Generator().manual_seed(50)
+    score = torch.rand((B, H, cap), generator=g)
+    ring_k = _rand((B, Hkv, cap, D), 51)
+    reps = torch.zeros((B, n_units + 1, H * D), dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros((B, n_units, H, r), dtype=torch.int32, device="cuda")
+    ops.repr_keys(score.cuda(), ring_k.cuda(), t0, bs, n_units, r, reps[:, 1], reps.stride(0), reps.stride(1), idx)
+    assert float(reps[:, 0].abs().max()) == 0.0
+    for b in range(B):
+        for u in range(n_units):
+            rows = [(t0 + u * bs + i) % cap for i in range(bs)]
+            sc = score[b][:, rows]
+            want_idx = sc.topk(r, dim=-1).indices
+            assert torch.equal(idx[b, u].cpu().long(), want_idx)
+            kx = ring_k[b][:, rows].float().repeat_interleave(H // Hkv, dim=0)
+            want = torch.gather(kx, 1, want_idx[:, :, None].expand(-1, -1, D)).mean(dim=1).reshape(-1)
+            assert torch.allclose(reps[b, u + 1].cpu().float(), want, atol=1e-2, rtol=1e-2)
+            assert torch.equal(reps[b, u + 1].cpu(), want.bfloat16())
+
+
+def test_gather_rows_and_copy_async():
+    ops = _ops()
+    B, Hkv, cap, bs = 2, 3, 256, 40
+    ring = _rand((B, Hkv, cap, D), 60).cuda()
+    t0, n_units = 200, 2
+    stage = torch.zeros((n_units, B, 2, Hkv, bs, D), dtype=torch.bfloat16, device="cuda")
+    ops.gather_rows(ring, t0, n_units * bs, stage[0, 0, 1].data_ptr(), stage.stride(1), stage.stride(3), unit_rows=bs,
+                    out_su=stage.stride(0))
+    for u in range(n_units):
+        rows = [(t0 + u * bs + i) % cap for i in range(bs)]
+        assert torch.equal(stage[u, :, 1], ring[:, :, rows])
+    assert float(stage[:, :, 0].abs().max()) == 0.0
+    host = torch.empty(stage[0].shape, dtype=torch.bfloat16, pin_memory=True)
+    ops.copy_async(host, stage[0], stage[0].numel() * 2, 2)
+    torch.cuda.synchronize()
+    assert torch.equal(host, stage[0].cpu())
+    back = torch.zeros_like(stage[0])
+    ops.copy_async(back, host, host.numel() * 2, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(back, stage[0])
+
+
+def test_bad_arguments_raise():
+    ops = _ops()
+    from infllm_amd._lib import InfLLMHipError
+    q = torch.zeros((1, 4, 8, D), dtype=torch.bfloat16, device="cuda")
+    k = torch.zeros((1, 3, 8, D), dtype=torch.bfloat16, device="cuda")
+    o = torch.zeros((1, 1, 4, 8, D), dtype=torch.float32, device="cuda")
+    l = torch.zeros((1, 1, 4, 8), dtype=torch.float32, device="cuda")
+    with pytest.raises(InfLLMHipError):
+        ops.attn_stage_linear(q, k, k, o, l)                      # 4 heads over 3 kv heads
+    with pytest.raises(InfLLMHipError):
+        ops.attn_stage_linear(q, k[:, :1], k[:, :1], o, l, cap=100)   # cap not a multiple of the tile
+    with pytest.raises(ValueError):
+        ops._bf16_4d(q.float(), "q")

@@ -1,0 +1,184 @@
+"""End-to-end parity of the streaming path on the GPU against the CPU oracle.
+
+The GPU ContextManager and oracle.stream.StreamOracle consume the same
+bf16-rounded stream.  Discrete choices (retrieved unit sets, representative
+keys) must be identical except where the oracle's own fp32 scores of the
+candidates that differ lie within 1e-3 relative of the selection boundary; in
+that case the oracle adopts the GPU's choice (so that the two trajectories stay
+comparable) and the event is counted.  Outputs must agree within max-abs 2e-2 /
+mean-abs 2e-3.
+"""
+import pytest
+import torch
+
+from oracle.rope import RopeOracle
+from oracle.stream import StreamOracle
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS, TIE_REL = 2e-2, 2e-3, 1e-3
+D = 128
+
+
+def _stream(T, H, Hkv, seed, B=1, mixture=True):
+    """q, v ~ N(0,1); keys from a 64-component Gaussian mixture (std 0.3 around N(0,1) means)."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, T, D, generator=g)
+    v = torch.randn(B, Hkv, T, D, generator=g)
+    if mixture:
+        means = torch.randn(Hkv, 64, D, generator=g)
+        comp = torch.randint(0, 64, (B, Hkv, T), generator=g)
+        k = torch.stack([means[h][comp[:, h]] for h in range(Hkv)], dim=1) + 0.3 * torch.randn(B, Hkv, T, D, generator=g)
+    else:
+        k = torch.randn(B, Hkv, T, D, generator=g)
+    return q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+
+def _run_gpu(q, k, v, calls, base, **kw):
+    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
+    rope = RotaryEmbeddingESM(D, base=base, device="cuda")
+    cm = ContextManager(rope, kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"], kw["topk"],
+                        kw["exc_block_size"], kw.get("score_decay"), False, kw.get("repr_topk", 1),
+                        kw.get("cache_strategy", "lru"), None, kw.get("async_global_stream", False), False, False,
+                        kw.get("perhead", False))
+    cm.record_trace = True
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    outs, pos = [], 0
+    for L in calls:
+        sl = slice(pos, pos + L)
+        outs.append(cm.append(qd[:, :, sl], kd[:, :, sl], vd[:, :, sl], qd[:, :, sl], kd[:, :, sl], vd[:, :, sl]))
+        pos += L
+    torch.cuda.synchronize()
+    return torch.cat(outs, dim=2).cpu(), cm
+
+
+class Follower:
+    """Oracle hooks that adopt the GPU's choices when the tie rule allows it."""
+
+    def __init__(self, cm, topk, repr_topk):
+        self.blocks = cm.trace_blocks
+        self.repr = cm.trace_repr_indices()
+        self.topk, self.repr_topk = topk, repr_topk
+        self.tie_topk = self.tie_repr = 0
+        self.violations = []
+
+    def topk_hook(self, block, row, scores):
+        gpu = set(self.blocks[block]["selected"][row])
+        mine = set(scores.topk(self.topk).indices.tolist())
+        if gpu == mine:
+            return None
+        kth = float(scores.topk(self.topk).values[-1])
+        bad = [i for i in gpu ^ mine if abs(float(scores[i]) - kth) > TIE_REL * abs(kth)]
+        if bad:
+            self.violations.append(("topk", block, row, bad))
+        self.tie_topk += 1
+        return sorted(gpu)
+
+    def repr_hook(self, unit, row, score):
+        gpu = self.repr[unit][row].long()                      # [H, r]
+        mine = score.topk(self.repr_topk, dim=-1)
+        for h in range(score.shape[0]):
+            a, b = set(gpu[h].tolist()), set(mine.indices[h].tolist())
+            if a != b:
+                rth = float(mine.values[h, -1])
+                bad = [i for i in a ^ b if abs(float(score[h, i]) - rth) > TIE_REL * abs(rth)]
+                if bad:
+                    self.violations.append(("repr", unit, row, h, bad))
+                self.tie_repr += 1
+        return gpu
+
+
+def _compare(T, calls, H, Hkv, base, seed, B=1, **kw):
+    q, k, v = _stream(T, H, Hkv, seed, B=B)
+    got, cm = _run_gpu(q, k, v, calls, base, **kw)
+    fol = Follower(cm, kw["topk"], kw.get("repr_topk", 1))
+    ora = StreamOracle(RopeOracle(D, base=base), kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"],
+                       kw["topk"], kw["exc_block_size"], repr_topk=kw.get("repr_topk", 1), perhead=kw.get("perhead", False),
+                       topk_hook=fol.topk_hook, repr_hook=fol.repr_hook)
+    outs, pos = [], 0
+    for L in calls:
+        sl = slice(pos, pos + L)
+        outs.append(ora.append(q[:, :, sl].float(), k[:, :, sl].float(), v[:, :, sl].float()))
+        pos += L
+    want = torch.cat(outs, dim=2)
+    assert not fol.violations, fol.violations[:5]
+    assert [b["selected"] for b in cm.trace_blocks] == [b["selected"] for b in ora.block_trace]
+    assert cm.num_global_block == ora.n_units and cm.length == ora.length == T
+    err = (got.float() - want).abs()
+    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (float(err.max()), float(err.mean()))
+    # the cache model saw the same selections, so residency events must match too
+    if not kw.get("perhead", False):
+        hits = sum(len(e["selected"]) - len(e["misses"]) for c in ora.cache for e in c.events)
+        assert cm.stats["hits"] == hits
+    return cm, ora, fol
+
+
+SMALL = dict(n_init=16, n_local=256, block_size=32, max_cached_block=8, topk=4, exc_block_size=64, repr_topk=2)
+
+
+@pytest.mark.parametrize("calls", [[1500], [64] * 20 + [100, 17, 3], [1] * 40 + [700] + [1] * 30])
+def test_small_geometry_follows_oracle(calls):
+    cm, ora, fol = _compare(sum(calls), calls, H=8, Hkv=2, base=1e4, seed=len(calls), **SMALL)
+    assert cm.num_global_block > SMALL["topk"]            # retrieval was exercised
+
+
+def test_unaligned_geometry_and_batch():
+    kw = dict(n_init=5, n_local=130, block_size=24, max_cached_block=3, topk=3, exc_block_size=50, repr_topk=3)
+    _compare(700, [333, 367], H=6, Hkv=3, base=1e4, seed=7, B=2, **kw)
+
+
+def test_no_gqa_and_perhead():
+    kw = dict(SMALL, perhead=True)
+    _compare(800, [800], H=2, Hkv=1, base=1e4, seed=8, **kw)
+    _compare(800, [800], H=2, Hkv=2, base=1e4, seed=9, **SMALL)
+
+
+def test_reference_geometry_16k():
+    """Mistral-7B geometry and the reference's default knobs (config/mistral-inf-llm.yaml)."""
+    kw = dict(n_init=128, n_local=4096, block_size=128, max_cached_block=32, topk=16, exc_block_size=512, repr_topk=4)
+    T = 8192 + 1024
+    cm, ora, fol = _compare(T, [8192, 1024], H=32, Hkv=8, base=1e6, seed=11, **kw)
+    assert cm.num_global_block == (T - 128 - 4096) // 128 > 16
+
+
+def test_call_splitting_cache_size_and_side_stream_do_not_change_results():
+    T = 1280
+    q, k, v = _stream(T, 8, 2, 12)
+    ref, cm0 = _run_gpu(q, k, v, [T], 1e4, **SMALL)
+    split, _ = _run_gpu(q, k, v, [640, 640], 1e4, **SMALL)
+    assert torch.equal(ref, split)
+    tight, cm1 = _run_gpu(q, k, v, [T], 1e4, **dict(SMALL, max_cached_block=4))
+    assert torch.equal(ref, tight) and cm1.stats["misses"] > cm0.stats["misses"]
+    side, cm2 = _run_gpu(q, k, v, [T], 1e4, **dict(SMALL, max_cached_block=4, async_global_stream=True))
+    assert torch.equal(ref, side) and cm2.stats == cm1.stats
+    fifo, _ = _run_gpu(q, k, v, [T], 1e4, **dict(SMALL, cache_strategy="fifo"))
+    assert torch.equal(ref, fifo)
+
+
+def test_attention_type_forward_contract():
+    """ATTN_FORWRAD['inf-llm'] closure: projections in, (output, ContextManager) out (inf_llm.py:20-77)."""
+    from infllm_amd.attention import ATTN_FORWRAD, ContextManager, RotaryEmbeddingESM
+    H, Hkv, hidden, L = 4, 2, 64, 96
+    torch.manual_seed(0)
+    mk = lambda o: torch.nn.Linear(hidden, o, bias=False).cuda().bfloat16()
+    pq, pk, pv, po = mk(H * D), mk(Hkv * D), mk(Hkv * D), torch.nn.Linear(H * D, hidden, bias=False).cuda().bfloat16()
+    fwd = ATTN_FORWRAD["inf-llm"](**dict(SMALL, fattn=False, type="inf-llm"))
+    rope = RotaryEmbeddingESM(D, base=1e4, device="cuda")
+    x = torch.randn(1, L, hidden, device="cuda").bfloat16()
+    with torch.no_grad():
+        o, cm = fwd(None, x, x, rope, True, None, pq, pk, pv, po, D, H, Hkv)
+        o2, cm2 = fwd(None, x[:, :1], x[:, :1], rope, True, cm, pq, pk, pv, po, D, H, Hkv)
+    assert isinstance(cm, ContextManager) and cm2 is cm and cm.length == L + 1 == cm.size()
+    assert o.shape == (1, L, hidden) and o2.shape == (1, 1, hidden) and torch.isfinite(o.float()).all()
+    # inside the window the path is plain causal attention with standard RoPE
+    q = pq(x).view(1, L, H, D).permute(0, 2, 1, 3).float().cpu()
+    k = pk(x).view(1, L, Hkv, D).permute(0, 2, 1, 3).float().cpu()
+    v = pv(x).view(1, L, Hkv, D).permute(0, 2, 1, 3).float().cpu()
+    ro = RopeOracle(D, base=1e4)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        ro.rotate(q, range(L)), ro.rotate(k, range(L)).repeat_interleave(2, 1), v.repeat_interleave(2, 1), is_causal=True)
+    want = po(want.permute(0, 2, 1, 3).reshape(1, L, H * D).cuda().bfloat16())
+    assert float((o.float() - want.float()).abs().max()) < 3e-2
+    bad = torch.zeros(1, H, 1, D, device="cuda")
+    with pytest.raises(TypeError):
+        cm.append(bad, bad, bad, bad, bad, bad)
