@@ -109,6 +109,7 @@ class ContextManager:
         self.initialized = False
         self.load_count = 0
         self.record_trace = False
+        self.kernel_timers = None          # dict(local=[], glob=[]) -> (start, end, n_queries, steady) event pairs
         self.trace_blocks, self.trace_units = [], []
         self.stats = dict(blocks=0, hits=0, misses=0, evictions=0)
         global _SIDE_STREAM
@@ -268,8 +269,15 @@ class ContextManager:
         ops.block_mean(q_glb, B, H, n, n, self.qbar)
         # local stage first: it keeps the GPU busy while the host resolves the retrieval
         lo = max(b0 - self.n_local, 0)
+        tm = self.kernel_timers
+        if tm is not None:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
         ops.attn_stage_linear(q_loc, self.ring_k_rot, self.ring_v, o_part[0:1], lse_part[0:1], cap=self.ring_cap,
                               j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW, offset=b0, window=self.n_local)
+        if tm is not None:
+            e1.record()
+            tm["local"].append((e0, e1, n, n == self.exc_block_size and lo == b0 - self.n_local))
 
         selected = self._retrieve()
         copy_stream = self._copy_stream()
@@ -293,7 +301,13 @@ class ContextManager:
 
         n_pages = self._build_pages(selected, b1)
         if n_pages > 0:
+            if tm is not None:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
             ops.attn_stage_paged(q_glb, self.pages_dev, n_pages, Hkv, o_part[1:2], lse_part[1:2])
+            if tm is not None:
+                e1.record()
+                tm["glob"].append((e0, e1, n, n == self.exc_block_size and self.num_global_block >= self.topk))
             if copy_stream is not main:
                 if self._global_done is None:
                     self._global_done = torch.cuda.Event()

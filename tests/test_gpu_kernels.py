@@ -70,7 +70,7 @@ def test_ingest_matches_rope_oracle(pos0, n):
         want = rot(src, a)
         ulp = want.abs().clamp_min(2.0 ** -126) * 2.0 ** -8          # half a bf16 ulp, relative, plus slack
         assert bool(((got.cpu().double() - want).abs() <= ulp * 1.01 + 1e-6).all())
-    if pos0 + n < 2 ** 20:   # small positions: also equal to the fp32 oracle up to one bf16 rounding
+    if pos0 + n < 10000:     # small positions (fp32 angles still exact enough): equal to the fp32 oracle up to one bf16 rounding
         want = rope.rotate(q.float(), list(range(pos0, pos0 + n)))
         assert float((q_loc.cpu().float() - want).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
 
