@@ -31,6 +31,8 @@ from ..ops import HEAD_DIM, KEY_TILE
 
 _SIDE_STREAM = None          # one process-wide side stream, like GLOBAL_STREAM (context_manager.py:193)
 _HOST_CHUNK_UNITS = 64       # units per pinned host allocation
+_MAX_SPLITS = 16             # key splits of one attention stage
+_NUM_CUS = 256               # MI355X
 
 
 class CachePolicy:
@@ -151,7 +153,7 @@ class ContextManager:
         self.q_loc = torch.empty((B * H * exc * D,), **bf)
         self.q_glb = torch.empty((B * H * exc * D,), **bf)
         self.qbar = torch.empty((B, 1, H * D), dtype=torch.float32, device=dev)
-        self.n_part = 2
+        self.n_part = 2 * _MAX_SPLITS
         self.o_part = torch.empty((self.n_part * B * H * exc * D,), dtype=torch.float32, device=dev)
         self.lse_part = torch.empty((self.n_part * B * H * exc,), dtype=torch.float32, device=dev)
         self.lse = torch.empty((B * H * exc,), dtype=torch.float32, device=dev)
@@ -175,6 +177,13 @@ class ContextManager:
         self._idx_event = torch.cuda.Event()
         self._global_done = None
         self.initialized = True
+
+    def _splits(self, n_queries, n_tiles):
+        """Key splits of one stage: enough workgroups to put about two on every CU, at least 8 tiles each."""
+        G = self.unit_size // self.unit_size_kv
+        wgs = ((n_queries + 31) // 32 * G + 3) // 4 * self.unit_size_kv * self.num_units
+        want = (2 * _NUM_CUS + wgs - 1) // wgs
+        return max(1, min(want, _MAX_SPLITS, n_tiles // 8))
 
     def size(self, *args, **kwargs):
         return self.length
@@ -273,8 +282,9 @@ class ContextManager:
         if tm is not None:
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-        ops.attn_stage_linear(q_loc, self.ring_k_rot, self.ring_v, o_part[0:1], lse_part[0:1], cap=self.ring_cap,
-                              j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW, offset=b0, window=self.n_local)
+        sl = self._splits(n, (b1 - lo + KEY_TILE - 1) // KEY_TILE)
+        ops.attn_stage_linear(q_loc, self.ring_k_rot, self.ring_v, o_part[0:sl], lse_part[0:sl], cap=self.ring_cap,
+                              j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW, offset=b0, window=self.n_local, nsplit=sl)
         if tm is not None:
             e1.record()
             tm["local"].append((e0, e1, n, n == self.exc_block_size and lo == b0 - self.n_local))
@@ -304,7 +314,8 @@ class ContextManager:
             if tm is not None:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
-            ops.attn_stage_paged(q_glb, self.pages_dev, n_pages, Hkv, o_part[1:2], lse_part[1:2])
+            sg = self._splits(n, n_pages)
+            ops.attn_stage_paged(q_glb, self.pages_dev, n_pages, Hkv, o_part[sl:sl + sg], lse_part[sl:sl + sg], nsplit=sg)
             if tm is not None:
                 e1.record()
                 tm["glob"].append((e0, e1, n, n == self.exc_block_size and self.num_global_block >= self.topk))
@@ -312,9 +323,9 @@ class ContextManager:
                 if self._global_done is None:
                     self._global_done = torch.cuda.Event()
                 self._global_done.record(main)
-            ops.attn_merge(o_part, lse_part, 2, out, lse)
+            ops.attn_merge(o_part, lse_part, sl + sg, out, lse)
         else:
-            ops.attn_merge(o_part, lse_part, 1, out, lse)
+            ops.attn_merge(o_part, lse_part, sl, out, lse)
         ops.local_score(q_loc, self.ring_k_rot, lse, self.ring_score, cap=self.ring_cap, j_lo=lo, j_hi=b1,
                         mask=ops.MASK_WINDOW, offset=b0, window=self.n_local, accumulate=True, score_cap=self.ring_cap)
         if self.cache_strategy == "lru-s":

@@ -23,8 +23,8 @@ namespace {
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kQTile = 32;                 // queries per wave
+constexpr int kBig = 1 << 29;              // clamp for mask distances held in int32
 constexpr int kKPad = kD + 8;              // LDS row of K  (bf16 elements)
-constexpr int kVPad = kTile + 8;           // LDS row of V^T (bf16 elements)
 
 struct StageRange {
     int64_t lo, hi;   // key index range [lo, hi) visible to a span of queries
@@ -44,10 +44,19 @@ __device__ __forceinline__ StageRange visible_range(const infllm_attn_args &a, i
 
 __device__ __forceinline__ int floordiv64(int64_t x) { return (int)(x >> 6); }   // arithmetic shift = floor
 
+// LDS layouts (both free of bank conflicts for the 16-byte MFMA operand reads):
+//   Ks[buf][row][kKPad]  row = key with bits 2 and 3 swapped inside each 32-key half, so that the
+//                        lane holding MFMA row r reads LDS row r; 272-byte rows rotate the banks.
+//   Vt[buf][d][64 keys]  128-byte rows cut into eight 16-byte units of 8 keys; unit u of row d is
+//                        stored at unit u ^ (d & 7) ^ ((d >> 3) & 7).
+__device__ __forceinline__ int k_lds_row(int key) { return (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1); }
+__device__ __forceinline__ int vt_unit(int d, int u) { return u ^ (d & 7) ^ ((d >> 3) & 7); }
+
 template <bool PAGED>
 __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[kTile][kKPad];
-    __shared__ __attribute__((aligned(16))) bf16_t Vt[kD][kVPad];
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[2][kTile][kKPad];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt[2][kD][kTile];
+    __shared__ int wg_lo[kWaves], wg_hi[kWaves];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
@@ -78,7 +87,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         }
     }
     // ---- workgroup range = union over its waves; the split takes a contiguous share of it
-    __shared__ int wg_lo[kWaves], wg_hi[kWaves];
     if (lane == 0) {
         wg_lo[wave] = w_t1 > w_t0 ? w_t0 : INT32_MAX;
         wg_hi[wave] = w_t1 > w_t0 ? w_t1 : INT32_MIN;
@@ -144,10 +152,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                                                    : u32x4{0, 0, 0, 0};
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *(u32x4 *)&Ks[ld_row + 16 * i][ld_chunk * 8] = kbuf[i];
-        // 4 keys x 8 dims -> 8 dims x 4 keys
+        for (int i = 0; i < 4; ++i) *(u32x4 *)&Ks[buf][k_lds_row(ld_row + 16 * i)][ld_chunk * 8] = kbuf[i];
+        // 4 keys x 8 dims -> 8 dims x 4 keys (8 bytes each)
+        const int unit = ld_row >> 1, half = (ld_row & 1) * 4;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             u32x2 even, odd;                  // dims 2w and 2w+1 of keys 0..3
@@ -155,12 +164,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             even[1] = (vbuf[2][w] & 0xffffu) | (vbuf[3][w] << 16);
             odd[0] = (vbuf[0][w] >> 16) | (vbuf[1][w] & 0xffff0000u);
             odd[1] = (vbuf[2][w] >> 16) | (vbuf[3][w] & 0xffff0000u);
-            *(u32x2 *)&Vt[ld_chunk * 8 + 2 * w][4 * ld_row] = even;
-            *(u32x2 *)&Vt[ld_chunk * 8 + 2 * w + 1][4 * ld_row] = odd;
+            const int d0 = ld_chunk * 8 + 2 * w;
+            *(u32x2 *)&Vt[buf][d0][vt_unit(d0, unit) * 8 + half] = even;
+            *(u32x2 *)&Vt[buf][d0 + 1][vt_unit(d0 + 1, unit) * 8 + half] = odd;
         }
     };
 
-    // ---- running softmax state of this lane's query
+    // ---- running softmax state of this lane's query (max kept in raw logit units)
     float m_run = -INFINITY, l_run = 0.f;
     f32x16 oacc[kD / 32];
 #pragma unroll
@@ -169,102 +179,113 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
 
     const float scale = a.softmax_scale * 1.4426950408889634f;
-    // MFMA row -> key of a 32-key sub-tile
-    const int pi_row = 16 * (col >> 4) + 8 * ((col >> 2) & 1) + 4 * ((col >> 3) & 1) + (col & 3);
-    const int64_t qpos = (int64_t)i0 + col + a.offset;          // query index shifted into key index space
 
-    if (g_t1 > g_t0) load_tile(g_t0);
+    if (g_t1 > g_t0) {
+        load_tile(g_t0);
+        store_tile(0);
+        if (g_t0 + 1 < g_t1) load_tile(g_t0 + 1);
+    }
+    __syncthreads();
     for (int t = g_t0; t < g_t1; ++t) {
-        __syncthreads();                       // previous tile fully consumed
-        store_tile();
-        __syncthreads();
-        if (t + 1 < g_t1) load_tile(t + 1);     // in flight while this tile is computed
-        if (t < w_t0 || t >= w_t1) continue;    // wave-uniform; barriers stay outside
-
-        f32x16 s[2];
+        const int cur = (t - g_t0) & 1;
+        if (t >= w_t0 && t < w_t1) {           // wave-uniform; the barrier stays outside
+            f32x16 s[2];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+            for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[ks][r] = 0.f;
-            const bf16_t *krow = &Ks[ks * 32 + pi_row][grp * 8];
+                for (int r = 0; r < 16; ++r) s[ks][r] = 0.f;
+                const bf16_t *krow = &Ks[cur][ks * 32 + col][grp * 8];
 #pragma unroll
-            for (int kk = 0; kk < kD / 16; ++kk) {
-                bf16x8 ka = *(const bf16x8 *)(krow + kk * 16);
-                s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[kk], s[ks], 0, 0, 0);
+                for (int kk = 0; kk < kD / 16; ++kk) {
+                    bf16x8 ka = *(const bf16x8 *)(krow + kk * 16);
+                    s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[kk], s[ks], 0, 0, 0);
+                }
             }
-        }
-        // ---- mask (only tiles that touch a boundary) and scale
-        bool need_mask;
-        int row_lo = 0, row_hi = kTile;
-        const int64_t j0 = (int64_t)t * kTile;
-        if (PAGED) {
-            row_hi = a.d_pages[(int64_t)b * a.n_pages + t].n_valid;
-            need_mask = row_hi < kTile;
-        } else {
-            row_lo = (int)max((int64_t)0, a.j_lo - j0);
-            row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
-            need_mask = row_lo > 0 || row_hi < kTile;
-            if (a.mask == INFLLM_MASK_WINDOW) {
-                // fully visible iff the oldest query still sees the newest key... check both ends
-                need_mask |= (j0 + kTile - 1 > (int64_t)i0 + a.offset) ||
-                             (j0 < (int64_t)i1 + a.offset - a.window + 1);
-            } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
-                need_mask |= (j0 + kTile - 1 > (int64_t)i0 + a.offset - a.window);
+            // ---- mask (only tiles that touch a boundary); distances are clamped into int32
+            bool need_mask;
+            int row_lo = 0, row_hi = kTile;
+            int d0 = 0;                            // dist of (this lane's query, key 0 of the tile)
+            if (PAGED) {
+                row_hi = a.d_pages[(int64_t)b * a.n_pages + t].n_valid;
+                need_mask = row_hi < kTile;
+            } else {
+                const int64_t j0 = (int64_t)t * kTile;
+                row_lo = (int)max((int64_t)0, a.j_lo - j0);
+                row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
+                need_mask = row_lo > 0 || row_hi < kTile;
+                const int64_t e0 = (int64_t)i0 + a.offset - j0;       // dist(query i0, key j0)
+                if (a.mask == INFLLM_MASK_WINDOW) {
+                    need_mask |= (e0 < kTile - 1) || (e0 + (i1 - i0) >= a.window);
+                } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
+                    need_mask |= (e0 - (kTile - 1) < a.window);
+                }
+                d0 = (int)min(max(e0, (int64_t)-kBig), (int64_t)kBig) + col;
             }
-        }
-        float tmax = -INFINITY;
+            if (need_mask) {
+                const int win = (int)min(a.window, (int64_t)2 * kBig);
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+                for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float x = s[ks][r] * scale;
-                if (need_mask) {
-                    const int ko = ks * 32 + 16 * (r >> 3) + 8 * grp + (r & 7);
-                    bool vis = ko >= row_lo && ko < row_hi;
-                    if (!PAGED) {
-                        const int64_t dist = qpos - (j0 + ko);
-                        if (a.mask == INFLLM_MASK_WINDOW) vis = vis && dist >= 0 && dist < a.window;
-                        if (a.mask == INFLLM_MASK_COMPLEMENT) vis = vis && dist >= a.window;
+                    for (int r = 0; r < 16; ++r) {
+                        const int ko = ks * 32 + 16 * (r >> 3) + 8 * grp + (r & 7);
+                        bool vis = ko >= row_lo && ko < row_hi;
+                        if (!PAGED) {
+                            const int dist = d0 - ko;
+                            if (a.mask == INFLLM_MASK_WINDOW) vis = vis && dist >= 0 && dist < win;
+                            if (a.mask == INFLLM_MASK_COMPLEMENT) vis = vis && dist >= win;
+                        }
+                        s[ks][r] = vis ? s[ks][r] : -INFINITY;
                     }
-                    x = vis ? x : -INFINITY;
+            }
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[ks][r]);
+            tmax = fmaxf(tmax, wave_xor32(tmax));
+            const float m_new = fmaxf(m_run, tmax);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale);
+            const float neg_ms = -m_use * scale;
+            float psum = 0.f;
+            uint32_t pw[2][8];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r], scale, neg_ms));
+                    float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r + 1], scale, neg_ms));
+                    psum += p0 + p1;
+                    pw[ks][r >> 1] = pack_bf16x2(p0, p1);
                 }
-                s[ks][r] = x;
-                tmax = fmaxf(tmax, x);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {     // some query of the wave moved its max
+#pragma unroll
+                for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
             }
-        tmax = fmaxf(tmax, wave_xor32(tmax));
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-        float psum = 0.f;
-        uint32_t pw[2][8];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+            for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                float p0 = __builtin_amdgcn_exp2f(s[ks][r] - m_use);
-                float p1 = __builtin_amdgcn_exp2f(s[ks][r + 1] - m_use);
-                psum += p0 + p1;
-                pw[ks][r >> 1] = pack_bf16x2(p0, p1);
-            }
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
+                for (int mm = 0; mm < 2; ++mm) {
+                    u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
+                    bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+                    const int u = ks * 4 + mm * 2 + grp;
 #pragma unroll
-        for (int dt = 0; dt < kD / 32; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int mm = 0; mm < 2; ++mm) {
-                u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
-                bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
-#pragma unroll
-                for (int dt = 0; dt < kD / 32; ++dt) {
-                    bf16x8 va = *(const bf16x8 *)&Vt[dt * 32 + col][ks * 32 + 16 * mm + 8 * grp];
-                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, oacc[dt], 0, 0, 0);
+                    for (int dt = 0; dt < kD / 32; ++dt) {
+                        const int d = dt * 32 + col;
+                        bf16x8 va = *(const bf16x8 *)&Vt[cur][d][vt_unit(d, u) * 8];
+                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, oacc[dt], 0, 0, 0);
+                    }
                 }
-            }
+        }
+        if (t + 1 < g_t1) {
+            store_tile(cur ^ 1);                // the other buffer was last read one barrier ago
+            if (t + 2 < g_t1) load_tile(t + 2);  // in flight during the next tile's math
+        }
+        __syncthreads();
     }
 
     // ---- epilogue: normalised partial + base-2 log-sum-exp
@@ -283,7 +304,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                      oacc[dt][4 * q4 + 3] * inv};
             *(f32x4 *)(orow + dt * 32 + 8 * q4 + 4 * grp) = o4;
         }
-    if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run + log2f(l_tot) : -INFINITY;
+    if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run * scale + log2f(l_tot) : -INFINITY;
 }
 
 // one thread per (row, 4 dims): P partials -> bf16 output row + final lse

@@ -44,8 +44,12 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     u += 0x7fffu + ((u >> 16) & 1u);
     return u >> 16;
 }
+// two fp32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 __device__ __forceinline__ float wave_xor32(float x) {
     return __shfl_xor(x, 32, 64);
