@@ -197,6 +197,91 @@ int infllm_gather_rows(const void *d_ring, int64_t ring_cap, int32_t B, int32_t 
                        int64_t out_su, int64_t out_sh, void *stream);
 int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int32_t kind, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * One execution block in two calls.
+ * Replaces the device work of ContextManager._append and append_global
+ * (context_manager.py:474-545, 614-679) for one block of at most exc_block_size
+ * queries; the host keeps the decisions (cache policy, state machine):
+ *
+ *   infllm_block_front   prologue (RoPE + rings), mean query, unit scores + top-k with
+ *                        an asynchronous copy of the indices to pinned memory, then the
+ *                        local stage (which keeps the GPU busy while the host decides);
+ *   infllm_layer_wait_topk   blocks until those indices are readable on the host;
+ *   infllm_block_back    fetch of missed units (copy stream), page table, global stage,
+ *                        merge, local score, init peeling, representatives of the new
+ *                        units and their copy to pinned host memory (copy stream).
+ *
+ * A layer handle owns only events, the rotation of the pinned page-table staging
+ * slots and of the carve staging slots; every buffer is the caller's.
+ */
+typedef struct {
+    int32_t B, H, Hkv;
+    int32_t n_local, n_init, block_size, exc, topk, repr_topk, max_cached;
+    int32_t max_splits, num_cus;
+    int64_t ring_cap;
+    void *d_ring_k_raw, *d_ring_k_rot, *d_ring_v;     /* [B,Hkv,ring_cap,128] */
+    float *d_ring_score;                              /* [B,H,ring_cap] */
+    void *d_init_kv;                                  /* [B,2,Hkv,init_cap,128] */
+    int64_t init_cap;
+    void *d_slab;                                     /* [B,max_cached,2,Hkv,block_size,128] */
+    void *d_q_loc, *d_q_glb;                          /* [B*H*exc*128] each */
+    float *d_qbar;                                    /* [B,H*128] */
+    float *d_o_part, *d_lse_part, *d_lse;             /* [2*max_splits,B,H,exc,(128)], [B,H,exc] */
+    int32_t *d_topk_idx, *h_topk_idx;                 /* [B,topk] device / pinned host */
+    infllm_page *d_pages;                             /* [B,max_pages] */
+    infllm_page *h_pages;                             /* pinned, [page_slots,B,max_pages] */
+    int32_t max_pages, page_slots;
+    void *d_carve_stage;                              /* [carve_slots,max_carve,B,2,Hkv,block_size,128] */
+    int32_t max_carve, carve_slots;
+    const float *d_inv_freq;
+    double distance_scale;
+    float softmax_scale;
+    int32_t reserved;
+} infllm_layer_desc;
+
+void *infllm_layer_create(const infllm_layer_desc *desc);    /* NULL + infllm_last_error() on failure */
+int infllm_layer_destroy(void *layer);
+
+typedef struct {
+    const void *d_q, *d_k, *d_v;                      /* this block's rows: [B,H,n,128], [B,Hkv,n,128] */
+    int64_t q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl;
+    int32_t n;                                        /* queries in the block, 1..exc */
+    int32_t n_units;                                  /* units carved so far (per batch row) */
+    int64_t b0;                                       /* stream position of the first query */
+    const void *d_reps;                               /* [B, rows, H*128] bf16 representatives */
+    int64_t rep_sb, rep_su;
+    float *d_unit_scores;                             /* [B, >= n_units] */
+    int64_t unit_scores_sb;
+} infllm_front_args;
+int infllm_block_front(void *layer, const infllm_front_args *a, void *stream);
+int infllm_layer_wait_topk(void *layer);
+
+typedef struct {
+    int32_t n, n_sel;                                 /* queries; selected units per batch row */
+    int64_t b0;
+    const int32_t *h_sel_slots;                       /* host [B,n_sel]: slab slot of each selected unit */
+    int32_t n_miss, init_len;                         /* units to fetch; init tokens present */
+    const int32_t *h_miss_row, *h_miss_slot;          /* host [n_miss] */
+    const void *const *h_miss_src;                    /* host [n_miss]: pinned [2,Hkv,block_size,128] */
+    int64_t cursor;                                   /* first un-carved stream position */
+    void *d_out;                                      /* [B,H,n,128] bf16 */
+    int64_t o_sb, o_sh, o_sl;
+    int32_t init_take, n_carve;                       /* state-machine actions after the block */
+    void *d_rep_out;                                  /* representative row of the first new unit */
+    int64_t rep_sb, rep_su;
+    int32_t *d_repr_idx;                              /* optional [B,n_carve,H,repr_topk] */
+    void *const *h_carve_dst;                         /* host [n_carve]: pinned [B,2,Hkv,block_size,128] */
+} infllm_back_args;
+int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream);
+
+/* Event timing of the two attention stages (for benchmarks): enable with a record
+ * capacity, read back (which: 0 local stage, 1 global stage) after a device sync.
+ * ms[i] is the launch-to-finish time of one stage launch, n_queries[i] its block size,
+ * n_keys[i] the key rows its source held. */
+int infllm_layer_timing(void *layer, int32_t capacity);
+int infllm_layer_read_timing(void *layer, int32_t which, float *ms, int32_t *n_queries, int32_t *n_keys,
+                             int32_t capacity);
+
 #ifdef __cplusplus
 }
 #endif

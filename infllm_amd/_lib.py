@@ -60,6 +60,48 @@ class ScoreArgs(C.Structure):
     ]
 
 
+class LayerDesc(C.Structure):
+    _fields_ = [
+        ("B", c_i32), ("H", c_i32), ("Hkv", c_i32),
+        ("n_local", c_i32), ("n_init", c_i32), ("block_size", c_i32), ("exc", c_i32), ("topk", c_i32),
+        ("repr_topk", c_i32), ("max_cached", c_i32), ("max_splits", c_i32), ("num_cus", c_i32),
+        ("ring_cap", c_i64),
+        ("d_ring_k_raw", c_vp), ("d_ring_k_rot", c_vp), ("d_ring_v", c_vp), ("d_ring_score", c_vp),
+        ("d_init_kv", c_vp), ("init_cap", c_i64), ("d_slab", c_vp),
+        ("d_q_loc", c_vp), ("d_q_glb", c_vp), ("d_qbar", c_vp),
+        ("d_o_part", c_vp), ("d_lse_part", c_vp), ("d_lse", c_vp),
+        ("d_topk_idx", c_vp), ("h_topk_idx", c_vp),
+        ("d_pages", c_vp), ("h_pages", c_vp), ("max_pages", c_i32), ("page_slots", c_i32),
+        ("d_carve_stage", c_vp), ("max_carve", c_i32), ("carve_slots", c_i32),
+        ("d_inv_freq", c_vp), ("distance_scale", c_f64), ("softmax_scale", c_f32), ("reserved", c_i32),
+    ]
+
+
+class FrontArgs(C.Structure):
+    _fields_ = [
+        ("d_q", c_vp), ("d_k", c_vp), ("d_v", c_vp),
+        ("q_sb", c_i64), ("q_sh", c_i64), ("q_sl", c_i64),
+        ("k_sb", c_i64), ("k_sh", c_i64), ("k_sl", c_i64),
+        ("v_sb", c_i64), ("v_sh", c_i64), ("v_sl", c_i64),
+        ("n", c_i32), ("n_units", c_i32), ("b0", c_i64),
+        ("d_reps", c_vp), ("rep_sb", c_i64), ("rep_su", c_i64),
+        ("d_unit_scores", c_vp), ("unit_scores_sb", c_i64),
+    ]
+
+
+class BackArgs(C.Structure):
+    _fields_ = [
+        ("n", c_i32), ("n_sel", c_i32), ("b0", c_i64),
+        ("h_sel_slots", c_vp), ("n_miss", c_i32), ("init_len", c_i32),
+        ("h_miss_row", c_vp), ("h_miss_slot", c_vp), ("h_miss_src", c_vp),
+        ("cursor", c_i64),
+        ("d_out", c_vp), ("o_sb", c_i64), ("o_sh", c_i64), ("o_sl", c_i64),
+        ("init_take", c_i32), ("n_carve", c_i32),
+        ("d_rep_out", c_vp), ("rep_sb", c_i64), ("rep_su", c_i64),
+        ("d_repr_idx", c_vp), ("h_carve_dst", c_vp),
+    ]
+
+
 # name -> (restype, argtypes); every symbol include/infllm_hip.h declares
 SYMBOLS = {
     "infllm_version": (c_i32, []),
@@ -74,6 +116,13 @@ SYMBOLS = {
                                  c_vp, c_i64, c_i64, c_vp, c_vp]),
     "infllm_gather_rows": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i64, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "infllm_copy_async": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_vp]),
+    "infllm_layer_create": (c_vp, [C.POINTER(LayerDesc)]),
+    "infllm_layer_destroy": (c_i32, [c_vp]),
+    "infllm_block_front": (c_i32, [c_vp, C.POINTER(FrontArgs), c_vp]),
+    "infllm_layer_wait_topk": (c_i32, [c_vp]),
+    "infllm_block_back": (c_i32, [c_vp, C.POINTER(BackArgs), c_vp, c_vp]),
+    "infllm_layer_timing": (c_i32, [c_vp, c_i32]),
+    "infllm_layer_read_timing": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32]),
 }
 
 _lib = None

@@ -15,24 +15,31 @@ stream positions and device-resident rings instead of torch.cat/trim:
   softmax; the local score (probability column sums) is a third kernel that
   needs the merged log-sum-exp;
 * memory units live in pinned host memory (always) and in a slab of
-  ``max_cached_block`` device slots managed by the reference's lru / lru-s
-  policy (plus fifo); misses are fetched with hipMemcpyAsync on a side stream.
+  ``max_cached_block`` device slots managed by the reference's lru policy
+  (plus fifo); misses are fetched with hipMemcpyAsync on a side stream.
 
-State machine in absolute positions (context_manager.py:614-679 restated):
-``cursor`` is the first token not yet carved, tokens [0, init_len) are the
-attention sinks, unit u is tokens [n_init + u*bs, n_init + (u+1)*bs).
+The host keeps the decisions - the cache policy and the state machine, in
+absolute positions (context_manager.py:614-679 restated): ``cursor`` is the
+first token not yet carved, tokens [0, init_len) are the attention sinks, unit
+u is tokens [n_init + u*bs, n_init + (u+1)*bs).  The device work of one
+execution block is issued by two native calls, infllm_block_front and
+infllm_block_back, with one host wait (for the retrieved unit ids) in between,
+which overlaps the local stage.
 """
 import ctypes
 
 import torch
 
-from .. import ops
+from .. import _lib
+from .._lib import BackArgs, FrontArgs, LayerDesc, check
 from ..ops import HEAD_DIM, KEY_TILE
 
 _SIDE_STREAM = None          # one process-wide side stream, like GLOBAL_STREAM (context_manager.py:193)
 _HOST_CHUNK_UNITS = 64       # units per pinned host allocation
 _MAX_SPLITS = 16             # key splits of one attention stage
 _NUM_CUS = 256               # MI355X
+_PAGE_SLOTS = 4
+_CARVE_SLOTS = 4
 
 
 class CachePolicy:
@@ -51,31 +58,32 @@ class CachePolicy:
 
     def touch(self, selected):
         """Returns (misses, evicted) and updates values; slots of evicted units are freed."""
-        misses = [b for b in selected if b not in self.cached]
-        surplus = len(self.cached) - self.capacity + len(misses)
+        cached = self.cached
+        misses = [b for b in selected if b not in cached]
+        surplus = len(cached) - self.capacity + len(misses)
         evicted = []
         if surplus > 0:
             chosen = set(selected)
-            for unit, _ in sorted(self.cached.items(), key=lambda kv: kv[1]):
+            for unit, _ in sorted(cached.items(), key=lambda kv: kv[1]):
                 if unit not in chosen:
                     evicted.append(unit)
                 if len(evicted) >= surplus:
                     break
             for unit in evicted:
-                del self.cached[unit]
+                del cached[unit]
                 self.free.append(self.slot_of.pop(unit))
         if self.strategy == "lru":
             self.clock += 1
             for b in selected:
-                self.cached[b] = self.clock
+                cached[b] = self.clock
         elif self.strategy == "fifo":
             self.clock += 1
             for b in selected:
-                self.cached.setdefault(b, self.clock)
+                cached.setdefault(b, self.clock)
         else:                                   # lru-s
             for b in selected:
-                self.cached[b] = 0
-        assert len(self.cached) <= self.capacity, "topk exceeds max_cached_block"
+                cached[b] = 0
+        assert len(cached) <= self.capacity, "topk exceeds max_cached_block"
         for b in misses:
             self.slot_of[b] = self.free.pop()
         return misses, evicted
@@ -95,8 +103,10 @@ class ContextManager:
         assert cache_strategy in ("lru", "lru-s", "fifo")
         if faiss:
             raise NotImplementedError("the faiss representative store is not available in this build")
-        if cache_strategy == "lru-s" and score_decay is None:
-            raise ValueError("cache_strategy='lru-s' needs score_decay")
+        if cache_strategy == "lru-s":
+            raise NotImplementedError("cache_strategy='lru-s' needs the per-unit global score kernel (not built yet)")
+        if chunk_topk_calc is not None:
+            raise NotImplementedError("chunk_topk_calc is not implemented yet")
         self.length = 0
         self.position_embedding = position_embedding
         self.n_init, self.n_local = n_init, n_local
@@ -111,12 +121,22 @@ class ContextManager:
         self.initialized = False
         self.load_count = 0
         self.record_trace = False
-        self.kernel_timers = None          # dict(local=[], glob=[]) -> (start, end, n_queries, steady) event pairs
         self.trace_blocks, self.trace_units = [], []
         self.stats = dict(blocks=0, hits=0, misses=0, evictions=0)
+        self._layer = None
+        self._timing_cap = 0
         global _SIDE_STREAM
         if async_global_stream and _SIDE_STREAM is None and torch.cuda.is_available():
             _SIDE_STREAM = torch.cuda.Stream()
+
+    def __del__(self):
+        layer, self._layer = getattr(self, "_layer", None), None
+        if layer:
+            try:
+                torch.cuda.synchronize()
+                _lib.load().infllm_layer_destroy(layer)
+            except Exception:
+                pass
 
     # ------------------------------------------------------------------ setup
     def _init(self, q, k):
@@ -127,24 +147,28 @@ class ContextManager:
             raise ValueError(f"the HIP kernels are built for head_dim {HEAD_DIM}, got {D}")
         if self.topk > self.max_cached_block:
             raise ValueError("topk must not exceed max_cached_block")
+        if self.repr_topk > self.block_size:
+            raise ValueError("repr_topk must not exceed block_size")
         self.batch_size = self.num_units = B
         self.num_heads = self.unit_size = H
         self.num_heads_kv = self.unit_size_kv = Hkv
         self.dim_head = D
         self.dtype = q.dtype
         self.device = dev
-        bs, exc = self.block_size, self.exc_block_size
+        bs, exc, topk = self.block_size, self.exc_block_size, self.topk
         cap = self.n_local + exc + bs
         self.ring_cap = cap = (cap + KEY_TILE - 1) // KEY_TILE * KEY_TILE + KEY_TILE
         bf = dict(dtype=torch.bfloat16, device=dev)
+        f32 = dict(dtype=torch.float32, device=dev)
         self.ring_k_raw = torch.zeros((B, Hkv, cap, D), **bf)
         self.ring_k_rot = torch.zeros((B, Hkv, cap, D), **bf)
         self.ring_v = torch.zeros((B, Hkv, cap, D), **bf)
-        self.ring_score = torch.zeros((B, H, cap), dtype=torch.float32, device=dev)
+        self.ring_score = torch.zeros((B, H, cap), **f32)
         self.init_kv = torch.zeros((B, 2, Hkv, max(self.n_init, 1), D), **bf)
         self.slab = torch.zeros((B, self.max_cached_block, 2, Hkv, bs, D), **bf)
         self.reps = torch.zeros((B, 16, H * D), **bf)
-        self.host_chunks = []
+        self.unit_scores = torch.empty((B, 16), **f32)
+        self.host_chunks, self._host_base = [], []
         self.policy = [CachePolicy(self.max_cached_block, self.cache_strategy, self.score_decay) for _ in range(B)]
         self.cursor = 0
         self.init_len = 0
@@ -152,240 +176,189 @@ class ContextManager:
         # workspaces of one execution block
         self.q_loc = torch.empty((B * H * exc * D,), **bf)
         self.q_glb = torch.empty((B * H * exc * D,), **bf)
-        self.qbar = torch.empty((B, 1, H * D), dtype=torch.float32, device=dev)
-        self.n_part = 2 * _MAX_SPLITS
-        self.o_part = torch.empty((self.n_part * B * H * exc * D,), dtype=torch.float32, device=dev)
-        self.lse_part = torch.empty((self.n_part * B * H * exc,), dtype=torch.float32, device=dev)
-        self.lse = torch.empty((B * H * exc,), dtype=torch.float32, device=dev)
-        self.topk_idx = torch.empty((B, max(self.topk, 1)), dtype=torch.int32, device=dev)
-        self.topk_idx_host = torch.empty((B, max(self.topk, 1)), dtype=torch.int32, pin_memory=True)
-        self.unit_scores = torch.empty((B, 16), dtype=torch.float32, device=dev)
+        self.qbar = torch.empty((B, H * D), **f32)
+        n_part = 2 * _MAX_SPLITS
+        self.o_part = torch.empty((n_part * B * H * exc * D,), **f32)
+        self.lse_part = torch.empty((n_part * B * H * exc,), **f32)
+        self.lse = torch.empty((B * H * exc,), **f32)
+        self.topk_idx = torch.zeros((B, max(topk, 1)), dtype=torch.int32, device=dev)
+        self.topk_idx_host = torch.zeros((B, max(topk, 1)), dtype=torch.int32, pin_memory=True)
         tiles_per_unit = (bs + KEY_TILE - 1) // KEY_TILE
-        self.max_pages = (self.topk * tiles_per_unit + (self.n_init + KEY_TILE - 1) // KEY_TILE
-                          + (exc + bs) // KEY_TILE + 3)
-        self.page_bytes = ctypes.sizeof(ops.Page)
-        self.pages_dev = torch.empty((B * self.max_pages * self.page_bytes,), dtype=torch.uint8, device=dev)
-        self._page_stage = [torch.empty((B * self.max_pages * self.page_bytes,), dtype=torch.uint8, pin_memory=True)
-                            for _ in range(4)]
-        self._page_stage_evt = [None] * 4
-        self._page_stage_cur = 0
-        self._carve_stage = [None] * 4
-        self._carve_evt = [None] * 4
-        self._carve_cur = 0
+        self.max_pages = topk * tiles_per_unit + (self.n_init + KEY_TILE - 1) // KEY_TILE + (exc + bs) // KEY_TILE + 3
+        page_bytes = ctypes.sizeof(_lib.Page)
+        self.pages_dev = torch.empty((B * self.max_pages * page_bytes,), dtype=torch.uint8, device=dev)
+        self.pages_host = torch.empty((_PAGE_SLOTS * B * self.max_pages * page_bytes,), dtype=torch.uint8, pin_memory=True)
+        self.max_carve = (exc + self.n_init) // bs + 2
+        self.carve_stage = torch.empty((_CARVE_SLOTS, self.max_carve, B, 2, Hkv, bs, D), **bf)
         self.inv_freq = self.position_embedding.inv_freq.to(device=dev, dtype=torch.float32).contiguous()
-        self.distance_scale = float(self.position_embedding.distance_scale)
-        self._idx_event = torch.cuda.Event()
-        self._global_done = None
-        self.initialized = True
+        self.slot_bytes = 2 * Hkv * bs * D * 2              # one unit of one batch row
+        self.unit_bytes = B * self.slot_bytes               # one unit, all batch rows
 
-    def _splits(self, n_queries, n_tiles):
-        """Key splits of one stage: enough workgroups to put about two on every CU, at least 8 tiles each."""
-        G = self.unit_size // self.unit_size_kv
-        wgs = ((n_queries + 31) // 32 * G + 3) // 4 * self.unit_size_kv * self.num_units
-        want = (2 * _NUM_CUS + wgs - 1) // wgs
-        return max(1, min(want, _MAX_SPLITS, n_tiles // 8))
+        d = LayerDesc()
+        d.B, d.H, d.Hkv = B, H, Hkv
+        d.n_local, d.n_init, d.block_size, d.exc = self.n_local, self.n_init, bs, exc
+        d.topk, d.repr_topk, d.max_cached = topk, self.repr_topk, self.max_cached_block
+        d.max_splits, d.num_cus, d.ring_cap = _MAX_SPLITS, _NUM_CUS, cap
+        d.d_ring_k_raw, d.d_ring_k_rot = self.ring_k_raw.data_ptr(), self.ring_k_rot.data_ptr()
+        d.d_ring_v, d.d_ring_score = self.ring_v.data_ptr(), self.ring_score.data_ptr()
+        d.d_init_kv, d.init_cap, d.d_slab = self.init_kv.data_ptr(), self.init_kv.shape[3], self.slab.data_ptr()
+        d.d_q_loc, d.d_q_glb, d.d_qbar = self.q_loc.data_ptr(), self.q_glb.data_ptr(), self.qbar.data_ptr()
+        d.d_o_part, d.d_lse_part, d.d_lse = self.o_part.data_ptr(), self.lse_part.data_ptr(), self.lse.data_ptr()
+        d.d_topk_idx, d.h_topk_idx = self.topk_idx.data_ptr(), self.topk_idx_host.data_ptr()
+        d.d_pages, d.h_pages = self.pages_dev.data_ptr(), self.pages_host.data_ptr()
+        d.max_pages, d.page_slots = self.max_pages, _PAGE_SLOTS
+        d.d_carve_stage, d.max_carve, d.carve_slots = self.carve_stage.data_ptr(), self.max_carve, _CARVE_SLOTS
+        d.d_inv_freq = self.inv_freq.data_ptr()
+        d.distance_scale = float(self.position_embedding.distance_scale)
+        d.softmax_scale = 1.0 / (D ** 0.5)
+        self._lib = _lib.load()
+        self._layer = self._lib.infllm_layer_create(ctypes.byref(d))
+        if not self._layer:
+            raise _lib.InfLLMHipError("infllm_layer_create failed: " + (self._lib.infllm_last_error() or b"").decode())
+        if self._timing_cap:
+            check(self._lib.infllm_layer_timing(self._layer, self._timing_cap), "infllm_layer_timing")
+        # argument blocks and host arrays reused by every block
+        self._fa, self._ba = FrontArgs(), BackArgs()
+        self._sel_slots = (ctypes.c_int32 * (B * max(topk, 1)))()
+        self._miss_row = (ctypes.c_int32 * (B * max(topk, 1)))()
+        self._miss_slot = (ctypes.c_int32 * (B * max(topk, 1)))()
+        self._miss_src = (ctypes.c_void_p * (B * max(topk, 1)))()
+        self._carve_dst = (ctypes.c_void_p * self.max_carve)()
+        ba = self._ba
+        ba.h_sel_slots = ctypes.addressof(self._sel_slots)
+        ba.h_miss_row, ba.h_miss_slot = ctypes.addressof(self._miss_row), ctypes.addressof(self._miss_slot)
+        ba.h_miss_src, ba.h_carve_dst = ctypes.addressof(self._miss_src), ctypes.addressof(self._carve_dst)
+        self._fa_ref, self._ba_ref = ctypes.byref(self._fa), ctypes.byref(self._ba)
+        self.initialized = True
 
     def size(self, *args, **kwargs):
         return self.length
 
     # ------------------------------------------------------------ host memory
-    def _host_unit(self, unit):
-        """Pinned host tensor [B, 2, Hkv, bs, D] of a unit."""
+    def _host_unit_addr(self, unit):
+        """Address of the pinned host copy [B, 2, Hkv, bs, D] of a unit."""
         chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
         while chunk >= len(self.host_chunks):
-            self.host_chunks.append(torch.empty(
-                (_HOST_CHUNK_UNITS, self.num_units, 2, self.unit_size_kv, self.block_size, self.dim_head),
-                dtype=torch.bfloat16, pin_memory=True))
+            t = torch.empty((_HOST_CHUNK_UNITS, self.num_units, 2, self.unit_size_kv, self.block_size, self.dim_head),
+                            dtype=torch.bfloat16, pin_memory=True)
+            self.host_chunks.append(t)
+            self._host_base.append(t.data_ptr())
+        return self._host_base[chunk] + idx * self.unit_bytes
+
+    def host_unit(self, unit):
+        """Pinned host tensor [B, 2, Hkv, bs, D] of a carved unit (K at index 0, V at 1)."""
+        chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
         return self.host_chunks[chunk][idx]
 
-    def _copy_stream(self):
-        return _SIDE_STREAM if self.async_global_stream else torch.cuda.current_stream()
+    # ----------------------------------------------------------------- timing
+    def enable_timing(self, capacity):
+        """Event-time every local / global stage launch (up to `capacity` of each) for benchmarks."""
+        self._timing_cap = capacity
+        if self._layer:
+            check(self._lib.infllm_layer_timing(self._layer, capacity), "infllm_layer_timing")
 
-    # -------------------------------------------------------------- retrieval
-    def _retrieve(self):
-        """Unit ids per batch row for the current block (context_manager.py:366-383)."""
-        N, B = self.num_global_block, self.num_units
-        if N <= self.topk:
-            return [list(range(N)) for _ in range(B)]
-        if self.unit_scores.shape[1] < N:
-            self.unit_scores = torch.empty((B, self.reps.shape[1]), dtype=torch.float32, device=self.device)
-        for u in range(B):
-            ops.score_topk(self.reps[u], N, self.qbar[u], self.topk, self.unit_scores[u], self.topk_idx[u])
-        self.topk_idx_host.copy_(self.topk_idx, non_blocking=True)
-        self._idx_event.record()
-        self._idx_event.synchronize()          # the one host sync of a block (context_manager.py:163)
-        return self.topk_idx_host.tolist()
-
-    # ------------------------------------------------------------- page table
-    def _build_pages(self, selected, b1):
-        B, bs, D = self.num_units, self.block_size, self.dim_head
-        esz = 2
-        unit_stride = self.unit_size_kv * bs * D                       # K -> V inside a slot
-        overflow_end = max(b1 - self.n_local, self.cursor)
-        rows = []
-        for u in range(B):
-            ent = []
-            slab_u = self.slab[u]
-            for unit in selected[u]:
-                slot = self.policy[u].slot_of[unit]
-                k_addr = slab_u[slot].data_ptr()
-                for t0 in range(0, bs, KEY_TILE):
-                    ent.append((k_addr + t0 * D * esz, k_addr + (unit_stride + t0 * D) * esz, bs * D, min(KEY_TILE, bs - t0)))
-            ik = self.init_kv[u, 0].data_ptr()
-            iv = self.init_kv[u, 1].data_ptr()
-            ilen = self.init_kv.shape[3]
-            for t0 in range(0, self.init_len, KEY_TILE):
-                ent.append((ik + t0 * D * esz, iv + t0 * D * esz, ilen * D, min(KEY_TILE, self.init_len - t0)))
-            rk, rv = self.ring_k_raw[u].data_ptr(), self.ring_v[u].data_ptr()
-            pos = self.cursor
-            while pos < overflow_end:
-                row = pos % self.ring_cap
-                n = min(KEY_TILE, overflow_end - pos, self.ring_cap - row)
-                ent.append((rk + row * D * esz, rv + row * D * esz, self.ring_cap * D, n))
-                pos += n
-            rows.append(ent)
-        n_pages = len(rows[0])
-        assert all(len(r) == n_pages for r in rows) and n_pages <= self.max_pages
-        if n_pages == 0:
-            return 0
-        arr = ops.make_pages([e for r in rows for e in r])
-        slot = self._page_stage_cur
-        self._page_stage_cur = (slot + 1) % len(self._page_stage)
-        if self._page_stage_evt[slot] is not None:
-            self._page_stage_evt[slot].synchronize()
-        nbytes = B * n_pages * self.page_bytes
-        ctypes.memmove(self._page_stage[slot].data_ptr(), arr, nbytes)
-        ops.copy_async(self.pages_dev, self._page_stage[slot], nbytes, 1)
-        evt = self._page_stage_evt[slot] or torch.cuda.Event()
-        evt.record()
-        self._page_stage_evt[slot] = evt
-        return n_pages
+    def read_timing(self, which):
+        """[(ms, n_queries, n_keys)] of the timed launches; which = 0 local stage, 1 global stage."""
+        cap = self._timing_cap
+        ms, nq, nk = (ctypes.c_float * cap)(), (ctypes.c_int32 * cap)(), (ctypes.c_int32 * cap)()
+        n = self._lib.infllm_layer_read_timing(self._layer, which, ms, nq, nk, cap)
+        if n < 0:
+            check(n, "infllm_layer_read_timing")
+        return [(ms[i], nq[i], nk[i]) for i in range(n)]
 
     # -------------------------------------------------------- one exec block
-    def _block(self, q, k, v, out, b0):
-        B, H, Hkv, D = self.num_units, self.unit_size, self.unit_size_kv, self.dim_head
-        n = q.shape[2]
+    def _block(self, st, n, out_ptr):
+        lib, layer, fa, ba = self._lib, self._layer, self._fa, self._ba
+        B, bs, topk = self.num_units, self.block_size, self.topk
+        b0 = self.length + st
         b1 = b0 + n
-        main = torch.cuda.current_stream()
-        q_loc = self.q_loc[:B * H * n * D].view(B, H, n, D)
-        q_glb = self.q_glb[:B * H * n * D].view(B, H, n, D)
-        o_part = self.o_part[:self.n_part * B * H * n * D].view(self.n_part, B, H, n, D)
-        lse_part = self.lse_part[:self.n_part * B * H * n].view(self.n_part, B, H, n)
-        lse = self.lse[:B * H * n].view(B, H, n)
-
-        ops.ingest(q, k, v, b0, self.n_local - 1, self.inv_freq, self.distance_scale,
-                   self.ring_k_raw, self.ring_k_rot, self.ring_v, self.ring_score, q_loc, q_glb)
-        ops.block_mean(q_glb, B, H, n, n, self.qbar)
-        # local stage first: it keeps the GPU busy while the host resolves the retrieval
-        lo = max(b0 - self.n_local, 0)
-        tm = self.kernel_timers
-        if tm is not None:
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-        sl = self._splits(n, (b1 - lo + KEY_TILE - 1) // KEY_TILE)
-        ops.attn_stage_linear(q_loc, self.ring_k_rot, self.ring_v, o_part[0:sl], lse_part[0:sl], cap=self.ring_cap,
-                              j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW, offset=b0, window=self.n_local, nsplit=sl)
-        if tm is not None:
-            e1.record()
-            tm["local"].append((e0, e1, n, n == self.exc_block_size and lo == b0 - self.n_local))
-
-        selected = self._retrieve()
-        copy_stream = self._copy_stream()
-        fetched = False
+        N = self.num_global_block
+        fa.d_q = self._q_ptr + st * self._q_step
+        fa.d_k = self._k_ptr + st * self._k_step
+        fa.d_v = self._v_ptr + st * self._v_step
+        fa.n, fa.n_units, fa.b0 = n, N, b0
+        rc = lib.infllm_block_front(layer, self._fa_ref, self._main_raw)
+        if rc:
+            check(rc, "infllm_block_front")
+        # ---- retrieval result (context_manager.py:366-383)
+        if N <= topk:
+            selected = [list(range(N))] * B
+        else:
+            rc = lib.infllm_layer_wait_topk(layer)           # the one host wait of a block
+            if rc:
+                check(rc, "infllm_layer_wait_topk")
+            selected = self.topk_idx_host.tolist()
+        # ---- cache policy (context_manager.py:495-515)
+        n_sel = len(selected[0])
+        n_miss = 0
+        stats = self.stats
         for u in range(B):
-            misses, evicted = self.policy[u].touch(selected[u])
-            self.stats["hits"] += len(selected[u]) - len(misses)
-            self.stats["misses"] += len(misses)
-            self.stats["evictions"] += len(evicted)
+            pol = self.policy[u]
+            misses, evicted = pol.touch(selected[u])
+            stats["hits"] += n_sel - len(misses)
+            stats["misses"] += len(misses)
+            stats["evictions"] += len(evicted)
+            slot_of = pol.slot_of
+            base = u * n_sel
+            for i, unit in enumerate(selected[u]):
+                self._sel_slots[base + i] = slot_of[unit]
             for unit in misses:
-                if not fetched and copy_stream is not main and self._global_done is not None:
-                    copy_stream.wait_event(self._global_done)   # the slot may still be read by the previous block
-                fetched = True
-                slot = self.policy[u].slot_of[unit]
-                src = self._host_unit(unit)[u]
-                ops.copy_async(self.slab[u, slot], src, src.numel() * 2, 1, copy_stream.cuda_stream)
-        if fetched and copy_stream is not main:
-            main.wait_stream(copy_stream)
+                self._miss_row[n_miss] = u
+                self._miss_slot[n_miss] = slot_of[unit]
+                self._miss_src[n_miss] = self._host_unit_addr(unit) + u * self.slot_bytes
+                n_miss += 1
         if self.cache_strategy == "lru":
             self.load_count += 1
-
-        n_pages = self._build_pages(selected, b1)
-        if n_pages > 0:
-            if tm is not None:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-            sg = self._splits(n, n_pages)
-            ops.attn_stage_paged(q_glb, self.pages_dev, n_pages, Hkv, o_part[sl:sl + sg], lse_part[sl:sl + sg], nsplit=sg)
-            if tm is not None:
-                e1.record()
-                tm["glob"].append((e0, e1, n, n == self.exc_block_size and self.num_global_block >= self.topk))
-            if copy_stream is not main:
-                if self._global_done is None:
-                    self._global_done = torch.cuda.Event()
-                self._global_done.record(main)
-            ops.attn_merge(o_part, lse_part, sl + sg, out, lse)
-        else:
-            ops.attn_merge(o_part, lse_part, sl, out, lse)
-        ops.local_score(q_loc, self.ring_k_rot, lse, self.ring_score, cap=self.ring_cap, j_lo=lo, j_hi=b1,
-                        mask=ops.MASK_WINDOW, offset=b0, window=self.n_local, accumulate=True, score_cap=self.ring_cap)
-        if self.cache_strategy == "lru-s":
-            raise NotImplementedError("lru-s needs the per-unit global score kernel")
-        if self.record_trace:
-            self.trace_blocks.append(dict(b0=b0, b1=b1, selected=[sorted(s) for s in selected], n_units=self.num_global_block,
-                                          init_len=self.init_len, n_pages=n_pages))
-        self.stats["blocks"] += 1
-        self._after_block(b1)
-
-    def _after_block(self, b1):
-        """Init peeling and unit carving (context_manager.py:614-679) in absolute positions."""
-        B, H, Hkv, D, bs = self.num_units, self.unit_size, self.unit_size_kv, self.dim_head, self.block_size
-        live = b1 - self.cursor
-        if self.init_len < self.n_init and live > self.n_local:
-            take = min(self.n_init - self.init_len, live - self.n_local)
-            ilen = self.init_kv.shape[3]
-            for which, ring in ((0, self.ring_k_raw), (1, self.ring_v)):
-                ops.gather_rows(ring, self.cursor, take, self.init_kv[:, which, :, self.init_len].data_ptr(),
-                                2 * Hkv * ilen * D, ilen * D)
-            self.init_len += take
-            self.cursor += take
+        # ---- state machine after the block (context_manager.py:614-679)
+        cursor, init_len = self.cursor, self.init_len
+        live = b1 - cursor
+        take = 0
+        if init_len < self.n_init and live > self.n_local:
+            take = min(self.n_init - init_len, live - self.n_local)
             live -= take
         c = max((live - self.n_local) // bs, 0)
-        if c == 0:
-            return
-        N = self.num_global_block
-        if N + c > self.reps.shape[1]:
-            grown = torch.zeros((B, max(2 * self.reps.shape[1], N + c), H * D), dtype=torch.bfloat16, device=self.device)
-            grown[:, :N] = self.reps[:, :N]
-            self.reps = grown
-        idx_out = torch.empty((B, c, H, self.repr_topk), dtype=torch.int32, device=self.device) if self.record_trace else None
-        ops.repr_keys(self.ring_score, self.ring_k_raw, self.cursor, bs, c, self.repr_topk,
-                      self.reps[:, N], self.reps.stride(0), self.reps.stride(1), idx_out)
+        ba.n, ba.n_sel, ba.b0 = n, n_sel, b0
+        ba.n_miss, ba.init_len, ba.cursor = n_miss, init_len, cursor
+        ba.d_out = out_ptr
+        ba.init_take, ba.n_carve = take, c
+        idx_out = None
+        if c:
+            if N + c > self.reps.shape[1]:
+                self._grow_reps(N + c)
+            ba.d_rep_out = self._reps_ptr + N * self._rep_su_bytes
+            for i in range(c):
+                self._carve_dst[i] = self._host_unit_addr(N + i)
+            if self.record_trace:
+                idx_out = torch.empty((B, c, self.unit_size, self.repr_topk), dtype=torch.int32, device=self.device)
+            ba.d_repr_idx = idx_out.data_ptr() if idx_out is not None else None
+        rc = lib.infllm_block_back(layer, self._ba_ref, self._main_raw, self._copy_raw)
+        if rc:
+            check(rc, "infllm_block_back")
         if self.record_trace:
-            self.trace_units.append((N, c, idx_out))
-        # carve: ring -> contiguous device staging -> pinned host (the units' permanent home)
-        slot = self._carve_cur
-        self._carve_cur = (slot + 1) % len(self._carve_stage)
-        if self._carve_evt[slot] is not None:
-            self._carve_evt[slot].synchronize()
-        stage = self._carve_stage[slot]
-        if stage is None or stage.shape[0] < c:
-            stage = torch.empty((max(c, 4), B, 2, Hkv, bs, D), dtype=torch.bfloat16, device=self.device)
-            self._carve_stage[slot] = stage
-        for which, ring in ((0, self.ring_k_raw), (1, self.ring_v)):
-            ops.gather_rows(ring, self.cursor, c * bs, stage[0, 0, which].data_ptr(), stage.stride(1), stage.stride(3),
-                            unit_rows=bs, out_su=stage.stride(0))
-        main = torch.cuda.current_stream()
-        copy_stream = self._copy_stream()
-        if copy_stream is not main:
-            copy_stream.wait_stream(main)
-        unit_bytes = B * 2 * Hkv * bs * D * 2
-        for i in range(c):
-            ops.copy_async(self._host_unit(N + i), stage[i], unit_bytes, 2, copy_stream.cuda_stream)
-        evt = self._carve_evt[slot] or torch.cuda.Event()
-        evt.record(copy_stream)
-        self._carve_evt[slot] = evt
-        self.cursor += c * bs
-        self.num_global_block += c
+            self.trace_blocks.append(dict(b0=b0, b1=b1, selected=[sorted(s) for s in selected], n_units=N, init_len=init_len))
+            if c:
+                self.trace_units.append((N, c, idx_out))
+        stats["blocks"] += 1
+        self.init_len = init_len + take
+        self.cursor = cursor + take + c * bs
+        self.num_global_block = N + c
+
+    def _grow_reps(self, need):
+        B, N = self.num_units, self.num_global_block
+        rows = max(2 * self.reps.shape[1], need)
+        grown = torch.zeros((B, rows, self.reps.shape[2]), dtype=torch.bfloat16, device=self.device)
+        grown[:, :N] = self.reps[:, :N]
+        self.reps = grown
+        self.unit_scores = torch.empty((B, rows), dtype=torch.float32, device=self.device)
+        self._bind_reps()
+
+    def _bind_reps(self):
+        fa, ba = self._fa, self._ba
+        self._reps_ptr = self.reps.data_ptr()
+        self._rep_su_bytes = self.reps.stride(1) * 2
+        fa.d_reps, fa.rep_sb, fa.rep_su = self._reps_ptr, self.reps.stride(0), self.reps.stride(1)
+        fa.d_unit_scores, fa.unit_scores_sb = self.unit_scores.data_ptr(), self.unit_scores.stride(0)
+        ba.rep_sb, ba.rep_su = self.reps.stride(0), self.reps.stride(1)
 
     # ----------------------------------------------------------------- append
     def append(self, local_q, local_k, local_v, global_q, global_k, global_v):
@@ -408,14 +381,28 @@ class ContextManager:
             q, k, v = q.reshape(batch_size * heads, 1, input_length, -1), rep(k), rep(v)
         if not self.initialized:
             self._init(q, k)
+            self._bind_reps()
         assert q.shape[:2] == (self.num_units, self.unit_size) and k.shape[1] == self.unit_size_kv
-        q, k, v = ops._bf16_4d(q, "q"), ops._bf16_4d(k, "k"), ops._bf16_4d(v, "v")
+
+        def rows16(t):          # rows must be contiguous and 16-byte aligned for the vector loads
+            ok = t.stride(-1) == 1 and not any(s % 8 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+            return t if ok else t.contiguous()
+        q, k, v = rows16(q), rows16(k), rows16(v)
         out = torch.empty((self.num_units, self.unit_size, input_length, self.dim_head), dtype=torch.bfloat16, device=q.device)
-        if self.chunk_topk_calc is not None and input_length > 1:
-            raise NotImplementedError("chunk_topk_calc is not implemented yet")
-        for st in range(0, input_length, self.exc_block_size):
-            ed = min(st + self.exc_block_size, input_length)
-            self._block(q[:, :, st:ed], k[:, :, st:ed], v[:, :, st:ed], out[:, :, st:ed], self.length + st)
+        fa, ba = self._fa, self._ba
+        fa.q_sb, fa.q_sh, fa.q_sl = q.stride(0), q.stride(1), q.stride(2)
+        fa.k_sb, fa.k_sh, fa.k_sl = k.stride(0), k.stride(1), k.stride(2)
+        fa.v_sb, fa.v_sh, fa.v_sl = v.stride(0), v.stride(1), v.stride(2)
+        ba.o_sb, ba.o_sh, ba.o_sl = out.stride(0), out.stride(1), out.stride(2)
+        self._q_ptr, self._k_ptr, self._v_ptr = q.data_ptr(), k.data_ptr(), v.data_ptr()
+        self._q_step, self._k_step, self._v_step = q.stride(2) * 2, k.stride(2) * 2, v.stride(2) * 2
+        main = torch.cuda.current_stream()
+        self._main_raw = main.cuda_stream
+        self._copy_raw = _SIDE_STREAM.cuda_stream if self.async_global_stream else self._main_raw
+        out_ptr, out_step = out.data_ptr(), out.stride(2) * 2
+        exc = self.exc_block_size
+        for st in range(0, input_length, exc):
+            self._block(st, min(exc, input_length - st), out_ptr + st * out_step)
         self.length += input_length
         if self.perhead:
             out = out.view(batch_size, heads, input_length, -1)

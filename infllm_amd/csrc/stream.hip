@@ -1,0 +1,387 @@
+// One execution block of the streaming path in two calls
+// (inf_llm/attention/context_manager.py:474-545, 614-679): the launches of a block are
+// issued natively, back to back, so that the host interpreter is not on the GPU's
+// critical path.  Decisions (which units are cached, what gets carved) stay with the caller.
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+struct StageTimer {
+    std::vector<hipEvent_t> ev;       // pairs
+    std::vector<int> n_queries, n_keys;
+    int used = 0;
+};
+
+struct Layer {
+    infllm_layer_desc d;
+    hipEvent_t topk_done = nullptr;       // indices of the last front() are in pinned memory
+    hipEvent_t global_done = nullptr;     // last global stage has read the slab
+    hipEvent_t fetch_done = nullptr;      // missed units are in their slots
+    hipEvent_t carve_ready = nullptr;     // carve staging filled
+    std::vector<hipEvent_t> page_evt, carve_evt;
+    std::vector<char> page_busy, carve_busy;
+    int page_cur = 0, carve_cur = 0;
+    bool has_global = false;
+    bool topk_pending = false;
+    int timing_cap = 0;
+    StageTimer timer[2];
+};
+
+#define HIP_OK(call, what)                                                              \
+    do {                                                                                \
+        hipError_t e_ = (call);                                                         \
+        if (e_ != hipSuccess) return infllm_fail(-2, "%s: %s", what, hipGetErrorString(e_)); \
+    } while (0)
+
+int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
+    const int G = d.H / d.Hkv;
+    const int wgs = (((n_queries + 31) / 32) * G + 3) / 4 * d.Hkv * d.B;
+    int want = (2 * d.num_cus + wgs - 1) / wgs;
+    int cap = n_tiles / 8;
+    int s = want < d.max_splits ? want : d.max_splits;
+    if (s > cap) s = cap;
+    return s < 1 ? 1 : s;
+}
+
+int timer_begin(Layer *L, int which, int n_queries, int n_keys, hipStream_t st) {
+    StageTimer &t = L->timer[which];
+    if (L->timing_cap <= 0 || t.used >= L->timing_cap) return -1;
+    const int i = t.used++;
+    t.n_queries[i] = n_queries;
+    t.n_keys[i] = n_keys;
+    (void)hipEventRecord(t.ev[2 * i], st);
+    return i;
+}
+
+void timer_end(Layer *L, int which, int i, hipStream_t st) {
+    if (i >= 0) (void)hipEventRecord(L->timer[which].ev[2 * i + 1], st);
+}
+
+}  // namespace
+
+extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
+    auto bad = [](const char *m) -> void * {
+        infllm_fail(-1, "layer_create: %s", m);
+        return nullptr;
+    };
+    if (!desc) return bad("null descriptor");
+    const infllm_layer_desc &d = *desc;
+    if (d.B <= 0 || d.H <= 0 || d.Hkv <= 0 || d.H % d.Hkv) return bad("bad head geometry");
+    if (d.exc <= 0 || d.exc > d.n_local || d.block_size <= 0 || d.topk < 0 || d.topk > d.max_cached) return bad("bad knobs");
+    if (d.ring_cap % kTile || d.ring_cap < (int64_t)d.n_local + d.exc + d.block_size) return bad("ring too small or unaligned");
+    if (!d.d_ring_k_raw || !d.d_ring_k_rot || !d.d_ring_v || !d.d_ring_score || !d.d_init_kv || !d.d_slab || !d.d_q_loc ||
+        !d.d_q_glb || !d.d_qbar || !d.d_o_part || !d.d_lse_part || !d.d_lse || !d.d_topk_idx || !d.h_topk_idx || !d.d_pages ||
+        !d.h_pages || !d.d_carve_stage || !d.d_inv_freq)
+        return bad("null buffer");
+    if (d.max_splits < 1 || d.max_splits > 64 || d.num_cus < 1 || d.page_slots < 1 || d.carve_slots < 1 || d.max_carve < 1 ||
+        d.max_pages < 1 || d.init_cap < 1)
+        return bad("bad capacities");
+    Layer *L = new Layer();
+    L->d = d;
+    bool ok = hipEventCreateWithFlags(&L->topk_done, hipEventDisableTiming) == hipSuccess &&
+              hipEventCreateWithFlags(&L->global_done, hipEventDisableTiming) == hipSuccess &&
+              hipEventCreateWithFlags(&L->fetch_done, hipEventDisableTiming) == hipSuccess &&
+              hipEventCreateWithFlags(&L->carve_ready, hipEventDisableTiming) == hipSuccess;
+    L->page_evt.resize(d.page_slots, nullptr);
+    L->carve_evt.resize(d.carve_slots, nullptr);
+    L->page_busy.assign(d.page_slots, 0);
+    L->carve_busy.assign(d.carve_slots, 0);
+    for (auto &e : L->page_evt) ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
+    for (auto &e : L->carve_evt) ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
+    if (!ok) {
+        infllm_layer_destroy(L);
+        return bad("hipEventCreate failed");
+    }
+    return L;
+}
+
+extern "C" int infllm_layer_destroy(void *layer) {
+    if (!layer) return 0;
+    Layer *L = (Layer *)layer;
+    for (hipEvent_t e : {L->topk_done, L->global_done, L->fetch_done, L->carve_ready})
+        if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : L->page_evt)
+        if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : L->carve_evt)
+        if (e) (void)hipEventDestroy(e);
+    for (auto &t : L->timer)
+        for (hipEvent_t e : t.ev)
+            if (e) (void)hipEventDestroy(e);
+    delete L;
+    return 0;
+}
+
+extern "C" int infllm_layer_timing(void *layer, int32_t capacity) {
+    INFLLM_REQUIRE(layer && capacity >= 0, "layer_timing: bad arguments");
+    Layer *L = (Layer *)layer;
+    for (auto &t : L->timer) {
+        while ((int)t.ev.size() < 2 * capacity) {
+            hipEvent_t e;
+            HIP_OK(hipEventCreate(&e), "layer_timing");
+            t.ev.push_back(e);
+        }
+        t.n_queries.resize(capacity);
+        t.n_keys.resize(capacity);
+        t.used = 0;
+    }
+    L->timing_cap = capacity;
+    return 0;
+}
+
+extern "C" int infllm_layer_read_timing(void *layer, int32_t which, float *ms, int32_t *n_queries, int32_t *n_keys,
+                                        int32_t capacity) {
+    INFLLM_REQUIRE(layer && (which == 0 || which == 1) && ms && capacity >= 0, "layer_read_timing: bad arguments");
+    Layer *L = (Layer *)layer;
+    StageTimer &t = L->timer[which];
+    int n = t.used < capacity ? t.used : capacity;
+    for (int i = 0; i < n; ++i) {
+        HIP_OK(hipEventElapsedTime(&ms[i], t.ev[2 * i], t.ev[2 * i + 1]), "layer_read_timing");
+        if (n_queries) n_queries[i] = t.n_queries[i];
+        if (n_keys) n_keys[i] = t.n_keys[i];
+    }
+    return n;
+}
+
+extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void *stream) {
+    INFLLM_REQUIRE(layer && a, "block_front: null argument");
+    Layer *L = (Layer *)layer;
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream;
+    INFLLM_REQUIRE(a->n >= 1 && a->n <= d.exc, "block_front: %d queries do not fit an execution block of %d", a->n, d.exc);
+    INFLLM_REQUIRE(a->n_units >= 0 && a->b0 >= 0, "block_front: negative state");
+
+    infllm_ingest_args in{};
+    in.d_q = a->d_q; in.d_k = a->d_k; in.d_v = a->d_v;
+    in.q_sb = a->q_sb; in.q_sh = a->q_sh; in.q_sl = a->q_sl;
+    in.k_sb = a->k_sb; in.k_sh = a->k_sh; in.k_sl = a->k_sl;
+    in.v_sb = a->v_sb; in.v_sh = a->v_sh; in.v_sl = a->v_sl;
+    in.B = d.B; in.H = d.H; in.Hkv = d.Hkv; in.n = a->n;
+    in.pos0 = a->b0; in.glb_pos = d.n_local - 1;
+    in.d_inv_freq = d.d_inv_freq; in.distance_scale = d.distance_scale;
+    in.d_ring_k_raw = d.d_ring_k_raw; in.d_ring_k_rot = d.d_ring_k_rot; in.d_ring_v = d.d_ring_v;
+    in.d_ring_score = d.d_ring_score; in.ring_cap = d.ring_cap;
+    in.d_q_loc = d.d_q_loc; in.d_q_glb = d.d_q_glb;
+    int rc = infllm_ingest(&in, stream);
+    if (rc) return rc;
+
+    L->topk_pending = false;
+    if (a->n_units > d.topk) {
+        INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
+        rc = infllm_block_mean(d.d_q_glb, d.B, d.H, a->n, a->n, d.d_qbar, stream);
+        if (rc) return rc;
+        const int C = d.H * kD;
+        for (int u = 0; u < d.B; ++u) {
+            rc = infllm_score_topk((const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb, a->rep_su, a->n_units, C,
+                                   d.d_qbar + (int64_t)u * C, d.topk, a->d_unit_scores + (int64_t)u * a->unit_scores_sb,
+                                   d.d_topk_idx + (int64_t)u * d.topk, stream);
+            if (rc) return rc;
+        }
+        HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st),
+               "block_front: index copy");
+        HIP_OK(hipEventRecord(L->topk_done, st), "block_front: event");
+        L->topk_pending = true;
+    }
+
+    // local stage: causal sliding window over the ring
+    const int64_t b1 = a->b0 + a->n;
+    const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
+    infllm_attn_args at{};
+    at.d_q = d.d_q_loc;
+    at.q_sl = kD; at.q_sh = (int64_t)a->n * kD; at.q_sb = (int64_t)d.H * a->n * kD;
+    at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = a->n;
+    at.d_k = d.d_ring_k_rot; at.d_v = d.d_ring_v;
+    at.k_sl = at.v_sl = kD;
+    at.k_sh = at.v_sh = d.ring_cap * kD;
+    at.k_sb = at.v_sb = (int64_t)d.Hkv * d.ring_cap * kD;
+    at.cap = d.ring_cap; at.j_lo = lo; at.j_hi = b1;
+    at.mask = INFLLM_MASK_WINDOW; at.offset = a->b0; at.window = d.n_local;
+    at.nsplit = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
+    at.softmax_scale = d.softmax_scale;
+    at.d_o_part = d.d_o_part; at.d_lse_part = d.d_lse_part;
+    const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
+    rc = infllm_attn_stage(&at, stream);
+    timer_end(L, 0, ti, st);
+    return rc;
+}
+
+extern "C" int infllm_layer_wait_topk(void *layer) {
+    INFLLM_REQUIRE(layer, "layer_wait_topk: null layer");
+    Layer *L = (Layer *)layer;
+    if (!L->topk_pending) return 0;
+    HIP_OK(hipEventSynchronize(L->topk_done), "layer_wait_topk");
+    L->topk_pending = false;
+    return 0;
+}
+
+extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream) {
+    INFLLM_REQUIRE(layer && a, "block_back: null argument");
+    Layer *L = (Layer *)layer;
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream, cs = (hipStream_t)copy_stream;
+    const bool side = cs != st;
+    const int bs = d.block_size;
+    INFLLM_REQUIRE(a->n >= 1 && a->n <= d.exc && a->n_sel >= 0 && a->n_sel <= d.topk, "block_back: bad block sizes");
+    INFLLM_REQUIRE(a->n_miss >= 0 && a->n_miss <= d.B * a->n_sel && a->init_len >= 0 && a->init_len <= d.init_cap,
+                   "block_back: bad miss / init counts");
+    INFLLM_REQUIRE(a->n_sel == 0 || a->h_sel_slots, "block_back: null slot list");
+    INFLLM_REQUIRE(a->n_miss == 0 || (a->h_miss_row && a->h_miss_slot && a->h_miss_src), "block_back: null miss list");
+    INFLLM_REQUIRE(a->d_out && a->cursor >= 0 && a->init_take >= 0 && a->n_carve >= 0 && a->n_carve <= d.max_carve,
+                   "block_back: bad output / carve arguments");
+    const int64_t b1 = a->b0 + a->n;
+    const int64_t unit_elems = (int64_t)d.Hkv * bs * kD;          // K (or V) of one unit
+    const int64_t slot_elems = 2 * unit_elems;
+
+    // ---- 1. fetch missed units into their slots (copy stream)
+    if (a->n_miss > 0) {
+        if (side && L->has_global) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "block_back: wait global");
+        for (int i = 0; i < a->n_miss; ++i) {
+            const int u = a->h_miss_row[i], slot = a->h_miss_slot[i];
+            INFLLM_REQUIRE(u >= 0 && u < d.B && slot >= 0 && slot < d.max_cached && a->h_miss_src[i], "block_back: bad miss entry");
+            bf16_t *dst = (bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + slot) * slot_elems;
+            HIP_OK(hipMemcpyAsync(dst, a->h_miss_src[i], slot_elems * sizeof(bf16_t), hipMemcpyHostToDevice, cs),
+                   "block_back: unit fetch");
+        }
+        if (side) {
+            HIP_OK(hipEventRecord(L->fetch_done, cs), "block_back: event");
+            HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
+        }
+    }
+
+    // ---- 2. page table of the global stage: units | init | overflow remainder
+    const int64_t overflow_end = b1 - d.n_local > a->cursor ? b1 - d.n_local : a->cursor;
+    int n_pages = 0;
+    {
+        const int slot = L->page_cur;
+        L->page_cur = (slot + 1) % d.page_slots;
+        if (L->page_busy[slot]) HIP_OK(hipEventSynchronize(L->page_evt[slot]), "block_back: page slot");
+        infllm_page *base = d.h_pages + (int64_t)slot * d.B * d.max_pages;
+        for (int u = 0; u < d.B; ++u) {
+            infllm_page *pg = base + (int64_t)u * d.max_pages;     // packed to n_pages below
+            int n = 0;
+            auto push = [&](const bf16_t *k, const bf16_t *v, int64_t hs, int valid) {
+                if (n < d.max_pages) pg[n] = infllm_page{k, v, hs, valid, 0};
+                ++n;
+            };
+            for (int s = 0; s < a->n_sel; ++s) {
+                const int sl = a->h_sel_slots[u * a->n_sel + s];
+                INFLLM_REQUIRE(sl >= 0 && sl < d.max_cached, "block_back: slot %d out of range", sl);
+                const bf16_t *kb = (const bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + sl) * slot_elems;
+                for (int t0 = 0; t0 < bs; t0 += kTile)
+                    push(kb + (int64_t)t0 * kD, kb + unit_elems + (int64_t)t0 * kD, (int64_t)bs * kD, bs - t0 < kTile ? bs - t0 : kTile);
+            }
+            const bf16_t *ik = (const bf16_t *)d.d_init_kv + (int64_t)u * 2 * d.Hkv * d.init_cap * kD;
+            const bf16_t *iv = ik + (int64_t)d.Hkv * d.init_cap * kD;
+            for (int t0 = 0; t0 < a->init_len; t0 += kTile)
+                push(ik + (int64_t)t0 * kD, iv + (int64_t)t0 * kD, d.init_cap * kD, a->init_len - t0 < kTile ? a->init_len - t0 : kTile);
+            const bf16_t *rk = (const bf16_t *)d.d_ring_k_raw + (int64_t)u * d.Hkv * d.ring_cap * kD;
+            const bf16_t *rv = (const bf16_t *)d.d_ring_v + (int64_t)u * d.Hkv * d.ring_cap * kD;
+            for (int64_t pos = a->cursor; pos < overflow_end;) {
+                const int64_t row = pos % d.ring_cap;
+                int64_t len = overflow_end - pos;
+                if (len > kTile) len = kTile;
+                if (len > d.ring_cap - row) len = d.ring_cap - row;
+                push(rk + row * kD, rv + row * kD, d.ring_cap * kD, (int)len);
+                pos += len;
+            }
+            INFLLM_REQUIRE(n <= d.max_pages, "block_back: %d pages exceed the table (%d)", n, d.max_pages);
+            if (u == 0) n_pages = n;
+            INFLLM_REQUIRE(n == n_pages, "block_back: batch rows disagree on the page count");
+        }
+        if (n_pages > 0) {
+            // device layout is [B, n_pages]: pack the rows
+            for (int u = 1; u < d.B; ++u)
+                for (int i = 0; i < n_pages; ++i) base[(int64_t)u * n_pages + i] = base[(int64_t)u * d.max_pages + i];
+            HIP_OK(hipMemcpyAsync(d.d_pages, base, sizeof(infllm_page) * d.B * n_pages, hipMemcpyHostToDevice, st),
+                   "block_back: page upload");
+            HIP_OK(hipEventRecord(L->page_evt[slot], st), "block_back: event");
+            L->page_busy[slot] = 1;
+        }
+    }
+
+    // ---- 3. global stage, merge, local score
+    const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
+    const int sl = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
+    int parts = sl;
+    const int64_t part_o = (int64_t)d.B * d.H * a->n * kD, part_l = (int64_t)d.B * d.H * a->n;
+    int rc;
+    if (n_pages > 0) {
+        infllm_attn_args at{};
+        at.d_q = d.d_q_glb;
+        at.q_sl = kD; at.q_sh = (int64_t)a->n * kD; at.q_sb = (int64_t)d.H * a->n * kD;
+        at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = a->n;
+        at.cap = kTile;
+        at.d_pages = d.d_pages; at.n_pages = n_pages;
+        at.nsplit = splits_for(d, a->n, n_pages);
+        at.softmax_scale = d.softmax_scale;
+        at.d_o_part = d.d_o_part + sl * part_o;
+        at.d_lse_part = d.d_lse_part + sl * part_l;
+        const int ti = timer_begin(L, 1, a->n, n_pages * kTile, st);
+        rc = infllm_attn_stage(&at, stream);
+        timer_end(L, 1, ti, st);
+        if (rc) return rc;
+        if (side) {
+            HIP_OK(hipEventRecord(L->global_done, st), "block_back: event");
+            L->has_global = true;
+        }
+        parts += at.nsplit;
+    }
+    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, d.d_lse, stream);
+    if (rc) return rc;
+    infllm_score_args sc{};
+    sc.d_q = d.d_q_loc;
+    sc.q_sl = kD; sc.q_sh = (int64_t)a->n * kD; sc.q_sb = (int64_t)d.H * a->n * kD;
+    sc.B = d.B; sc.H = d.H; sc.Hkv = d.Hkv; sc.Lq = a->n;
+    sc.d_k = d.d_ring_k_rot;
+    sc.k_sl = kD; sc.k_sh = d.ring_cap * kD; sc.k_sb = (int64_t)d.Hkv * d.ring_cap * kD;
+    sc.cap = d.ring_cap; sc.j_lo = lo; sc.j_hi = b1;
+    sc.mask = INFLLM_MASK_WINDOW; sc.accumulate = 1; sc.offset = a->b0; sc.window = d.n_local;
+    sc.d_lse = d.d_lse; sc.softmax_scale = d.softmax_scale;
+    sc.d_score = d.d_ring_score; sc.score_sh = d.ring_cap; sc.score_sb = (int64_t)d.H * d.ring_cap; sc.score_cap = d.ring_cap;
+    rc = infllm_local_score(&sc, stream);
+    if (rc) return rc;
+
+    // ---- 4. state-machine actions: init peeling, new units
+    int64_t cursor = a->cursor;
+    if (a->init_take > 0) {
+        INFLLM_REQUIRE(a->init_len + a->init_take <= d.init_cap, "block_back: init overflow");
+        bf16_t *ik = (bf16_t *)d.d_init_kv + (int64_t)a->init_len * kD;
+        const int64_t sb = 2 * (int64_t)d.Hkv * d.init_cap * kD, sh = d.init_cap * kD;
+        rc = infllm_gather_rows(d.d_ring_k_raw, d.ring_cap, d.B, d.Hkv, cursor, a->init_take, a->init_take, ik, sb, 0, sh, stream);
+        if (rc) return rc;
+        rc = infllm_gather_rows(d.d_ring_v, d.ring_cap, d.B, d.Hkv, cursor, a->init_take, a->init_take,
+                                ik + (int64_t)d.Hkv * d.init_cap * kD, sb, 0, sh, stream);
+        if (rc) return rc;
+        cursor += a->init_take;
+    }
+    if (a->n_carve > 0) {
+        INFLLM_REQUIRE(a->d_rep_out && a->h_carve_dst, "block_back: null carve outputs");
+        rc = infllm_repr_keys(d.d_ring_score, d.d_ring_k_raw, d.ring_cap, d.B, d.H, d.Hkv, cursor, bs, a->n_carve, d.repr_topk,
+                              a->d_rep_out, a->rep_sb, a->rep_su, a->d_repr_idx, stream);
+        if (rc) return rc;
+        const int slot = L->carve_cur;
+        L->carve_cur = (slot + 1) % d.carve_slots;
+        if (L->carve_busy[slot]) HIP_OK(hipEventSynchronize(L->carve_evt[slot]), "block_back: carve slot");
+        const int64_t unit_all = (int64_t)d.B * slot_elems;                       // one unit, all batch rows
+        bf16_t *stage = (bf16_t *)d.d_carve_stage + (int64_t)slot * d.max_carve * unit_all;
+        rc = infllm_gather_rows(d.d_ring_k_raw, d.ring_cap, d.B, d.Hkv, cursor, a->n_carve * bs, bs, stage, slot_elems, unit_all,
+                                (int64_t)bs * kD, stream);
+        if (rc) return rc;
+        rc = infllm_gather_rows(d.d_ring_v, d.ring_cap, d.B, d.Hkv, cursor, a->n_carve * bs, bs, stage + unit_elems, slot_elems,
+                                unit_all, (int64_t)bs * kD, stream);
+        if (rc) return rc;
+        if (side) {
+            HIP_OK(hipEventRecord(L->carve_ready, st), "block_back: event");
+            HIP_OK(hipStreamWaitEvent(cs, L->carve_ready, 0), "block_back: wait carve");
+        }
+        for (int i = 0; i < a->n_carve; ++i) {
+            INFLLM_REQUIRE(a->h_carve_dst[i], "block_back: null carve destination");
+            HIP_OK(hipMemcpyAsync(a->h_carve_dst[i], stage + (int64_t)i * unit_all, unit_all * sizeof(bf16_t), hipMemcpyDeviceToHost, cs),
+                   "block_back: unit offload");
+        }
+        HIP_OK(hipEventRecord(L->carve_evt[slot], cs), "block_back: event");
+        L->carve_busy[slot] = 1;
+    }
+    return 0;
+}

@@ -16,8 +16,28 @@ MASK_NONE, MASK_WINDOW, MASK_COMPLEMENT = 0, 1, 2
 NO_WRAP = 1 << 40          # "cap" of a plain tensor source (a multiple of the key tile)
 
 
+_pinned_stream = None      # raw hipStream_t fixed by stream_scope(); None -> ask torch every call
+
+
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    return _pinned_stream if _pinned_stream is not None else torch.cuda.current_stream().cuda_stream
+
+
+class stream_scope:
+    """Pins the launch stream for a run of calls (torch.cuda.current_stream() costs several microseconds)."""
+
+    def __init__(self, raw_stream):
+        self.raw = raw_stream
+
+    def __enter__(self):
+        global _pinned_stream
+        self.prev, _pinned_stream = _pinned_stream, self.raw
+        return self
+
+    def __exit__(self, *exc):
+        global _pinned_stream
+        _pinned_stream = self.prev
+        return False
 
 
 def _need(cond, msg):
