@@ -65,8 +65,14 @@ typedef struct {
     float *d_ring_score;
     int64_t ring_cap;
     void *d_q_loc, *d_q_glb;
+    float *d_qpart;                /* optional fp32 [B, ceil(n/16), H*128]: sums of q_glb over each run of 16 positions */
 } infllm_ingest_args;
 int infllm_ingest(const infllm_ingest_args *a, void *stream);
+
+/* out[b,c] = scale * sum_p parts[b,p,c] (p ascending): turns the d_qpart sums of infllm_ingest into
+ * the mean global query of a block (context_manager.py:373-375) with scale = 1/n. */
+int infllm_reduce_partials(const float *d_parts, int32_t B, int32_t n_parts, int32_t C, float scale,
+                           float *d_out, void *stream);
 
 /* Mean of q_glb over each execution block (context_manager.py:373-375):
  * q_glb [B,H,n,128] contiguous -> d_qbar fp32 [B, n_blocks, H*128],
@@ -226,6 +232,7 @@ typedef struct {
     void *d_slab;                                     /* [B,max_cached,2,Hkv,block_size,128] */
     void *d_q_loc, *d_q_glb;                          /* [B*H*exc*128] each */
     float *d_qbar;                                    /* [B,H*128] */
+    float *d_qpart;                                   /* [B,ceil(exc/16),H*128] */
     float *d_o_part, *d_lse_part, *d_lse;             /* [2*max_splits,B,H,exc,(128)], [B,H,exc] */
     int32_t *d_topk_idx, *h_topk_idx;                 /* [B,topk] device / pinned host */
     infllm_page *d_pages;                             /* [B,max_pages] */

@@ -23,7 +23,7 @@ class IngestArgs(C.Structure):
         ("d_inv_freq", c_vp), ("distance_scale", c_f64),
         ("d_ring_k_raw", c_vp), ("d_ring_k_rot", c_vp), ("d_ring_v", c_vp),
         ("d_ring_score", c_vp), ("ring_cap", c_i64),
-        ("d_q_loc", c_vp), ("d_q_glb", c_vp),
+        ("d_q_loc", c_vp), ("d_q_glb", c_vp), ("d_qpart", c_vp),
     ]
 
 
@@ -68,7 +68,7 @@ class LayerDesc(C.Structure):
         ("ring_cap", c_i64),
         ("d_ring_k_raw", c_vp), ("d_ring_k_rot", c_vp), ("d_ring_v", c_vp), ("d_ring_score", c_vp),
         ("d_init_kv", c_vp), ("init_cap", c_i64), ("d_slab", c_vp),
-        ("d_q_loc", c_vp), ("d_q_glb", c_vp), ("d_qbar", c_vp),
+        ("d_q_loc", c_vp), ("d_q_glb", c_vp), ("d_qbar", c_vp), ("d_qpart", c_vp),
         ("d_o_part", c_vp), ("d_lse_part", c_vp), ("d_lse", c_vp),
         ("d_topk_idx", c_vp), ("h_topk_idx", c_vp),
         ("d_pages", c_vp), ("h_pages", c_vp), ("max_pages", c_i32), ("page_slots", c_i32),
@@ -107,6 +107,7 @@ SYMBOLS = {
     "infllm_version": (c_i32, []),
     "infllm_last_error": (C.c_char_p, []),
     "infllm_ingest": (c_i32, [C.POINTER(IngestArgs), c_vp]),
+    "infllm_reduce_partials": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_f32, c_vp, c_vp]),
     "infllm_block_mean": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "infllm_attn_stage": (c_i32, [C.POINTER(AttnArgs), c_vp]),
     "infllm_attn_merge": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),

@@ -177,6 +177,7 @@ class ContextManager:
         self.q_loc = torch.empty((B * H * exc * D,), **bf)
         self.q_glb = torch.empty((B * H * exc * D,), **bf)
         self.qbar = torch.empty((B, H * D), **f32)
+        self.qpart = torch.empty((B, (exc + 15) // 16, H * D), **f32)
         n_part = 2 * _MAX_SPLITS
         self.o_part = torch.empty((n_part * B * H * exc * D,), **f32)
         self.lse_part = torch.empty((n_part * B * H * exc,), **f32)
@@ -203,6 +204,7 @@ class ContextManager:
         d.d_ring_v, d.d_ring_score = self.ring_v.data_ptr(), self.ring_score.data_ptr()
         d.d_init_kv, d.init_cap, d.d_slab = self.init_kv.data_ptr(), self.init_kv.shape[3], self.slab.data_ptr()
         d.d_q_loc, d.d_q_glb, d.d_qbar = self.q_loc.data_ptr(), self.q_glb.data_ptr(), self.qbar.data_ptr()
+        d.d_qpart = self.qpart.data_ptr()
         d.d_o_part, d.d_lse_part, d.d_lse = self.o_part.data_ptr(), self.lse_part.data_ptr(), self.lse.data_ptr()
         d.d_topk_idx, d.h_topk_idx = self.topk_idx.data_ptr(), self.topk_idx_host.data_ptr()
         d.d_pages, d.h_pages = self.pages_dev.data_ptr(), self.pages_host.data_ptr()

@@ -27,11 +27,16 @@ __device__ __forceinline__ Rot8 rotate8(u32x4 xlo, u32x4 xhi, const float2 *cs) 
     return r;
 }
 
+// grid = (position tiles of 16, batch rows, kv heads): a workgroup rotates the query heads of one
+// kv-head group plus that group's key head, copies its value head, and leaves the sum of its
+// rotated-to-one-position queries over its positions in d_qpart (for the block's mean query).
 __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
     __shared__ float2 cs_pos[kPosPerBlock][kHalf];
     __shared__ float2 cs_glb[kHalf];
+    __shared__ float red[4][kPosPerBlock][kD];        // q_glb of 4 heads x 16 positions, for the partial sums
     const int tid = threadIdx.x;
-    const int b = blockIdx.y;
+    const int b = blockIdx.y, g = blockIdx.z;
+    const int G = a.H / a.Hkv;
     const int p0 = blockIdx.x * kPosPerBlock;
     const int np = min(kPosPerBlock, a.n - p0);
 
@@ -51,54 +56,86 @@ __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
     __syncthreads();
 
     const bf16_t *q = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb;
-    const bf16_t *k = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb;
-    const bf16_t *v = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb;
+    const bf16_t *k = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh;
+    const bf16_t *v = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh;
     bf16_t *q_loc = (bf16_t *)a.d_q_loc + (int64_t)b * a.H * a.n * kD;
     bf16_t *q_glb = (bf16_t *)a.d_q_glb + (int64_t)b * a.H * a.n * kD;
-    const int64_t ring_b = (int64_t)b * a.Hkv * a.ring_cap * kD;
-    bf16_t *rk_raw = (bf16_t *)a.d_ring_k_raw + ring_b;
-    bf16_t *rk_rot = (bf16_t *)a.d_ring_k_rot + ring_b;
-    bf16_t *rv = (bf16_t *)a.d_ring_v + ring_b;
+    const int64_t ring_g = ((int64_t)b * a.Hkv + g) * a.ring_cap * kD;
+    bf16_t *rk_raw = (bf16_t *)a.d_ring_k_raw + ring_g;
+    bf16_t *rk_rot = (bf16_t *)a.d_ring_k_rot + ring_g;
+    bf16_t *rv = (bf16_t *)a.d_ring_v + ring_g;
+    const int n_tiles = (a.n + kPosPerBlock - 1) / kPosPerBlock;
 
-    // query heads: 8 threads per (head, position) row
-    for (int e = tid; e < a.H * np * 8; e += 256) {
-        int c = e & 7, p = (e >> 3) % np, h = (e >> 3) / np;
-        const bf16_t *src = q + (int64_t)h * a.q_sh + (int64_t)(p0 + p) * a.q_sl;
-        u32x4 lo = *(const u32x4 *)(src + c * 8), hi = *(const u32x4 *)(src + kHalf + c * 8);
-        int64_t o = ((int64_t)h * a.n + p0 + p) * kD;
-        Rot8 r = rotate8(lo, hi, &cs_pos[p][c * 8]);
-        *(u32x4 *)(q_loc + o + c * 8) = r.lo;
-        *(u32x4 *)(q_loc + o + kHalf + c * 8) = r.hi;
-        r = rotate8(lo, hi, &cs_glb[c * 8]);
-        *(u32x4 *)(q_glb + o + c * 8) = r.lo;
-        *(u32x4 *)(q_glb + o + kHalf + c * 8) = r.hi;
+    // query heads of the group, 4 at a time: 8 threads per (head, position) row
+    for (int hg0 = 0; hg0 < G; hg0 += 4) {
+        const int nh = min(4, G - hg0);
+        for (int e = tid; e < nh * np * 8; e += 256) {
+            const int c = e & 7, p = (e >> 3) % np, hl = (e >> 3) / np;
+            const int h = g * G + hg0 + hl;
+            const bf16_t *src = q + (int64_t)h * a.q_sh + (int64_t)(p0 + p) * a.q_sl;
+            u32x4 lo = *(const u32x4 *)(src + c * 8), hi = *(const u32x4 *)(src + kHalf + c * 8);
+            int64_t o = ((int64_t)h * a.n + p0 + p) * kD;
+            Rot8 r = rotate8(lo, hi, &cs_pos[p][c * 8]);
+            *(u32x4 *)(q_loc + o + c * 8) = r.lo;
+            *(u32x4 *)(q_loc + o + kHalf + c * 8) = r.hi;
+            r = rotate8(lo, hi, &cs_glb[c * 8]);
+            *(u32x4 *)(q_glb + o + c * 8) = r.lo;
+            *(u32x4 *)(q_glb + o + kHalf + c * 8) = r.hi;
+            if (a.d_qpart) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    red[hl][p][c * 8 + 2 * w] = bf16_bits_to_f32(r.lo[w] & 0xffffu);
+                    red[hl][p][c * 8 + 2 * w + 1] = bf16_bits_to_f32(r.lo[w] >> 16);
+                    red[hl][p][kHalf + c * 8 + 2 * w] = bf16_bits_to_f32(r.hi[w] & 0xffffu);
+                    red[hl][p][kHalf + c * 8 + 2 * w + 1] = bf16_bits_to_f32(r.hi[w] >> 16);
+                }
+            }
+        }
+        if (a.d_qpart) {
+            __syncthreads();
+            for (int e = tid; e < nh * kD; e += 256) {
+                const int d = e % kD, hl = e / kD;
+                float s = 0.f;
+                for (int p = 0; p < np; ++p) s += red[hl][p][d];          // fixed order
+                a.d_qpart[(((int64_t)b * n_tiles + blockIdx.x) * a.H + g * G + hg0 + hl) * kD + d] = s;
+            }
+            __syncthreads();
+        }
     }
-    // key heads: raw copy + rotated copy into the rings
-    for (int e = tid; e < a.Hkv * np * 8; e += 256) {
-        int c = e & 7, p = (e >> 3) % np, h = (e >> 3) / np;
-        const bf16_t *src = k + (int64_t)h * a.k_sh + (int64_t)(p0 + p) * a.k_sl;
+    // key head: raw copy + rotated copy into the rings
+    for (int e = tid; e < np * 8; e += 256) {
+        const int c = e & 7, p = e >> 3;
+        const bf16_t *src = k + (int64_t)(p0 + p) * a.k_sl;
         u32x4 lo = *(const u32x4 *)(src + c * 8), hi = *(const u32x4 *)(src + kHalf + c * 8);
-        int64_t row = (a.pos0 + p0 + p) % a.ring_cap;
-        int64_t o = ((int64_t)h * a.ring_cap + row) * kD;
+        const int64_t o = ((a.pos0 + p0 + p) % a.ring_cap) * kD;
         *(u32x4 *)(rk_raw + o + c * 8) = lo;
         *(u32x4 *)(rk_raw + o + kHalf + c * 8) = hi;
         Rot8 r = rotate8(lo, hi, &cs_pos[p][c * 8]);
         *(u32x4 *)(rk_rot + o + c * 8) = r.lo;
         *(u32x4 *)(rk_rot + o + kHalf + c * 8) = r.hi;
     }
-    // values: plain copy, 16 threads per row
-    for (int e = tid; e < a.Hkv * np * 16; e += 256) {
-        int c = e & 15, p = (e >> 4) % np, h = (e >> 4) / np;
-        const bf16_t *src = v + (int64_t)h * a.v_sh + (int64_t)(p0 + p) * a.v_sl;
-        int64_t row = (a.pos0 + p0 + p) % a.ring_cap;
-        *(u32x4 *)(rv + ((int64_t)h * a.ring_cap + row) * kD + c * 8) = *(const u32x4 *)(src + c * 8);
+    // value head: plain copy, 16 threads per row
+    for (int e = tid; e < np * 16; e += 256) {
+        const int c = e & 15, p = e >> 4;
+        const bf16_t *src = v + (int64_t)(p0 + p) * a.v_sl;
+        *(u32x4 *)(rv + ((a.pos0 + p0 + p) % a.ring_cap) * kD + c * 8) = *(const u32x4 *)(src + c * 8);
     }
     // the score track of a new token starts at zero (context_manager.py:733-741)
-    for (int e = tid; e < a.H * np; e += 256) {
-        int p = e % np, h = e / np;
-        int64_t row = (a.pos0 + p0 + p) % a.ring_cap;
-        a.d_ring_score[((int64_t)b * a.H + h) * a.ring_cap + row] = 0.f;
+    for (int e = tid; e < G * np; e += 256) {
+        const int p = e % np, h = g * G + e / np;
+        a.d_ring_score[((int64_t)b * a.H + h) * a.ring_cap + (a.pos0 + p0 + p) % a.ring_cap] = 0.f;
     }
+}
+
+// out[b, c] = scale * sum_p parts[b, p, c], p ascending
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float *parts, int n_parts, int C, float scale,
+                                                              float *out) {
+    const int c = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+    if (c >= C) return;
+    const float *src = parts + (int64_t)b * n_parts * C + c;
+    float s = 0.f;
+    for (int p = 0; p < n_parts; ++p) s += src[(int64_t)p * C];
+    out[(int64_t)b * C + c] = s * scale;
 }
 
 constexpr int kMeanThreads = 512;
@@ -161,9 +198,19 @@ extern "C" int infllm_ingest(const infllm_ingest_args *a, void *stream) {
                     a->v_sh % 8 | a->v_sb % 8) == 0,
                    "ingest: strides must be multiples of 8 elements (16-byte rows)");
     if (a->n == 0) return 0;
-    dim3 grid((a->n + kPosPerBlock - 1) / kPosPerBlock, a->B);
+    dim3 grid((a->n + kPosPerBlock - 1) / kPosPerBlock, a->B, a->Hkv);
     hipLaunchKernelGGL(ingest_kernel, grid, dim3(256), 0, (hipStream_t)stream, *a);
     INFLLM_CHECK_LAUNCH("ingest");
+    return 0;
+}
+
+extern "C" int infllm_reduce_partials(const float *d_parts, int32_t B, int32_t n_parts, int32_t C, float scale, float *d_out,
+                                      void *stream) {
+    INFLLM_REQUIRE(d_parts && d_out, "reduce_partials: null pointer");
+    INFLLM_REQUIRE(B > 0 && n_parts > 0 && C > 0, "reduce_partials: bad sizes B=%d n_parts=%d C=%d", B, n_parts, C);
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((C + 255) / 256, B), dim3(256), 0, (hipStream_t)stream, d_parts, n_parts, C,
+                       scale, d_out);
+    INFLLM_CHECK_LAUNCH("reduce_partials");
     return 0;
 }
 

@@ -89,14 +89,15 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
             if ((key & pmask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1);
         }
         __syncthreads();
-        if (tid == 0) {
-            int remaining = need, d = 255;
-            for (; d > 0; --d) {
-                if (hist[d] >= remaining) break;
-                remaining -= hist[d];
+        {
+            // digit of the need-th largest key: scan the buckets from the top (thread t <-> digit 255 - t)
+            const int v = tid < 256 ? hist[255 - tid] : 0;
+            int tot;
+            const int excl = block_exclusive_scan(v, wave_tot, &tot);
+            if (tid < 256 && excl < need && excl + v >= need) {
+                sh_prefix = prefix | ((uint32_t)(255 - tid) << shift);
+                sh_need = need - excl;
             }
-            sh_prefix = prefix | ((uint32_t)d << shift);
-            sh_need = remaining;
         }
         __syncthreads();
         prefix = sh_prefix;

@@ -5,112 +5,159 @@
 //
 // It needs the final log-sum-exp of every query, so it runs after the merge and
 // recomputes Q.K^T.  Orientation: S[query, key] with keys in the MFMA column, so a lane
-// owns one key and the column sum is a running per-lane scalar.  A workgroup owns 64
-// keys of one kv head; its waves take the query heads of the group (two waves per head,
-// one 32-key half each, when the group has fewer than 4 heads); K stays in registers
-// and query tiles stream from L2.  Exactly one lane writes each (head, key) cell, so
-// results are deterministic.
+// owns one key and the column sum is a running per-lane scalar.  A workgroup owns 256
+// consecutive keys of one query head: each of its 4 waves keeps 64 keys in registers
+// (B operand) for the whole kernel, while tiles of 64 queries stream through LDS
+// (A operand, shared by the 4 waves, double buffered).  Exactly one lane writes each
+// (head, key) cell, so results are deterministic.
 #include "common.h"
 
 namespace {
 
-constexpr int kQT = 32;
+constexpr int kQStage = 64;                // queries per LDS stage
+constexpr int kQPad = kD + 8;              // LDS row of Q (bf16 elements): 272 bytes rotates the banks
+constexpr int kKeysPerWg = 4 * kTile;
 
 __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a) {
+    __shared__ __attribute__((aligned(16))) bf16_t Qs[2][kQStage][kQPad];
+    __shared__ __attribute__((aligned(16))) float Ls[2][kQStage];
+
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
     const int G = a.H / a.Hkv;
-    const int b = blockIdx.y / a.Hkv, g = blockIdx.y % a.Hkv;
-    const int64_t j0 = ((a.j_lo >> 6) + blockIdx.x) * (int64_t)kTile;       // first key of this tile
-
-    const int halves = G >= 4 ? 1 : 2;          // waves per head
-    const int head_step = 4 / halves;
-    const int ks_lo = halves == 1 ? 0 : (wave & 1), ks_hi = halves == 1 ? 2 : (wave & 1) + 1;
+    const int b = blockIdx.y / a.H, h = blockIdx.y % a.H, g = h / G;
+    const int64_t jg = ((a.j_lo >> 6) + (int64_t)blockIdx.x * 4) * kTile;   // first key of the workgroup
+    const int64_t j0 = jg + (int64_t)wave * kTile;                          // first key of this wave
     const float scale = a.softmax_scale * 1.4426950408889634f;
 
-    // queries that can see any key of the tile
-    int64_t i_lo = 0, i_hi = a.Lq;               // [i_lo, i_hi)
-    const int64_t jf = max(j0, a.j_lo), jl = min(j0 + kTile, a.j_hi) - 1;
-    if (a.mask == INFLLM_MASK_WINDOW) {
-        i_lo = max(i_lo, jf - a.offset);
-        i_hi = min(i_hi, jl - a.offset + a.window);
-    } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
-        i_lo = max(i_lo, jf - a.offset + a.window);
+    // ---- this wave's 64 keys as the B operand (lane = key column)
+    bf16x8 kreg[2][kD / 16];
+    bool jok[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const int64_t j = j0 + ks * 32 + col;
+        jok[ks] = j >= a.j_lo && j < a.j_hi;
+        const bf16_t *krow = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh + (j % a.cap) * a.k_sl;
+#pragma unroll
+        for (int kk = 0; kk < kD / 16; ++kk) {
+            u32x4 raw = jok[ks] ? *(const u32x4 *)(krow + kk * 16 + grp * 8) : u32x4{0, 0, 0, 0};
+            kreg[ks][kk] = __builtin_bit_cast(bf16x8, raw);
+        }
     }
-    const int qt_lo = (int)(i_lo / kQT), qt_hi = i_hi > i_lo ? (int)((i_hi - 1) / kQT) + 1 : qt_lo;
 
-    for (int hg = wave / halves; hg < G; hg += head_step) {
-        const int h = g * G + hg;
-        // ---- keys of this wave in registers (B operand: lane = key column)
-        bf16x8 kreg[2][kD / 16];
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            const int64_t j = j0 + ks * 32 + col;
-            const bool ok = ks >= ks_lo && ks < ks_hi && j >= a.j_lo && j < a.j_hi;
-            const bf16_t *krow = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh + (j % a.cap) * a.k_sl;
-#pragma unroll
-            for (int kk = 0; kk < kD / 16; ++kk) {
-                u32x4 raw = ok ? *(const u32x4 *)(krow + kk * 16 + grp * 8) : u32x4{0, 0, 0, 0};
-                kreg[ks][kk] = __builtin_bit_cast(bf16x8, raw);
-            }
+    // ---- query range: what the workgroup stages, and what this wave needs of it
+    auto query_range = [&](int64_t jf, int64_t jl, int64_t &lo, int64_t &hi) {   // keys [jf, jl] -> queries [lo, hi)
+        lo = 0;
+        hi = a.Lq;
+        jf = max(jf, a.j_lo);
+        jl = min(jl, a.j_hi - 1);
+        if (jl < jf) {
+            hi = 0;
+            return;
         }
-        float colsum[2] = {0.f, 0.f};
-        const bf16_t *qbase = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
-        const float *lse = a.d_lse + ((int64_t)b * a.H + h) * a.Lq;
+        if (a.mask == INFLLM_MASK_WINDOW) {
+            lo = max(lo, jf - a.offset);
+            hi = min(hi, jl - a.offset + a.window);
+        } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
+            lo = max(lo, jf - a.offset + a.window);
+        }
+    };
+    int64_t g_lo, g_hi, w_lo, w_hi;
+    query_range(jg, jg + kKeysPerWg - 1, g_lo, g_hi);
+    query_range(j0, j0 + kTile - 1, w_lo, w_hi);
+    const int st_lo = (int)(g_lo / kQStage), st_hi = g_hi > g_lo ? (int)((g_hi - 1) / kQStage) + 1 : st_lo;
 
-        for (int qt = qt_lo; qt < qt_hi; ++qt) {
-            const int i0 = qt * kQT;
-            bf16x8 qa[kD / 16];                  // A operand: lane = query row
-            {
-                const int qi = i0 + col;
-                const bool ok = qi < a.Lq;
-                const bf16_t *qrow = qbase + (int64_t)qi * a.q_sl;
+    const bf16_t *qbase = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+    const float *lse = a.d_lse + ((int64_t)b * a.H + h) * a.Lq;
+    const int ld_chunk = tid & 15, ld_row = tid >> 4;
+    u32x4 qbuf[4];
+    float lbuf = 0.f;
+    auto load_stage = [&](int s) {
+        const int i0 = s * kQStage;
 #pragma unroll
-                for (int kk = 0; kk < kD / 16; ++kk) {
-                    u32x4 raw = ok ? *(const u32x4 *)(qrow + kk * 16 + grp * 8) : u32x4{0, 0, 0, 0};
-                    qa[kk] = __builtin_bit_cast(bf16x8, raw);
+        for (int i = 0; i < 4; ++i) {
+            const int qi = i0 + ld_row + 16 * i;
+            qbuf[i] = qi < a.Lq ? *(const u32x4 *)(qbase + (int64_t)qi * a.q_sl + ld_chunk * 8) : u32x4{0, 0, 0, 0};
+        }
+        if (tid < kQStage) lbuf = i0 + tid < a.Lq ? lse[i0 + tid] : INFINITY;      // +inf => probability 0
+    };
+    auto store_stage = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(u32x4 *)&Qs[buf][ld_row + 16 * i][ld_chunk * 8] = qbuf[i];
+        if (tid < kQStage) Ls[buf][tid] = lbuf;
+    };
+
+    float colsum[2] = {0.f, 0.f};
+    if (st_hi > st_lo) {
+        load_stage(st_lo);
+        store_stage(0);
+        if (st_lo + 1 < st_hi) load_stage(st_lo + 1);
+    }
+    __syncthreads();
+    for (int s = st_lo; s < st_hi; ++s) {
+        const int cur = (s - st_lo) & 1;
+        const int64_t i0 = (int64_t)s * kQStage;
+        if (i0 < w_hi && i0 + kQStage > w_lo) {                  // wave-uniform
+#pragma unroll
+            for (int qs = 0; qs < 2; ++qs) {
+                const int64_t iq = i0 + qs * 32;
+                if (iq >= w_hi || iq + 32 <= w_lo) continue;
+                bf16x8 qa[kD / 16];                              // A operand: lane = query row
+                const bf16_t *qrow = &Qs[cur][qs * 32 + col][grp * 8];
+#pragma unroll
+                for (int kk = 0; kk < kD / 16; ++kk) qa[kk] = *(const bf16x8 *)(qrow + kk * 16);
+                f32x4 l4[4];                                     // lse of rows 8*(r>>2) + 4*grp + (r&3)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) l4[q4] = *(const f32x4 *)&Ls[cur][qs * 32 + 8 * q4 + 4 * grp];
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    f32x16 sacc;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+                    for (int kk = 0; kk < kD / 16; ++kk)
+                        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[kk], kreg[ks][kk], sacc, 0, 0, 0);
+                    // dist(i, j) = i - j + offset for the first query row and this lane's key
+                    const int64_t jk = j0 + ks * 32;
+                    const int64_t e0 = iq - jk + a.offset;       // query iq, key jk
+                    bool need_mask = false;
+                    if (a.mask == INFLLM_MASK_WINDOW) need_mask = (e0 - 31 < 0) || (e0 + 31 >= a.window);
+                    if (a.mask == INFLLM_MASK_COMPLEMENT) need_mask = (e0 - 31 < a.window);
+                    float acc = 0.f;
+                    if (!need_mask) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            acc += __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], scale, -l4[r >> 2][r & 3]));
+                    } else {
+                        const int d0 = (int)min(max(e0, (int64_t)-(1 << 29)), (int64_t)(1 << 29)) - col;
+                        const int win = (int)min(a.window, (int64_t)(1 << 30));
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int dist = d0 + 8 * (r >> 2) + 4 * grp + (r & 3);
+                            bool vis = true;
+                            if (a.mask == INFLLM_MASK_WINDOW) vis = dist >= 0 && dist < win;
+                            if (a.mask == INFLLM_MASK_COMPLEMENT) vis = dist >= win;
+                            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], scale, -l4[r >> 2][r & 3]));
+                            acc += vis ? p : 0.f;
+                        }
+                    }
+                    colsum[ks] += acc;
                 }
             }
-            float lrow[16];                      // lse of the 16 query rows this lane sees
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int qi = i0 + 8 * (r >> 2) + 4 * grp + (r & 3);
-                lrow[r] = qi < a.Lq ? lse[qi] : INFINITY;          // +inf => probability 0
-            }
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                if (ks < ks_lo || ks >= ks_hi) continue;
-                f32x16 s;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[r] = 0.f;
-#pragma unroll
-                for (int kk = 0; kk < kD / 16; ++kk)
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[kk], kreg[ks][kk], s, 0, 0, 0);
-                const int64_t j = j0 + ks * 32 + col;
-                const bool jok = j >= a.j_lo && j < a.j_hi;
-                float acc = 0.f;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int64_t qi = i0 + 8 * (r >> 2) + 4 * grp + (r & 3);
-                    const int64_t dist = qi - j + a.offset;
-                    bool vis = jok;
-                    if (a.mask == INFLLM_MASK_WINDOW) vis = vis && dist >= 0 && dist < a.window;
-                    if (a.mask == INFLLM_MASK_COMPLEMENT) vis = vis && dist >= a.window;
-                    float p = __builtin_amdgcn_exp2f(s[r] * scale - lrow[r]);
-                    acc += vis ? p : 0.f;
-                }
-                colsum[ks] += acc;
-            }
         }
+        if (s + 1 < st_hi) {
+            store_stage(cur ^ 1);
+            if (s + 2 < st_hi) load_stage(s + 2);
+        }
+        __syncthreads();
+    }
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            if (ks < ks_lo || ks >= ks_hi) continue;
-            const float tot = colsum[ks] + wave_xor32(colsum[ks]);
-            const int64_t j = j0 + ks * 32 + col;
-            if (grp == 0 && j >= a.j_lo && j < a.j_hi) {
-                float *dst = a.d_score + (int64_t)b * a.score_sb + (int64_t)h * a.score_sh + (j % a.score_cap);
-                *dst = a.accumulate ? *dst + tot : tot;
-            }
+    for (int ks = 0; ks < 2; ++ks) {
+        const float tot = colsum[ks] + wave_xor32(colsum[ks]);
+        const int64_t j = j0 + ks * 32 + col;
+        if (grp == 0 && jok[ks]) {
+            float *dst = a.d_score + (int64_t)b * a.score_sb + (int64_t)h * a.score_sh + (j % a.score_cap);
+            *dst = a.accumulate ? *dst + tot : tot;
         }
     }
 }
@@ -130,7 +177,7 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
                    "local_score: strides must be multiples of 8");
     if (a->j_hi <= a->j_lo) return 0;
     const int64_t tiles = ((a->j_hi - 1) >> 6) - (a->j_lo >> 6) + 1;
-    hipLaunchKernelGGL(local_score_kernel, dim3((unsigned)tiles, a->B * a->Hkv), dim3(256), 0, (hipStream_t)stream, *a);
+    hipLaunchKernelGGL(local_score_kernel, dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
     INFLLM_CHECK_LAUNCH("local_score");
     return 0;
 }

@@ -72,7 +72,7 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
     if (d.exc <= 0 || d.exc > d.n_local || d.block_size <= 0 || d.topk < 0 || d.topk > d.max_cached) return bad("bad knobs");
     if (d.ring_cap % kTile || d.ring_cap < (int64_t)d.n_local + d.exc + d.block_size) return bad("ring too small or unaligned");
     if (!d.d_ring_k_raw || !d.d_ring_k_rot || !d.d_ring_v || !d.d_ring_score || !d.d_init_kv || !d.d_slab || !d.d_q_loc ||
-        !d.d_q_glb || !d.d_qbar || !d.d_o_part || !d.d_lse_part || !d.d_lse || !d.d_topk_idx || !d.h_topk_idx || !d.d_pages ||
+        !d.d_q_glb || !d.d_qbar || !d.d_qpart || !d.d_o_part || !d.d_lse_part || !d.d_lse || !d.d_topk_idx || !d.h_topk_idx || !d.d_pages ||
         !d.h_pages || !d.d_carve_stage || !d.d_inv_freq)
         return bad("null buffer");
     if (d.max_splits < 1 || d.max_splits > 64 || d.num_cus < 1 || d.page_slots < 1 || d.carve_slots < 1 || d.max_carve < 1 ||
@@ -163,13 +163,14 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     in.d_ring_k_raw = d.d_ring_k_raw; in.d_ring_k_rot = d.d_ring_k_rot; in.d_ring_v = d.d_ring_v;
     in.d_ring_score = d.d_ring_score; in.ring_cap = d.ring_cap;
     in.d_q_loc = d.d_q_loc; in.d_q_glb = d.d_q_glb;
+    in.d_qpart = a->n_units > d.topk ? d.d_qpart : nullptr;
     int rc = infllm_ingest(&in, stream);
     if (rc) return rc;
 
     L->topk_pending = false;
     if (a->n_units > d.topk) {
         INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
-        rc = infllm_block_mean(d.d_q_glb, d.B, d.H, a->n, a->n, d.d_qbar, stream);
+        rc = infllm_reduce_partials(d.d_qpart, d.B, (a->n + 15) / 16, d.H * kD, 1.f / (float)a->n, d.d_qbar, stream);
         if (rc) return rc;
         const int C = d.H * kD;
         for (int u = 0; u < d.B; ++u) {

@@ -54,7 +54,8 @@ def _bf16_4d(t, name):
     return t
 
 
-def ingest(q, k, v, pos0, glb_pos, inv_freq, distance_scale, ring_k_raw, ring_k_rot, ring_v, ring_score, q_loc, q_glb):
+def ingest(q, k, v, pos0, glb_pos, inv_freq, distance_scale, ring_k_raw, ring_k_rot, ring_v, ring_score, q_loc, q_glb,
+           qpart=None):
     """RoPE + staging of the new tokens; see infllm_ingest."""
     q, k, v = _bf16_4d(q, "q"), _bf16_4d(k, "k"), _bf16_4d(v, "v")
     B, H, n, _ = q.shape
@@ -72,8 +73,15 @@ def ingest(q, k, v, pos0, glb_pos, inv_freq, distance_scale, ring_k_raw, ring_k_
                    v.stride(0), v.stride(1), v.stride(2), B, H, Hkv, n, pos0, glb_pos,
                    inv_freq.data_ptr(), float(distance_scale),
                    ring_k_raw.data_ptr(), ring_k_rot.data_ptr(), ring_v.data_ptr(), ring_score.data_ptr(), cap,
-                   q_loc.data_ptr(), q_glb.data_ptr())
+                   q_loc.data_ptr(), q_glb.data_ptr(), qpart.data_ptr() if qpart is not None else None)
     check(_lib.load().infllm_ingest(a, _stream()), "infllm_ingest")
+
+
+def reduce_partials(parts, scale, out):
+    """out[b, c] = scale * sum_p parts[b, p, c]."""
+    B, n_parts, C = parts.shape
+    check(_lib.load().infllm_reduce_partials(parts.data_ptr(), B, n_parts, C, float(scale), out.data_ptr(), _stream()),
+          "infllm_reduce_partials")
 
 
 def block_mean(q_glb, B, H, n, exc, qbar):

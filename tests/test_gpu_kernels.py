@@ -75,6 +75,24 @@ def test_ingest_matches_rope_oracle(pos0, n):
         assert float((q_loc.cpu().float() - want).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
 
 
+def test_ingest_partial_sums_give_the_mean_global_query():
+    ops = _ops()
+    B, H, Hkv, n, cap = 2, 8, 2, 77, 128
+    q, k, v = _rand((B, H, n, D), 5), _rand((B, Hkv, n, D), 6), _rand((B, Hkv, n, D), 7)
+    rope = RopeOracle(D, base=1e4)
+    z = lambda *s: torch.zeros(s, dtype=torch.bfloat16, device="cuda")
+    rk_raw, rk_rot, rv = z(B, Hkv, cap, D), z(B, Hkv, cap, D), z(B, Hkv, cap, D)
+    rscore = torch.zeros((B, H, cap), dtype=torch.float32, device="cuda")
+    q_loc, q_glb = z(B, H, n, D), z(B, H, n, D)
+    qpart = torch.full((B, (n + 15) // 16, H * D), 9.0, dtype=torch.float32, device="cuda")
+    ops.ingest(q.cuda(), k.cuda(), v.cuda(), 3, 63, rope.inv_freq.cuda(), 1.0, rk_raw, rk_rot, rv, rscore, q_loc, q_glb, qpart)
+    qbar = torch.zeros((B, H * D), dtype=torch.float32, device="cuda")
+    ops.reduce_partials(qpart, 1.0 / n, qbar)
+    want = q_glb.float().mean(dim=2).reshape(B, H * D)
+    assert torch.allclose(qbar, want, atol=1e-5)
+    assert torch.allclose(want.cpu(), rope.one_angle(q.float(), 64).mean(dim=2).reshape(B, H * D), atol=1e-2)
+
+
 def test_block_mean():
     ops = _ops()
     B, H, n, exc = 2, 3, 70, 32

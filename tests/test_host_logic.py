@@ -41,7 +41,7 @@ def test_struct_layouts_match_header_sizes():
     # sizes follow from the field lists in include/infllm_hip.h under natural alignment
     import ctypes
     assert ctypes.sizeof(_lib.Page) == 32
-    assert ctypes.sizeof(_lib.IngestArgs) == 3 * 8 + 9 * 8 + 4 * 4 + 2 * 8 + 8 + 8 + 4 * 8 + 8 + 2 * 8
+    assert ctypes.sizeof(_lib.IngestArgs) == 3 * 8 + 9 * 8 + 4 * 4 + 2 * 8 + 8 + 8 + 4 * 8 + 8 + 3 * 8
     assert ctypes.sizeof(_lib.AttnArgs) == 8 + 24 + 16 + 16 + 48 + 24 + 8 + 16 + 8 + 8 + 8 + 16
     assert ctypes.sizeof(_lib.ScoreArgs) == 8 + 24 + 16 + 8 + 24 + 24 + 8 + 16 + 8 + 8 + 8 + 24
 
