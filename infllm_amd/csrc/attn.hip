@@ -24,7 +24,8 @@ constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kQTile = 32;                 // queries per wave
 constexpr int kBig = 1 << 29;              // clamp for mask distances held in int32
-constexpr int kKPad = kD + 8;              // LDS row of K  (bf16 elements)
+constexpr int kKPad = kD + 8;              // LDS row of K (bf16 elements)
+constexpr int kVPad = kD + 16;             // LDS row of V (bf16 elements)
 
 struct StageRange {
     int64_t lo, hi;   // key index range [lo, hi) visible to a span of queries
@@ -47,15 +48,22 @@ __device__ __forceinline__ int floordiv64(int64_t x) { return (int)(x >> 6); }  
 // LDS layouts (both free of bank conflicts for the 16-byte MFMA operand reads):
 //   Ks[buf][row][kKPad]  row = key with bits 2 and 3 swapped inside each 32-key half, so that the
 //                        lane holding MFMA row r reads LDS row r; 272-byte rows rotate the banks.
-//   Vt[buf][d][64 keys]  128-byte rows cut into eight 16-byte units of 8 keys; unit u of row d is
-//                        stored at unit u ^ (d & 7) ^ ((d >> 3) & 7).
+//   Vs[buf][key][kVPad]  natural rows; the V^T operand of the second MFMA is formed by the transposing
+//                        LDS read ds_read_b64_tr_b16: in a group of 16 lanes, lane 4*j + q supplies the
+//                        address of 4 consecutive d of key j, and lane i receives element i of key
+//                        j = 0..3, i.e. 4 consecutive keys at one d.  288-byte rows keep the 4 rows of a
+//                        read on disjoint banks.
 __device__ __forceinline__ int k_lds_row(int key) { return (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1); }
-__device__ __forceinline__ int vt_unit(int d, int u) { return u ^ (d & 7) ^ ((d >> 3) & 7); }
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ s16x4 lds_read_tr(const bf16_t *p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
+}
 
 template <bool PAGED>
 __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a) {
     __shared__ __attribute__((aligned(16))) bf16_t Ks[2][kTile][kKPad];
-    __shared__ __attribute__((aligned(16))) bf16_t Vt[2][kD][kTile];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[2][kTile][kVPad];
     __shared__ int wg_lo[kWaves], wg_hi[kWaves];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -119,7 +127,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     // ---- cooperative tile loads: thread -> (rows, 16-byte chunk)
     const int ld_chunk = tid & 15;            // 8 head_dim elements
     const int ld_row = tid >> 4;              // 0..15
-    u32x4 kbuf[4], vbuf[4];                   // K rows ld_row + 16*i ; V rows 4*ld_row + i
+    u32x4 kbuf[4], vbuf[4];                   // K and V rows ld_row + 16*i
 
     auto load_tile = [&](int t) {
         const bf16_t *kbase, *vbase;
@@ -147,27 +155,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             int r = ld_row + 16 * i;
             kbuf[i] = (r >= row_lo && r < row_hi) ? *(const u32x4 *)(kbase + (int64_t)r * k_sl + ld_chunk * 8)
                                                  : u32x4{0, 0, 0, 0};
-            int rv = 4 * ld_row + i;
-            vbuf[i] = (rv >= row_lo && rv < row_hi) ? *(const u32x4 *)(vbase + (int64_t)rv * v_sl + ld_chunk * 8)
-                                                   : u32x4{0, 0, 0, 0};
+            vbuf[i] = (r >= row_lo && r < row_hi) ? *(const u32x4 *)(vbase + (int64_t)r * v_sl + ld_chunk * 8)
+                                                 : u32x4{0, 0, 0, 0};
         }
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) *(u32x4 *)&Ks[buf][k_lds_row(ld_row + 16 * i)][ld_chunk * 8] = kbuf[i];
-        // 4 keys x 8 dims -> 8 dims x 4 keys (8 bytes each)
-        const int unit = ld_row >> 1, half = (ld_row & 1) * 4;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            u32x2 even, odd;                  // dims 2w and 2w+1 of keys 0..3
-            even[0] = (vbuf[0][w] & 0xffffu) | (vbuf[1][w] << 16);
-            even[1] = (vbuf[2][w] & 0xffffu) | (vbuf[3][w] << 16);
-            odd[0] = (vbuf[0][w] >> 16) | (vbuf[1][w] & 0xffff0000u);
-            odd[1] = (vbuf[2][w] >> 16) | (vbuf[3][w] & 0xffff0000u);
-            const int d0 = ld_chunk * 8 + 2 * w;
-            *(u32x2 *)&Vt[buf][d0][vt_unit(d0, unit) * 8 + half] = even;
-            *(u32x2 *)&Vt[buf][d0 + 1][vt_unit(d0 + 1, unit) * 8 + half] = odd;
-        }
+        for (int i = 0; i < 4; ++i) *(u32x4 *)&Vs[buf][ld_row + 16 * i][ld_chunk * 8] = vbuf[i];
     };
 
     // ---- running softmax state of this lane's query (max kept in raw logit units)
@@ -194,12 +190,19 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[ks][r] = 0.f;
-                const bf16_t *krow = &Ks[cur][ks * 32 + col][grp * 8];
+            }
+            {
+                bf16x8 ka[2][kD / 16];             // all 16 K operands are requested before the first MFMA
 #pragma unroll
-                for (int kk = 0; kk < kD / 16; ++kk) {
-                    bf16x8 ka = *(const bf16x8 *)(krow + kk * 16);
-                    s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[kk], s[ks], 0, 0, 0);
-                }
+                for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                    for (int kk = 0; kk < kD / 16; ++kk)
+                        ka[ks][kk] = *(const bf16x8 *)&Ks[cur][ks * 32 + col][grp * 8 + kk * 16];
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                    for (int kk = 0; kk < kD / 16; ++kk)
+                        s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kk], qreg[kk], s[ks], 0, 0, 0);
             }
             // ---- mask (only tiles that touch a boundary); distances are clamped into int32
             bool need_mask;
@@ -266,20 +269,32 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
 #pragma unroll
                     for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
             }
+            {
+                // V^T operands: lane -> (4 keys j, 4 d) address pattern of the transposing read
+                const int lam = lane & 15, g16 = lane >> 4;
+                const bf16_t *vrow = &Vs[cur][8 * (g16 >> 1) + (lam >> 2)][16 * (g16 & 1) + 4 * (lam & 3)];
+                s16x4 va[4][kD / 32][2];           // [ks*2+mm][dt][key half]
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int mm = 0; mm < 2; ++mm) {
-                    u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
-                    bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
-                    const int u = ks * 4 + mm * 2 + grp;
+                for (int gi = 0; gi < 4; ++gi)
 #pragma unroll
                     for (int dt = 0; dt < kD / 32; ++dt) {
-                        const int d = dt * 32 + col;
-                        bf16x8 va = *(const bf16x8 *)&Vt[cur][d][vt_unit(d, u) * 8];
-                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb, oacc[dt], 0, 0, 0);
+                        const bf16_t *p0 = vrow + (gi * 16) * kVPad + dt * 32;
+                        va[gi][dt][0] = lds_read_tr(p0);
+                        va[gi][dt][1] = lds_read_tr(p0 + 4 * kVPad);
+                    }
+#pragma unroll
+                for (int gi = 0; gi < 4; ++gi) {
+                    const int ks = gi >> 1, mm = gi & 1;
+                    u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
+                    bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+#pragma unroll
+                    for (int dt = 0; dt < kD / 32; ++dt) {
+                        typedef short s16x8 __attribute__((ext_vector_type(8)));
+                        s16x8 v8 = __builtin_shufflevector(va[gi][dt][0], va[gi][dt][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, v8), pb, oacc[dt], 0, 0, 0);
                     }
                 }
+            }
         }
         if (t + 1 < g_t1) {
             store_tile(cur ^ 1);                // the other buffer was last read one barrier ago
