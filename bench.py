@@ -81,7 +81,10 @@ def main():
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--chunk", type=int, default=8192, help="tokens per append() call")
     ap.add_argument("--cpu-tokens", type=int, default=16384, help="0 disables the CPU baseline")
+    ap.add_argument("--max-cached-block", type=int, default=KNOBS["max_cached_block"],
+                    help="GPU unit-cache slots (the headline number uses the reference's 32)")
     args = ap.parse_args()
+    KNOBS["max_cached_block"] = args.max_cached_block
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the path has no cross-GPU step); use --gpus 1")
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -117,7 +120,7 @@ def main():
         "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"config 2: one InfLLM layer, {T}-token stream, exc 512, H32/Hkv8/D128, "
-                               "n_init128 n_local4096 bs128 topk16 repr_topk4 max_cached32 lru, GMM keys",
+                               f"n_init128 n_local4096 bs128 topk16 repr_topk4 max_cached{KNOBS['max_cached_block']} lru, GMM keys",
                    "append_chunk": args.chunk},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,

@@ -172,6 +172,12 @@ int infllm_local_score(const infllm_score_args *a, void *stream);
 int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C,
                       const float *d_qbar, int32_t k,
                       float *d_scores, int32_t *d_idx, void *stream);
+/* The two halves of infllm_score_topk: scores of rows [first, first+count) into d_scores[first..], and the
+ * selection over d_scores[0..N).  Scoring the units that exist early and only the newly carved ones late keeps
+ * the retrieval of the next block short. */
+int infllm_unit_scores(const void *d_reps, int64_t rep_stride, int32_t first, int32_t count, int32_t C,
+                       const float *d_qbar, float *d_scores, void *stream);
+int infllm_topk(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, void *stream);
 
 /* Representative key of carved units.
  * Replaces get_block_k + mean (context_manager.py:268-277, 664-670).
@@ -202,6 +208,14 @@ int infllm_gather_rows(const void *d_ring, int64_t ring_cap, int32_t B, int32_t 
                        int64_t t0, int32_t n, int32_t unit_rows, void *d_out, int64_t out_sb,
                        int64_t out_su, int64_t out_sh, void *stream);
 int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int32_t kind, void *stream);
+/* infllm_fetch_units: n copies of nbytes each, pinned host -> device, in ONE kernel launch that reads the
+ *   device-mapped pinned memory directly (the misses of a block are scattered over the host arena; issuing a
+ *   hipMemcpyAsync per 512 KiB unit costs more than moving it).  h_src[i] must be the device-visible address
+ *   of pinned memory (infllm_host_device_pointer), both sides 16-byte aligned.  Replaces the H2D half of
+ *   MemoryUnit.load (context_manager.py:76-91).
+ * infllm_host_device_pointer: hipHostGetDevicePointer of a pinned allocation (NULL on failure). */
+int infllm_fetch_units(const void *const *h_src, void *const *d_dst, int32_t n, int64_t nbytes, void *stream);
+void *infllm_host_device_pointer(void *h_pinned);
 
 /* ---------------------------------------------------------------------------
  * One execution block in two calls.
@@ -209,16 +223,29 @@ int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int32_t kind, 
  * (context_manager.py:474-545, 614-679) for one block of at most exc_block_size
  * queries; the host keeps the decisions (cache policy, state machine):
  *
- *   infllm_block_front   prologue (RoPE + rings), mean query, unit scores + top-k with
- *                        an asynchronous copy of the indices to pinned memory, then the
- *                        local stage (which keeps the GPU busy while the host decides);
- *   infllm_layer_wait_topk   blocks until those indices are readable on the host;
- *   infllm_block_back    fetch of missed units (copy stream), page table, global stage,
- *                        merge, local score, init peeling, representatives of the new
- *                        units and their copy to pinned host memory (copy stream).
+ *   infllm_block_front   the block's prologue (RoPE + rings) and retrieval (mean query, unit
+ *                        scores, top-k, asynchronous copy of the ids to pinned memory) unless
+ *                        the previous block already did them ahead; the local stage; then,
+ *                        when the caller passes the NEXT block's rows, that block's prologue
+ *                        and the scores of the units that already exist;
+ *   infllm_layer_wait_topk   blocks until the ids of this block are readable on the host;
+ *   infllm_block_back    fetch of missed units (copy stream), page table, global stage, merge,
+ *                        local score of the tokens about to be carved, init peeling,
+ *                        representatives of the new units, and - when the next block was
+ *                        prepared - the scores of the new units, the next block's top-k and
+ *                        the copy of its ids; only then the rest of the local score and the
+ *                        copy of the new units to pinned host memory (copy stream).
  *
- * A layer handle owns only events, the rotation of the pinned page-table staging
- * slots and of the carve staging slots; every buffer is the caller's.
+ * The chain from one block's ids to the next block's ids is therefore: fetch, global stage,
+ * merge, a small score launch, representatives, a small score launch, top-k.
+ *
+ * The copy of newly carved units to pinned host memory is deferred: it is issued on the copy
+ * stream right after the NEXT block's fetch (or before it, when that fetch needs one of those
+ * units), so a fetch never queues behind it; infllm_layer_flush issues whatever is still
+ * pending and must be called when no further block follows (end of an append() call).
+ *
+ * A layer handle owns only events, the rotation of the pinned page-table staging slots and of
+ * the carve staging slots; every buffer is the caller's.
  */
 typedef struct {
     int32_t B, H, Hkv;
@@ -230,9 +257,10 @@ typedef struct {
     void *d_init_kv;                                  /* [B,2,Hkv,init_cap,128] */
     int64_t init_cap;
     void *d_slab;                                     /* [B,max_cached,2,Hkv,block_size,128] */
-    void *d_q_loc, *d_q_glb;                          /* [B*H*exc*128] each */
-    float *d_qbar;                                    /* [B,H*128] */
-    float *d_qpart;                                   /* [B,ceil(exc/16),H*128] */
+    /* two slots each (a block and the one prepared ahead) */
+    void *d_q_loc, *d_q_glb;                          /* [2][B*H*exc*128] */
+    float *d_qbar;                                    /* [2][B,H*128] */
+    float *d_qpart;                                   /* [2][B,ceil(exc/16),H*128] */
     float *d_o_part, *d_lse_part, *d_lse;             /* [2*max_splits,B,H,exc,(128)], [B,H,exc] */
     int32_t *d_topk_idx, *h_topk_idx;                 /* [B,topk] device / pinned host */
     infllm_page *d_pages;                             /* [B,max_pages] */
@@ -259,6 +287,8 @@ typedef struct {
     int64_t rep_sb, rep_su;
     float *d_unit_scores;                             /* [B, >= n_units] */
     int64_t unit_scores_sb;
+    const void *d_q_next, *d_k_next, *d_v_next;       /* rows of the next block (same strides), or NULL */
+    int32_t n_next, reserved;
 } infllm_front_args;
 int infllm_block_front(void *layer, const infllm_front_args *a, void *stream);
 int infllm_layer_wait_topk(void *layer);
@@ -269,7 +299,8 @@ typedef struct {
     const int32_t *h_sel_slots;                       /* host [B,n_sel]: slab slot of each selected unit */
     int32_t n_miss, init_len;                         /* units to fetch; init tokens present */
     const int32_t *h_miss_row, *h_miss_slot;          /* host [n_miss] */
-    const void *const *h_miss_src;                    /* host [n_miss]: pinned [2,Hkv,block_size,128] */
+    const int32_t *h_miss_unit;                       /* host [n_miss]: unit ids (to order a fetch after that unit's offload) */
+    const void *const *h_miss_src;                    /* host [n_miss]: device-visible address of pinned [2,Hkv,block_size,128] */
     int64_t cursor;                                   /* first un-carved stream position */
     void *d_out;                                      /* [B,H,n,128] bf16 */
     int64_t o_sb, o_sh, o_sl;
@@ -278,8 +309,13 @@ typedef struct {
     int64_t rep_sb, rep_su;
     int32_t *d_repr_idx;                              /* optional [B,n_carve,H,repr_topk] */
     void *const *h_carve_dst;                         /* host [n_carve]: pinned [B,2,Hkv,block_size,128] */
+    int32_t n_units, reserved;                        /* units before this block's carving */
+    const void *d_reps;                               /* [B, rows, H*128] (rep_sb / rep_su above) */
+    float *d_unit_scores;                             /* [B, >= n_units + n_carve] */
+    int64_t unit_scores_sb;
 } infllm_back_args;
 int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream);
+int infllm_layer_flush(void *layer, void *copy_stream);
 
 /* Event timing of the two attention stages (for benchmarks): enable with a record
  * capacity, read back (which: 0 local stage, 1 global stage) after a device sync.

@@ -86,6 +86,7 @@ class FrontArgs(C.Structure):
         ("n", c_i32), ("n_units", c_i32), ("b0", c_i64),
         ("d_reps", c_vp), ("rep_sb", c_i64), ("rep_su", c_i64),
         ("d_unit_scores", c_vp), ("unit_scores_sb", c_i64),
+        ("d_q_next", c_vp), ("d_k_next", c_vp), ("d_v_next", c_vp), ("n_next", c_i32), ("reserved", c_i32),
     ]
 
 
@@ -93,12 +94,13 @@ class BackArgs(C.Structure):
     _fields_ = [
         ("n", c_i32), ("n_sel", c_i32), ("b0", c_i64),
         ("h_sel_slots", c_vp), ("n_miss", c_i32), ("init_len", c_i32),
-        ("h_miss_row", c_vp), ("h_miss_slot", c_vp), ("h_miss_src", c_vp),
+        ("h_miss_row", c_vp), ("h_miss_slot", c_vp), ("h_miss_unit", c_vp), ("h_miss_src", c_vp),
         ("cursor", c_i64),
         ("d_out", c_vp), ("o_sb", c_i64), ("o_sh", c_i64), ("o_sl", c_i64),
         ("init_take", c_i32), ("n_carve", c_i32),
         ("d_rep_out", c_vp), ("rep_sb", c_i64), ("rep_su", c_i64),
         ("d_repr_idx", c_vp), ("h_carve_dst", c_vp),
+        ("n_units", c_i32), ("reserved", c_i32), ("d_reps", c_vp), ("d_unit_scores", c_vp), ("unit_scores_sb", c_i64),
     ]
 
 
@@ -112,16 +114,21 @@ SYMBOLS = {
     "infllm_attn_stage": (c_i32, [C.POINTER(AttnArgs), c_vp]),
     "infllm_attn_merge": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
     "infllm_local_score": (c_i32, [C.POINTER(ScoreArgs), c_vp]),
+    "infllm_unit_scores": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp]),
+    "infllm_topk": (c_i32, [c_vp, c_i32, c_i32, c_vp, c_vp]),
     "infllm_score_topk": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_vp, c_i32, c_vp, c_vp, c_vp]),
     "infllm_repr_keys": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i64, c_i32, c_i32, c_i32,
                                  c_vp, c_i64, c_i64, c_vp, c_vp]),
     "infllm_gather_rows": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i64, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "infllm_copy_async": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_vp]),
+    "infllm_fetch_units": (c_i32, [c_vp, c_vp, c_i32, c_i64, c_vp]),
+    "infllm_host_device_pointer": (c_vp, [c_vp]),
     "infllm_layer_create": (c_vp, [C.POINTER(LayerDesc)]),
     "infllm_layer_destroy": (c_i32, [c_vp]),
     "infllm_block_front": (c_i32, [c_vp, C.POINTER(FrontArgs), c_vp]),
     "infllm_layer_wait_topk": (c_i32, [c_vp]),
     "infllm_block_back": (c_i32, [c_vp, C.POINTER(BackArgs), c_vp, c_vp]),
+    "infllm_layer_flush": (c_i32, [c_vp, c_vp]),
     "infllm_layer_timing": (c_i32, [c_vp, c_i32]),
     "infllm_layer_read_timing": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32]),
 }

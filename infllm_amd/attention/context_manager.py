@@ -156,7 +156,7 @@ class ContextManager:
         self.dtype = q.dtype
         self.device = dev
         bs, exc, topk = self.block_size, self.exc_block_size, self.topk
-        cap = self.n_local + exc + bs
+        cap = self.n_local + 2 * exc + bs          # one block is prepared ahead of the one being attended
         self.ring_cap = cap = (cap + KEY_TILE - 1) // KEY_TILE * KEY_TILE + KEY_TILE
         bf = dict(dtype=torch.bfloat16, device=dev)
         f32 = dict(dtype=torch.float32, device=dev)
@@ -168,16 +168,16 @@ class ContextManager:
         self.slab = torch.zeros((B, self.max_cached_block, 2, Hkv, bs, D), **bf)
         self.reps = torch.zeros((B, 16, H * D), **bf)
         self.unit_scores = torch.empty((B, 16), **f32)
-        self.host_chunks, self._host_base = [], []
+        self.host_chunks, self._host_base, self._host_dev_base = [], [], []
         self.policy = [CachePolicy(self.max_cached_block, self.cache_strategy, self.score_decay) for _ in range(B)]
         self.cursor = 0
         self.init_len = 0
         self.num_global_block = 0
         # workspaces of one execution block
-        self.q_loc = torch.empty((B * H * exc * D,), **bf)
-        self.q_glb = torch.empty((B * H * exc * D,), **bf)
-        self.qbar = torch.empty((B, H * D), **f32)
-        self.qpart = torch.empty((B, (exc + 15) // 16, H * D), **f32)
+        self.q_loc = torch.empty((2, B * H * exc * D), **bf)        # two slots: this block / the one prepared ahead
+        self.q_glb = torch.empty((2, B * H * exc * D), **bf)
+        self.qbar = torch.empty((2, B, H * D), **f32)
+        self.qpart = torch.empty((2, B, (exc + 15) // 16, H * D), **f32)
         n_part = 2 * _MAX_SPLITS
         self.o_part = torch.empty((n_part * B * H * exc * D,), **f32)
         self.lse_part = torch.empty((n_part * B * H * exc,), **f32)
@@ -224,11 +224,13 @@ class ContextManager:
         self._sel_slots = (ctypes.c_int32 * (B * max(topk, 1)))()
         self._miss_row = (ctypes.c_int32 * (B * max(topk, 1)))()
         self._miss_slot = (ctypes.c_int32 * (B * max(topk, 1)))()
+        self._miss_unit = (ctypes.c_int32 * (B * max(topk, 1)))()
         self._miss_src = (ctypes.c_void_p * (B * max(topk, 1)))()
         self._carve_dst = (ctypes.c_void_p * self.max_carve)()
         ba = self._ba
         ba.h_sel_slots = ctypes.addressof(self._sel_slots)
         ba.h_miss_row, ba.h_miss_slot = ctypes.addressof(self._miss_row), ctypes.addressof(self._miss_slot)
+        ba.h_miss_unit = ctypes.addressof(self._miss_unit)
         ba.h_miss_src, ba.h_carve_dst = ctypes.addressof(self._miss_src), ctypes.addressof(self._carve_dst)
         self._fa_ref, self._ba_ref = ctypes.byref(self._fa), ctypes.byref(self._ba)
         self.initialized = True
@@ -245,6 +247,10 @@ class ContextManager:
                             dtype=torch.bfloat16, pin_memory=True)
             self.host_chunks.append(t)
             self._host_base.append(t.data_ptr())
+            dev = self._lib.infllm_host_device_pointer(t.data_ptr())       # address the fetch kernel reads through
+            if not dev:
+                raise _lib.InfLLMHipError((self._lib.infllm_last_error() or b"").decode())
+            self._host_dev_base.append(dev)
         return self._host_base[chunk] + idx * self.unit_bytes
 
     def host_unit(self, unit):
@@ -269,7 +275,7 @@ class ContextManager:
         return [(ms[i], nq[i], nk[i]) for i in range(n)]
 
     # -------------------------------------------------------- one exec block
-    def _block(self, st, n, out_ptr):
+    def _block(self, st, n, out_ptr, n_next):
         lib, layer, fa, ba = self._lib, self._layer, self._fa, self._ba
         B, bs, topk = self.num_units, self.block_size, self.topk
         b0 = self.length + st
@@ -279,6 +285,11 @@ class ContextManager:
         fa.d_k = self._k_ptr + st * self._k_step
         fa.d_v = self._v_ptr + st * self._v_step
         fa.n, fa.n_units, fa.b0 = n, N, b0
+        fa.n_next = n_next
+        if n_next:
+            fa.d_q_next = fa.d_q + n * self._q_step
+            fa.d_k_next = fa.d_k + n * self._k_step
+            fa.d_v_next = fa.d_v + n * self._v_step
         rc = lib.infllm_block_front(layer, self._fa_ref, self._main_raw)
         if rc:
             check(rc, "infllm_block_front")
@@ -307,7 +318,9 @@ class ContextManager:
             for unit in misses:
                 self._miss_row[n_miss] = u
                 self._miss_slot[n_miss] = slot_of[unit]
-                self._miss_src[n_miss] = self._host_unit_addr(unit) + u * self.slot_bytes
+                self._miss_unit[n_miss] = unit
+                chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
+                self._miss_src[n_miss] = self._host_dev_base[chunk] + idx * self.unit_bytes + u * self.slot_bytes
                 n_miss += 1
         if self.cache_strategy == "lru":
             self.load_count += 1
@@ -322,7 +335,7 @@ class ContextManager:
         ba.n, ba.n_sel, ba.b0 = n, n_sel, b0
         ba.n_miss, ba.init_len, ba.cursor = n_miss, init_len, cursor
         ba.d_out = out_ptr
-        ba.init_take, ba.n_carve = take, c
+        ba.init_take, ba.n_carve, ba.n_units = take, c, N
         idx_out = None
         if c:
             if N + c > self.reps.shape[1]:
@@ -350,8 +363,9 @@ class ContextManager:
         rows = max(2 * self.reps.shape[1], need)
         grown = torch.zeros((B, rows, self.reps.shape[2]), dtype=torch.bfloat16, device=self.device)
         grown[:, :N] = self.reps[:, :N]
-        self.reps = grown
-        self.unit_scores = torch.empty((B, rows), dtype=torch.float32, device=self.device)
+        scores = torch.empty((B, rows), dtype=torch.float32, device=self.device)
+        scores[:, :N] = self.unit_scores[:, :N]          # scores prepared ahead for the next block
+        self.reps, self.unit_scores = grown, scores
         self._bind_reps()
 
     def _bind_reps(self):
@@ -361,6 +375,7 @@ class ContextManager:
         fa.d_reps, fa.rep_sb, fa.rep_su = self._reps_ptr, self.reps.stride(0), self.reps.stride(1)
         fa.d_unit_scores, fa.unit_scores_sb = self.unit_scores.data_ptr(), self.unit_scores.stride(0)
         ba.rep_sb, ba.rep_su = self.reps.stride(0), self.reps.stride(1)
+        ba.d_reps, ba.d_unit_scores, ba.unit_scores_sb = fa.d_reps, fa.d_unit_scores, fa.unit_scores_sb
 
     # ----------------------------------------------------------------- append
     def append(self, local_q, local_k, local_v, global_q, global_k, global_v):
@@ -404,8 +419,10 @@ class ContextManager:
         out_ptr, out_step = out.data_ptr(), out.stride(2) * 2
         exc = self.exc_block_size
         for st in range(0, input_length, exc):
-            self._block(st, min(exc, input_length - st), out_ptr + st * out_step)
+            n = min(exc, input_length - st)
+            self._block(st, n, out_ptr + st * out_step, min(exc, input_length - st - n))
         self.length += input_length
+        check(self._lib.infllm_layer_flush(self._layer, self._copy_raw), "infllm_layer_flush")
         if self.perhead:
             out = out.view(batch_size, heads, input_length, -1)
         return out

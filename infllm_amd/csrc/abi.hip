@@ -1,4 +1,6 @@
 // Library identity, error text and the plain copy entry point.
+#include <stdlib.h>
+
 #include "common.h"
 
 static thread_local char g_err[512];
@@ -30,4 +32,83 @@ extern "C" int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int
     hipError_t e = hipMemcpyAsync(dst, src, (size_t)nbytes, k, (hipStream_t)stream);
     if (e != hipSuccess) return infllm_fail(-2, "copy_async: %s", hipGetErrorString(e));
     return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Unit fetch: pinned host memory -> device slots in ONE launch.
+// The sources of a block's cache misses are scattered over the host arena, and a
+// hipMemcpyAsync per unit costs more to issue than the 512 KiB take to move; here the
+// kernel reads the (device-mapped) pinned memory directly over PCIe.
+namespace {
+
+constexpr int kFetchMax = 64;          // units per launch
+constexpr int kFetchChunk = 16384;     // bytes moved by one workgroup iteration (256 threads x 4 x 16 B)
+
+struct FetchList {
+    const uint4 *src[kFetchMax];
+    uint4 *dst[kFetchMax];
+};
+
+// A small, fixed number of workgroups walks all (unit, chunk) pairs: reads that cross PCIe stay
+// outstanding for microseconds, and spreading them over every CU stalls the memory pipelines of the
+// kernels running beside the fetch.  4 independent 16-byte loads per thread keep the link busy.
+__global__ __launch_bounds__(256) void unit_fetch_kernel(FetchList list, int n_units, int64_t nbytes) {
+    const int chunks_per_unit = (int)((nbytes + kFetchChunk - 1) / kFetchChunk);
+    const int total = n_units * chunks_per_unit;
+    for (int w = blockIdx.x; w < total; w += gridDim.x) {
+        const int unit = w / chunks_per_unit;
+        const int64_t begin = (int64_t)(w % chunks_per_unit) * kFetchChunk / 16;
+        const int64_t end = nbytes / 16;
+        const uint4 *src = list.src[unit];
+        uint4 *dst = list.dst[unit];
+        uint4 v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (begin + threadIdx.x + 256 * i < end) v[i] = src[begin + threadIdx.x + 256 * i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (begin + threadIdx.x + 256 * i < end) dst[begin + threadIdx.x + 256 * i] = v[i];
+    }
+}
+
+int fetch_workgroups() {
+    static int n = [] {
+        const char *e = getenv("INFLLM_FETCH_WGS");
+        int v = e ? atoi(e) : 0;
+        return v > 0 ? v : 32;
+    }();
+    return n;
+}
+
+}  // namespace
+
+extern "C" int infllm_fetch_units(const void *const *h_src, void *const *d_dst, int32_t n, int64_t nbytes, void *stream) {
+    INFLLM_REQUIRE(n >= 0 && nbytes >= 0 && nbytes % 16 == 0, "fetch_units: bad sizes n=%d nbytes=%lld", n, (long long)nbytes);
+    INFLLM_REQUIRE(n == 0 || (h_src && d_dst), "fetch_units: null list");
+    if (nbytes == 0) return 0;
+    for (int first = 0; first < n; first += kFetchMax) {
+        const int m = n - first < kFetchMax ? n - first : kFetchMax;
+        FetchList list;
+        for (int i = 0; i < m; ++i) {
+            INFLLM_REQUIRE(h_src[first + i] && d_dst[first + i], "fetch_units: null entry %d", first + i);
+            INFLLM_REQUIRE(((uintptr_t)h_src[first + i] | (uintptr_t)d_dst[first + i]) % 16 == 0, "fetch_units: entry %d is not 16-byte aligned",
+                           first + i);
+            list.src[i] = (const uint4 *)h_src[first + i];
+            list.dst[i] = (uint4 *)d_dst[first + i];
+        }
+        const int64_t work = (int64_t)m * ((nbytes + kFetchChunk - 1) / kFetchChunk);
+        const int wgs = work < fetch_workgroups() ? (int)work : fetch_workgroups();
+        hipLaunchKernelGGL(unit_fetch_kernel, dim3(wgs), dim3(256), 0, (hipStream_t)stream, list, m, nbytes);
+        INFLLM_CHECK_LAUNCH("unit_fetch");
+    }
+    return 0;
+}
+
+extern "C" void *infllm_host_device_pointer(void *h_pinned) {
+    void *d = nullptr;
+    if (!h_pinned || hipHostGetDevicePointer(&d, h_pinned, 0) != hipSuccess) {
+        infllm_fail(-2, "host_device_pointer: %p is not device-mapped pinned memory", h_pinned);
+        return nullptr;
+    }
+    return d;
 }

@@ -174,22 +174,34 @@ __global__ __launch_bounds__(64) void repr_keys_kernel(const float *ring_score, 
 
 }  // namespace
 
+extern "C" int infllm_unit_scores(const void *d_reps, int64_t rep_stride, int32_t first, int32_t count, int32_t C,
+                                  const float *d_qbar, float *d_scores, void *stream) {
+    INFLLM_REQUIRE(d_reps && d_qbar && d_scores, "unit_scores: null pointer");
+    INFLLM_REQUIRE(first >= 0 && count >= 0 && C > 0 && C % 8 == 0 && C <= 16384, "unit_scores: bad sizes first=%d count=%d C=%d",
+                   first, count, C);
+    INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "unit_scores: row stride %lld", (long long)rep_stride);
+    if (count == 0) return 0;
+    const int wgs = count < 4 * 2048 ? (count + 3) / 4 : 2048;
+    hipLaunchKernelGGL(unit_scores_kernel, dim3(wgs), dim3(256), (size_t)C * sizeof(float), (hipStream_t)stream,
+                       (const bf16_t *)d_reps + (int64_t)first * rep_stride, rep_stride, count, C, d_qbar, d_scores + first);
+    INFLLM_CHECK_LAUNCH("unit_scores");
+    return 0;
+}
+
+extern "C" int infllm_topk(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, void *stream) {
+    INFLLM_REQUIRE(d_scores && d_idx, "topk: null pointer");
+    INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && k <= 1024, "topk: k=%d with N=%d", k, N);
+    hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, (hipStream_t)stream, d_scores, N, k, d_idx);
+    INFLLM_CHECK_LAUNCH("topk");
+    return 0;
+}
+
 extern "C" int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbar,
                                  int32_t k, float *d_scores, int32_t *d_idx, void *stream) {
-    INFLLM_REQUIRE(d_reps && d_qbar && d_scores, "score_topk: null pointer");
-    INFLLM_REQUIRE(N > 0 && C > 0 && C % 8 == 0 && C <= 16384, "score_topk: bad sizes N=%d C=%d", N, C);
-    INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "score_topk: row stride %lld", (long long)rep_stride);
-    INFLLM_REQUIRE(k >= 0 && k <= N && k <= 1024, "score_topk: k=%d with N=%d", k, N);
-    INFLLM_REQUIRE(k == 0 || d_idx, "score_topk: null index output");
-    const int wgs = N < 4 * 2048 ? (N + 3) / 4 : 2048;
-    hipLaunchKernelGGL(unit_scores_kernel, dim3(wgs), dim3(256), (size_t)C * sizeof(float), (hipStream_t)stream,
-                       (const bf16_t *)d_reps, rep_stride, N, C, d_qbar, d_scores);
-    INFLLM_CHECK_LAUNCH("unit_scores");
-    if (k > 0) {
-        hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, (hipStream_t)stream, d_scores, N, k, d_idx);
-        INFLLM_CHECK_LAUNCH("topk");
-    }
-    return 0;
+    INFLLM_REQUIRE(N > 0 && k >= 0 && k <= N, "score_topk: k=%d with N=%d", k, N);
+    int rc = infllm_unit_scores(d_reps, rep_stride, 0, N, C, d_qbar, d_scores, stream);
+    if (rc == 0 && k > 0) rc = infllm_topk(d_scores, N, k, d_idx, stream);
+    return rc;
 }
 
 extern "C" int infllm_repr_keys(const float *d_ring_score, const void *d_ring_k_raw, int64_t ring_cap, int32_t B, int32_t H,

@@ -22,9 +22,23 @@ struct Layer {
     hipEvent_t carve_ready = nullptr;     // carve staging filled
     std::vector<hipEvent_t> page_evt, carve_evt;
     std::vector<char> page_busy, carve_busy;
+    std::vector<void *> fetch_dst;
+    hipStream_t copy_stream = nullptr;
+    // device-to-host copy of the units carved by the previous block: issued on the copy stream
+    // right AFTER the next block's fetch, so that it never delays a fetch
+    struct Offload {
+        bool pending = false;
+        int slot = 0, first_unit = 0, count = 0;
+        std::vector<void *> dst;
+    } off;
     int page_cur = 0, carve_cur = 0;
     bool has_global = false;
     bool topk_pending = false;
+    int slot = 0;                         // workspace slot written last
+    int cur_slot = 0;                     // workspace slot of the block between front() and back()
+    bool prepared = false;                // the next block's prologue already ran
+    int64_t prepared_b0 = 0;
+    int prepared_n = 0;
     int timing_cap = 0;
     StageTimer timer[2];
 };
@@ -43,6 +57,27 @@ int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
     int s = want < d.max_splits ? want : d.max_splits;
     if (s > cap) s = cap;
     return s < 1 ? 1 : s;
+}
+
+// copy the pending units from their staging slot to pinned host memory on `cs`
+int issue_offload(Layer *L, hipStream_t cs) {
+    const infllm_layer_desc &d = L->d;
+    const int64_t unit_all = (int64_t)d.B * 2 * d.Hkv * d.block_size * kD;        // one unit, all batch rows
+    const bf16_t *stage = (const bf16_t *)d.d_carve_stage + (int64_t)L->off.slot * d.max_carve * unit_all;
+    HIP_OK(hipStreamWaitEvent(cs, L->carve_ready, 0), "offload: wait carve");
+    const int n = L->off.count;
+    for (int i = 0; i < n;) {                   // one copy per run of units that are contiguous on the host
+        int j = i + 1;
+        while (j < n && (char *)L->off.dst[j] == (char *)L->off.dst[j - 1] + unit_all * sizeof(bf16_t)) ++j;
+        HIP_OK(hipMemcpyAsync(L->off.dst[i], stage + (int64_t)i * unit_all, (size_t)(j - i) * unit_all * sizeof(bf16_t),
+                              hipMemcpyDeviceToHost, cs),
+               "offload: copy");
+        i = j;
+    }
+    HIP_OK(hipEventRecord(L->carve_evt[L->off.slot], cs), "offload: event");
+    L->carve_busy[L->off.slot] = 1;
+    L->off.pending = false;
+    return 0;
 }
 
 int timer_begin(Layer *L, int which, int n_queries, int n_keys, hipStream_t st) {
@@ -70,7 +105,7 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
     const infllm_layer_desc &d = *desc;
     if (d.B <= 0 || d.H <= 0 || d.Hkv <= 0 || d.H % d.Hkv) return bad("bad head geometry");
     if (d.exc <= 0 || d.exc > d.n_local || d.block_size <= 0 || d.topk < 0 || d.topk > d.max_cached) return bad("bad knobs");
-    if (d.ring_cap % kTile || d.ring_cap < (int64_t)d.n_local + d.exc + d.block_size) return bad("ring too small or unaligned");
+    if (d.ring_cap % kTile || d.ring_cap < (int64_t)d.n_local + 2 * d.exc + d.block_size) return bad("ring too small or unaligned");
     if (!d.d_ring_k_raw || !d.d_ring_k_rot || !d.d_ring_v || !d.d_ring_score || !d.d_init_kv || !d.d_slab || !d.d_q_loc ||
         !d.d_q_glb || !d.d_qbar || !d.d_qpart || !d.d_o_part || !d.d_lse_part || !d.d_lse || !d.d_topk_idx || !d.h_topk_idx || !d.d_pages ||
         !d.h_pages || !d.d_carve_stage || !d.d_inv_freq)
@@ -88,6 +123,7 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
     L->carve_evt.resize(d.carve_slots, nullptr);
     L->page_busy.assign(d.page_slots, 0);
     L->carve_busy.assign(d.carve_slots, 0);
+
     for (auto &e : L->page_evt) ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
     for (auto &e : L->carve_evt) ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
     if (!ok) {
@@ -144,6 +180,75 @@ extern "C" int infllm_layer_read_timing(void *layer, int32_t which, float *ms, i
     return n;
 }
 
+namespace {
+
+int run_ingest(Layer *L, const infllm_front_args *a, const void *q, const void *k, const void *v, int n, int64_t b0, int slot,
+               bool want_mean, void *stream) {
+    const infllm_layer_desc &d = L->d;
+    infllm_ingest_args in{};
+    in.d_q = q; in.d_k = k; in.d_v = v;
+    in.q_sb = a->q_sb; in.q_sh = a->q_sh; in.q_sl = a->q_sl;
+    in.k_sb = a->k_sb; in.k_sh = a->k_sh; in.k_sl = a->k_sl;
+    in.v_sb = a->v_sb; in.v_sh = a->v_sh; in.v_sl = a->v_sl;
+    in.B = d.B; in.H = d.H; in.Hkv = d.Hkv; in.n = n;
+    in.pos0 = b0; in.glb_pos = d.n_local - 1;
+    in.d_inv_freq = d.d_inv_freq; in.distance_scale = d.distance_scale;
+    in.d_ring_k_raw = d.d_ring_k_raw; in.d_ring_k_rot = d.d_ring_k_rot; in.d_ring_v = d.d_ring_v;
+    in.d_ring_score = d.d_ring_score; in.ring_cap = d.ring_cap;
+    const int64_t qws = (int64_t)d.B * d.H * d.exc * kD;
+    in.d_q_loc = (bf16_t *)d.d_q_loc + slot * qws;
+    in.d_q_glb = (bf16_t *)d.d_q_glb + slot * qws;
+    const int C = d.H * kD;
+    float *qpart = d.d_qpart + (int64_t)slot * d.B * ((d.exc + 15) / 16) * C;
+    in.d_qpart = want_mean ? qpart : nullptr;
+    int rc = infllm_ingest(&in, stream);
+    if (rc || !want_mean) return rc;
+    return infllm_reduce_partials(qpart, d.B, (n + 15) / 16, C, 1.f / (float)n, d.d_qbar + (int64_t)slot * d.B * C, stream);
+}
+
+int run_unit_scores(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_su, float *scores, int64_t scores_sb, int first,
+                    int count, int slot, void *stream) {
+    const infllm_layer_desc &d = L->d;
+    const int C = d.H * kD;
+    for (int u = 0; u < d.B; ++u) {
+        int rc = infllm_unit_scores((const bf16_t *)reps + (int64_t)u * rep_sb, rep_su, first, count, C,
+                                    d.d_qbar + ((int64_t)slot * d.B + u) * C, scores + (int64_t)u * scores_sb, stream);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+int run_topk(Layer *L, const float *scores, int64_t scores_sb, int n_units, void *stream) {
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream;
+    for (int u = 0; u < d.B; ++u) {
+        int rc = infllm_topk(scores + (int64_t)u * scores_sb, n_units, d.topk, d.d_topk_idx + (int64_t)u * d.topk, stream);
+        if (rc) return rc;
+    }
+    HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
+    HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    L->topk_pending = true;
+    return 0;
+}
+
+int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t j_hi, void *stream) {
+    const infllm_layer_desc &d = L->d;
+    if (j_hi <= j_lo) return 0;
+    infllm_score_args sc{};
+    sc.d_q = (const bf16_t *)d.d_q_loc + (int64_t)slot * d.B * d.H * d.exc * kD;
+    sc.q_sl = kD; sc.q_sh = (int64_t)n * kD; sc.q_sb = (int64_t)d.H * n * kD;
+    sc.B = d.B; sc.H = d.H; sc.Hkv = d.Hkv; sc.Lq = n;
+    sc.d_k = d.d_ring_k_rot;
+    sc.k_sl = kD; sc.k_sh = d.ring_cap * kD; sc.k_sb = (int64_t)d.Hkv * d.ring_cap * kD;
+    sc.cap = d.ring_cap; sc.j_lo = j_lo; sc.j_hi = j_hi;
+    sc.mask = INFLLM_MASK_WINDOW; sc.accumulate = 1; sc.offset = b0; sc.window = d.n_local;
+    sc.d_lse = d.d_lse; sc.softmax_scale = d.softmax_scale;
+    sc.d_score = d.d_ring_score; sc.score_sh = d.ring_cap; sc.score_sb = (int64_t)d.H * d.ring_cap; sc.score_cap = d.ring_cap;
+    return infllm_local_score(&sc, stream);
+}
+
+}  // namespace
+
 extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void *stream) {
     INFLLM_REQUIRE(layer && a, "block_front: null argument");
     Layer *L = (Layer *)layer;
@@ -151,45 +256,32 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     hipStream_t st = (hipStream_t)stream;
     INFLLM_REQUIRE(a->n >= 1 && a->n <= d.exc, "block_front: %d queries do not fit an execution block of %d", a->n, d.exc);
     INFLLM_REQUIRE(a->n_units >= 0 && a->b0 >= 0, "block_front: negative state");
+    INFLLM_REQUIRE(a->n_next >= 0 && a->n_next <= d.exc, "block_front: bad next block size %d", a->n_next);
+    int rc;
 
-    infllm_ingest_args in{};
-    in.d_q = a->d_q; in.d_k = a->d_k; in.d_v = a->d_v;
-    in.q_sb = a->q_sb; in.q_sh = a->q_sh; in.q_sl = a->q_sl;
-    in.k_sb = a->k_sb; in.k_sh = a->k_sh; in.k_sl = a->k_sl;
-    in.v_sb = a->v_sb; in.v_sh = a->v_sh; in.v_sl = a->v_sl;
-    in.B = d.B; in.H = d.H; in.Hkv = d.Hkv; in.n = a->n;
-    in.pos0 = a->b0; in.glb_pos = d.n_local - 1;
-    in.d_inv_freq = d.d_inv_freq; in.distance_scale = d.distance_scale;
-    in.d_ring_k_raw = d.d_ring_k_raw; in.d_ring_k_rot = d.d_ring_k_rot; in.d_ring_v = d.d_ring_v;
-    in.d_ring_score = d.d_ring_score; in.ring_cap = d.ring_cap;
-    in.d_q_loc = d.d_q_loc; in.d_q_glb = d.d_q_glb;
-    in.d_qpart = a->n_units > d.topk ? d.d_qpart : nullptr;
-    int rc = infllm_ingest(&in, stream);
-    if (rc) return rc;
-
-    L->topk_pending = false;
-    if (a->n_units > d.topk) {
-        INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
-        rc = infllm_reduce_partials(d.d_qpart, d.B, (a->n + 15) / 16, d.H * kD, 1.f / (float)a->n, d.d_qbar, stream);
+    // ---- this block's prologue and retrieval, unless the previous block prepared them
+    if (!(L->prepared && L->prepared_b0 == a->b0 && L->prepared_n == a->n)) {
+        L->slot ^= 1;
+        const bool retrieve = a->n_units > d.topk;
+        rc = run_ingest(L, a, a->d_q, a->d_k, a->d_v, a->n, a->b0, L->slot, retrieve, stream);
         if (rc) return rc;
-        const int C = d.H * kD;
-        for (int u = 0; u < d.B; ++u) {
-            rc = infllm_score_topk((const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb, a->rep_su, a->n_units, C,
-                                   d.d_qbar + (int64_t)u * C, d.topk, a->d_unit_scores + (int64_t)u * a->unit_scores_sb,
-                                   d.d_topk_idx + (int64_t)u * d.topk, stream);
+        L->topk_pending = false;
+        if (retrieve) {
+            INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
+            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->slot, stream);
+            if (rc) return rc;
+            rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, stream);
             if (rc) return rc;
         }
-        HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st),
-               "block_front: index copy");
-        HIP_OK(hipEventRecord(L->topk_done, st), "block_front: event");
-        L->topk_pending = true;
     }
+    L->prepared = false;
+    L->cur_slot = L->slot;
 
-    // local stage: causal sliding window over the ring
+    // ---- local stage: causal sliding window over the ring
     const int64_t b1 = a->b0 + a->n;
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
     infllm_attn_args at{};
-    at.d_q = d.d_q_loc;
+    at.d_q = (const bf16_t *)d.d_q_loc + (int64_t)L->cur_slot * d.B * d.H * d.exc * kD;
     at.q_sl = kD; at.q_sh = (int64_t)a->n * kD; at.q_sb = (int64_t)d.H * a->n * kD;
     at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = a->n;
     at.d_k = d.d_ring_k_rot; at.d_v = d.d_ring_v;
@@ -204,7 +296,23 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
     rc = infllm_attn_stage(&at, stream);
     timer_end(L, 0, ti, st);
-    return rc;
+    if (rc) return rc;
+
+    // ---- the next block's prologue and the scores of the units that exist already
+    if (a->n_next > 0 && a->d_q_next && a->d_k_next && a->d_v_next) {
+        L->slot ^= 1;
+        rc = run_ingest(L, a, a->d_q_next, a->d_k_next, a->d_v_next, a->n_next, b1, L->slot, true, stream);
+        if (rc) return rc;
+        if (a->n_units > 0) {
+            INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
+            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->slot, stream);
+            if (rc) return rc;
+        }
+        L->prepared = true;
+        L->prepared_b0 = b1;
+        L->prepared_n = a->n_next;
+    }
+    return 0;
 }
 
 extern "C" int infllm_layer_wait_topk(void *layer) {
@@ -227,27 +335,45 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     INFLLM_REQUIRE(a->n_miss >= 0 && a->n_miss <= d.B * a->n_sel && a->init_len >= 0 && a->init_len <= d.init_cap,
                    "block_back: bad miss / init counts");
     INFLLM_REQUIRE(a->n_sel == 0 || a->h_sel_slots, "block_back: null slot list");
-    INFLLM_REQUIRE(a->n_miss == 0 || (a->h_miss_row && a->h_miss_slot && a->h_miss_src), "block_back: null miss list");
+    INFLLM_REQUIRE(a->n_miss == 0 || (a->h_miss_row && a->h_miss_slot && a->h_miss_src && a->h_miss_unit), "block_back: null miss list");
     INFLLM_REQUIRE(a->d_out && a->cursor >= 0 && a->init_take >= 0 && a->n_carve >= 0 && a->n_carve <= d.max_carve,
                    "block_back: bad output / carve arguments");
+    INFLLM_REQUIRE(a->n_units >= 0, "block_back: negative unit count");
     const int64_t b1 = a->b0 + a->n;
     const int64_t unit_elems = (int64_t)d.Hkv * bs * kD;          // K (or V) of one unit
     const int64_t slot_elems = 2 * unit_elems;
+    const int cur = L->cur_slot;
 
     // ---- 1. fetch missed units into their slots (copy stream)
     if (a->n_miss > 0) {
         if (side && L->has_global) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "block_back: wait global");
+        // a missed unit that is still waiting for its copy to the host must land there first
+        if (L->off.pending) {
+            bool hit = false;
+            for (int i = 0; i < a->n_miss && !hit; ++i)
+                hit = a->h_miss_unit[i] >= L->off.first_unit && a->h_miss_unit[i] < L->off.first_unit + L->off.count;
+            if (hit) {
+                int orc = issue_offload(L, cs);
+                if (orc) return orc;
+            }
+        }
+        L->fetch_dst.resize(a->n_miss);
         for (int i = 0; i < a->n_miss; ++i) {
             const int u = a->h_miss_row[i], slot = a->h_miss_slot[i];
             INFLLM_REQUIRE(u >= 0 && u < d.B && slot >= 0 && slot < d.max_cached && a->h_miss_src[i], "block_back: bad miss entry");
-            bf16_t *dst = (bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + slot) * slot_elems;
-            HIP_OK(hipMemcpyAsync(dst, a->h_miss_src[i], slot_elems * sizeof(bf16_t), hipMemcpyHostToDevice, cs),
-                   "block_back: unit fetch");
+            L->fetch_dst[i] = (bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + slot) * slot_elems;
         }
+        int frc = infllm_fetch_units(a->h_miss_src, L->fetch_dst.data(), a->n_miss, slot_elems * (int64_t)sizeof(bf16_t), copy_stream);
+        if (frc) return frc;
         if (side) {
             HIP_OK(hipEventRecord(L->fetch_done, cs), "block_back: event");
             HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
         }
+    }
+
+    if (L->off.pending) {
+        int orc = issue_offload(L, cs);
+        if (orc) return orc;
     }
 
     // ---- 2. page table of the global stage: units | init | overflow remainder
@@ -301,7 +427,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         }
     }
 
-    // ---- 3. global stage, merge, local score
+    // ---- 3. global stage and merge
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
     const int sl = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
     int parts = sl;
@@ -309,7 +435,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     int rc;
     if (n_pages > 0) {
         infllm_attn_args at{};
-        at.d_q = d.d_q_glb;
+        at.d_q = (const bf16_t *)d.d_q_glb + (int64_t)cur * d.B * d.H * d.exc * kD;
         at.q_sl = kD; at.q_sh = (int64_t)a->n * kD; at.q_sb = (int64_t)d.H * a->n * kD;
         at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = a->n;
         at.cap = kTile;
@@ -330,20 +456,13 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     }
     rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, d.d_lse, stream);
     if (rc) return rc;
-    infllm_score_args sc{};
-    sc.d_q = d.d_q_loc;
-    sc.q_sl = kD; sc.q_sh = (int64_t)a->n * kD; sc.q_sb = (int64_t)d.H * a->n * kD;
-    sc.B = d.B; sc.H = d.H; sc.Hkv = d.Hkv; sc.Lq = a->n;
-    sc.d_k = d.d_ring_k_rot;
-    sc.k_sl = kD; sc.k_sh = d.ring_cap * kD; sc.k_sb = (int64_t)d.Hkv * d.ring_cap * kD;
-    sc.cap = d.ring_cap; sc.j_lo = lo; sc.j_hi = b1;
-    sc.mask = INFLLM_MASK_WINDOW; sc.accumulate = 1; sc.offset = a->b0; sc.window = d.n_local;
-    sc.d_lse = d.d_lse; sc.softmax_scale = d.softmax_scale;
-    sc.d_score = d.d_ring_score; sc.score_sh = d.ring_cap; sc.score_sb = (int64_t)d.H * d.ring_cap; sc.score_cap = d.ring_cap;
-    rc = infllm_local_score(&sc, stream);
-    if (rc) return rc;
 
-    // ---- 4. state-machine actions: init peeling, new units
+    // ---- 4. what the next block's retrieval waits for: scores of the tokens that leave the ring now,
+    //         init peeling, representatives of the new units
+    const int64_t new_cursor = a->cursor + a->init_take + (int64_t)a->n_carve * bs;
+    const int64_t urgent_hi = new_cursor < b1 ? new_cursor : b1;
+    rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, stream);
+    if (rc) return rc;
     int64_t cursor = a->cursor;
     if (a->init_take > 0) {
         INFLLM_REQUIRE(a->init_len + a->init_take <= d.init_cap, "block_back: init overflow");
@@ -361,6 +480,22 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         rc = infllm_repr_keys(d.d_ring_score, d.d_ring_k_raw, d.ring_cap, d.B, d.H, d.Hkv, cursor, bs, a->n_carve, d.repr_topk,
                               a->d_rep_out, a->rep_sb, a->rep_su, a->d_repr_idx, stream);
         if (rc) return rc;
+    }
+    // ---- 5. the next block's retrieval (its prologue ran in block_front)
+    L->topk_pending = false;
+    const int n_units_next = a->n_units + a->n_carve;
+    if (L->prepared && n_units_next > d.topk) {
+        INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_back: null representative / score buffer");
+        rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->slot,
+                             stream);
+        if (rc) return rc;
+        rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, n_units_next, stream);
+        if (rc) return rc;
+    }
+    // ---- 6. off the critical path: the rest of the local score, new units to pinned host memory
+    rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, stream);
+    if (rc) return rc;
+    if (a->n_carve > 0) {
         const int slot = L->carve_cur;
         L->carve_cur = (slot + 1) % d.carve_slots;
         if (L->carve_busy[slot]) HIP_OK(hipEventSynchronize(L->carve_evt[slot]), "block_back: carve slot");
@@ -372,17 +507,21 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         rc = infllm_gather_rows(d.d_ring_v, d.ring_cap, d.B, d.Hkv, cursor, a->n_carve * bs, bs, stage + unit_elems, slot_elems,
                                 unit_all, (int64_t)bs * kD, stream);
         if (rc) return rc;
-        if (side) {
-            HIP_OK(hipEventRecord(L->carve_ready, st), "block_back: event");
-            HIP_OK(hipStreamWaitEvent(cs, L->carve_ready, 0), "block_back: wait carve");
-        }
-        for (int i = 0; i < a->n_carve; ++i) {
-            INFLLM_REQUIRE(a->h_carve_dst[i], "block_back: null carve destination");
-            HIP_OK(hipMemcpyAsync(a->h_carve_dst[i], stage + (int64_t)i * unit_all, unit_all * sizeof(bf16_t), hipMemcpyDeviceToHost, cs),
-                   "block_back: unit offload");
-        }
-        HIP_OK(hipEventRecord(L->carve_evt[slot], cs), "block_back: event");
-        L->carve_busy[slot] = 1;
+        HIP_OK(hipEventRecord(L->carve_ready, st), "block_back: event");
+        for (int i = 0; i < a->n_carve; ++i) INFLLM_REQUIRE(a->h_carve_dst[i], "block_back: null carve destination");
+        L->off.pending = true;
+        L->off.slot = slot;
+        L->off.first_unit = a->n_units;
+        L->off.count = a->n_carve;
+        L->off.dst.assign(a->h_carve_dst, a->h_carve_dst + a->n_carve);
+        L->copy_stream = cs;
     }
+    return 0;
+}
+
+extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
+    INFLLM_REQUIRE(layer, "layer_flush: null layer");
+    Layer *L = (Layer *)layer;
+    if (L->off.pending) return issue_offload(L, (hipStream_t)copy_stream);
     return 0;
 }

@@ -324,6 +324,28 @@ def test_gather_rows_and_copy_async():
     assert torch.equal(back, stage[0])
 
 
+def test_fetch_units_reads_pinned_memory_in_one_launch():
+    import ctypes
+    from infllm_amd import _lib
+    lib = _lib.load()
+    n, elems = 70, 2 * 3 * 40 * D                    # more units than one launch takes, odd-sized units
+    host = torch.empty((n, elems), dtype=torch.bfloat16, pin_memory=True)
+    host.copy_(torch.randn(n, elems).bfloat16())
+    dev_base = lib.infllm_host_device_pointer(host.data_ptr())
+    assert dev_base
+    slab = torch.zeros((n + 3, elems), dtype=torch.bfloat16, device="cuda")
+    order = torch.randperm(n).tolist()
+    src = (ctypes.c_void_p * n)(*[dev_base + i * elems * 2 for i in range(n)])
+    dst = (ctypes.c_void_p * n)(*[slab[order[i]].data_ptr() for i in range(n)])
+    _lib.check(lib.infllm_fetch_units(src, dst, n, elems * 2, torch.cuda.current_stream().cuda_stream), "fetch")
+    torch.cuda.synchronize()
+    for i in range(n):
+        assert torch.equal(slab[order[i]].cpu(), host[i])
+    assert float(slab[n:].abs().max()) == 0.0
+    assert lib.infllm_fetch_units(src, dst, 1, 24, None) < 0           # not a multiple of 16 bytes
+    assert not lib.infllm_host_device_pointer(None)
+
+
 def test_bad_arguments_raise():
     ops = _ops()
     from infllm_amd._lib import InfLLMHipError
