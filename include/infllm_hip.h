@@ -262,7 +262,9 @@ typedef struct {
     float *d_qbar;                                    /* [2][B,H*128] */
     float *d_qpart;                                   /* [2][B,ceil(exc/16),H*128] */
     float *d_o_part, *d_lse_part, *d_lse;             /* [2*max_splits,B,H,exc,(128)], [B,H,exc] */
-    int32_t *d_topk_idx, *h_topk_idx;                 /* [B,topk] device / pinned host */
+    int32_t *d_topk_idx, *h_topk_idx;                 /* [B,topk] device / pinned host; h_topk_idx may be NULL when
+                                                         d_topk_idx is the device-visible address of pinned memory:
+                                                         the top-k kernel then writes the ids where the host reads them */
     infllm_page *d_pages;                             /* [B,max_pages] */
     infllm_page *h_pages;                             /* pinned, [page_slots,B,max_pages] */
     int32_t max_pages, page_slots;
@@ -314,6 +316,10 @@ typedef struct {
     float *d_unit_scores;                             /* [B, >= n_units + n_carve] */
     int64_t unit_scores_sb;
 } infllm_back_args;
+/* Optional: issue the fetch of infllm_block_back ahead of it, as soon as the misses are known (the rest of
+ * the host's bookkeeping then overlaps the transfer); infllm_block_back must follow with the same lists. */
+int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_miss_row, const int32_t *h_miss_slot,
+                       const int32_t *h_miss_unit, const void *const *h_miss_src, void *stream, void *copy_stream);
 int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream);
 int infllm_layer_flush(void *layer, void *copy_stream);
 

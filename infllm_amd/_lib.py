@@ -127,6 +127,7 @@ SYMBOLS = {
     "infllm_layer_destroy": (c_i32, [c_vp]),
     "infllm_block_front": (c_i32, [c_vp, C.POINTER(FrontArgs), c_vp]),
     "infllm_layer_wait_topk": (c_i32, [c_vp]),
+    "infllm_block_fetch": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "infllm_block_back": (c_i32, [c_vp, C.POINTER(BackArgs), c_vp, c_vp]),
     "infllm_layer_flush": (c_i32, [c_vp, c_vp]),
     "infllm_layer_timing": (c_i32, [c_vp, c_i32]),

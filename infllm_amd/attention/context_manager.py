@@ -206,7 +206,12 @@ class ContextManager:
         d.d_q_loc, d.d_q_glb, d.d_qbar = self.q_loc.data_ptr(), self.q_glb.data_ptr(), self.qbar.data_ptr()
         d.d_qpart = self.qpart.data_ptr()
         d.d_o_part, d.d_lse_part, d.d_lse = self.o_part.data_ptr(), self.lse_part.data_ptr(), self.lse.data_ptr()
-        d.d_topk_idx, d.h_topk_idx = self.topk_idx.data_ptr(), self.topk_idx_host.data_ptr()
+        self._lib = _lib.load()
+        # the top-k kernel writes the ids straight into pinned host memory (no copy in the chain)
+        d.d_topk_idx = self._lib.infllm_host_device_pointer(self.topk_idx_host.data_ptr())
+        d.h_topk_idx = None
+        if not d.d_topk_idx:
+            d.d_topk_idx, d.h_topk_idx = self.topk_idx.data_ptr(), self.topk_idx_host.data_ptr()
         d.d_pages, d.h_pages = self.pages_dev.data_ptr(), self.pages_host.data_ptr()
         d.max_pages, d.page_slots = self.max_pages, _PAGE_SLOTS
         d.d_carve_stage, d.max_carve, d.carve_slots = self.carve_stage.data_ptr(), self.max_carve, _CARVE_SLOTS
@@ -322,6 +327,10 @@ class ContextManager:
                 chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
                 self._miss_src[n_miss] = self._host_dev_base[chunk] + idx * self.unit_bytes + u * self.slot_bytes
                 n_miss += 1
+        rc = lib.infllm_block_fetch(layer, n_miss, self._miss_row, self._miss_slot, self._miss_unit, self._miss_src,
+                                    self._main_raw, self._copy_raw)     # the transfer starts now; the rest overlaps it
+        if rc:
+            check(rc, "infllm_block_fetch")
         if self.cache_strategy == "lru":
             self.load_count += 1
         # ---- state machine after the block (context_manager.py:614-679)

@@ -24,6 +24,8 @@ struct Layer {
     std::vector<char> page_busy, carve_busy;
     std::vector<void *> fetch_dst;
     hipStream_t copy_stream = nullptr;
+    bool fetch_issued = false;            // infllm_block_fetch ran for the block in flight
+    bool fetch_wait = false;              // the main stream still has to wait for fetch_done
     // device-to-host copy of the units carved by the previous block: issued on the copy stream
     // right AFTER the next block's fetch, so that it never delays a fetch
     struct Offload {
@@ -59,6 +61,56 @@ int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
     return s < 1 ? 1 : s;
 }
 
+// ---- page table built on the device from the slot list (no host staging, no copy in the chain)
+constexpr int kPageJobSlots = 64;
+struct PageJob {
+    int32_t B, Hkv, bs, max_cached, n_sel, init_len;
+    int32_t n_unit_pages, n_init_pages, n_pages;
+    int64_t cursor, overflow_end, ring_cap, init_cap;
+    const bf16_t *slab, *init_kv, *ring_k, *ring_v;
+    int32_t slots[kPageJobSlots];
+};
+
+__global__ __launch_bounds__(64) void build_pages_kernel(PageJob j, infllm_page *out) {
+    const int p = blockIdx.x * 64 + threadIdx.x, u = blockIdx.y;
+    if (p >= j.n_pages) return;
+    const int64_t unit_elems = (int64_t)j.Hkv * j.bs * kD;
+    infllm_page pg;
+    pg.reserved = 0;
+    if (p < j.n_unit_pages) {
+        const int tpu = (j.bs + kTile - 1) / kTile;
+        const int s = p / tpu, t0 = (p % tpu) * kTile;
+        const bf16_t *kb = j.slab + ((int64_t)u * j.max_cached + j.slots[u * j.n_sel + s]) * 2 * unit_elems;
+        pg.k = kb + (int64_t)t0 * kD;
+        pg.v = kb + unit_elems + (int64_t)t0 * kD;
+        pg.head_stride = (int64_t)j.bs * kD;
+        pg.n_valid = j.bs - t0 < kTile ? j.bs - t0 : kTile;
+    } else if (p < j.n_unit_pages + j.n_init_pages) {
+        const int t0 = (p - j.n_unit_pages) * kTile;
+        const bf16_t *ik = j.init_kv + (int64_t)u * 2 * j.Hkv * j.init_cap * kD;
+        pg.k = ik + (int64_t)t0 * kD;
+        pg.v = ik + (int64_t)j.Hkv * j.init_cap * kD + (int64_t)t0 * kD;
+        pg.head_stride = j.init_cap * kD;
+        pg.n_valid = j.init_len - t0 < kTile ? j.init_len - t0 : kTile;
+    } else {
+        const int want = p - j.n_unit_pages - j.n_init_pages;
+        int64_t pos = j.cursor, len = 0;
+        for (int i = 0; i <= want; ++i) {          // runs of <= 64 rows that do not cross the end of the ring
+            pos += len;
+            len = j.overflow_end - pos;
+            if (len > kTile) len = kTile;
+            const int64_t row = pos % j.ring_cap;
+            if (len > j.ring_cap - row) len = j.ring_cap - row;
+        }
+        const int64_t row = pos % j.ring_cap;
+        pg.k = j.ring_k + ((int64_t)u * j.Hkv * j.ring_cap + row) * kD;
+        pg.v = j.ring_v + ((int64_t)u * j.Hkv * j.ring_cap + row) * kD;
+        pg.head_stride = j.ring_cap * kD;
+        pg.n_valid = (int)len;
+    }
+    out[(int64_t)u * j.n_pages + p] = pg;
+}
+
 // copy the pending units from their staging slot to pinned host memory on `cs`
 int issue_offload(Layer *L, hipStream_t cs) {
     const infllm_layer_desc &d = L->d;
@@ -77,6 +129,40 @@ int issue_offload(Layer *L, hipStream_t cs) {
     HIP_OK(hipEventRecord(L->carve_evt[L->off.slot], cs), "offload: event");
     L->carve_busy[L->off.slot] = 1;
     L->off.pending = false;
+    return 0;
+}
+
+// missed units -> their slab slots on the copy stream; then the pending offload (never ahead of a fetch
+// unless the fetch needs one of the units that are still on their way to the host)
+int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, const int32_t *units, const void *const *srcs,
+             hipStream_t st, hipStream_t cs) {
+    const infllm_layer_desc &d = L->d;
+    const bool side = cs != st;
+    const int64_t slot_elems = 2 * (int64_t)d.Hkv * d.block_size * kD;
+    if (n_miss > 0) {
+        INFLLM_REQUIRE(rows && slots && units && srcs, "fetch: null miss list");
+        if (side && L->has_global) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "fetch: wait global");
+        if (L->off.pending) {
+            bool hit = false;
+            for (int i = 0; i < n_miss && !hit; ++i) hit = units[i] >= L->off.first_unit && units[i] < L->off.first_unit + L->off.count;
+            if (hit) {
+                int orc = issue_offload(L, cs);
+                if (orc) return orc;
+            }
+        }
+        L->fetch_dst.resize(n_miss);
+        for (int i = 0; i < n_miss; ++i) {
+            INFLLM_REQUIRE(rows[i] >= 0 && rows[i] < d.B && slots[i] >= 0 && slots[i] < d.max_cached && srcs[i], "fetch: bad miss entry");
+            L->fetch_dst[i] = (bf16_t *)d.d_slab + ((int64_t)rows[i] * d.max_cached + slots[i]) * slot_elems;
+        }
+        int frc = infllm_fetch_units(srcs, L->fetch_dst.data(), n_miss, slot_elems * (int64_t)sizeof(bf16_t), cs);
+        if (frc) return frc;
+        if (side) {
+            HIP_OK(hipEventRecord(L->fetch_done, cs), "fetch: event");
+            L->fetch_wait = true;
+        }
+    }
+    if (L->off.pending) return issue_offload(L, cs);
     return 0;
 }
 
@@ -107,7 +193,7 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
     if (d.exc <= 0 || d.exc > d.n_local || d.block_size <= 0 || d.topk < 0 || d.topk > d.max_cached) return bad("bad knobs");
     if (d.ring_cap % kTile || d.ring_cap < (int64_t)d.n_local + 2 * d.exc + d.block_size) return bad("ring too small or unaligned");
     if (!d.d_ring_k_raw || !d.d_ring_k_rot || !d.d_ring_v || !d.d_ring_score || !d.d_init_kv || !d.d_slab || !d.d_q_loc ||
-        !d.d_q_glb || !d.d_qbar || !d.d_qpart || !d.d_o_part || !d.d_lse_part || !d.d_lse || !d.d_topk_idx || !d.h_topk_idx || !d.d_pages ||
+        !d.d_q_glb || !d.d_qbar || !d.d_qpart || !d.d_o_part || !d.d_lse_part || !d.d_lse || !d.d_topk_idx || !d.d_pages ||
         !d.h_pages || !d.d_carve_stage || !d.d_inv_freq)
         return bad("null buffer");
     if (d.max_splits < 1 || d.max_splits > 64 || d.num_cus < 1 || d.page_slots < 1 || d.carve_slots < 1 || d.max_carve < 1 ||
@@ -225,7 +311,8 @@ int run_topk(Layer *L, const float *scores, int64_t scores_sb, int n_units, void
         int rc = infllm_topk(scores + (int64_t)u * scores_sb, n_units, d.topk, d.d_topk_idx + (int64_t)u * d.topk, stream);
         if (rc) return rc;
     }
-    HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
+    if (d.h_topk_idx)      // NULL: d_topk_idx is itself host-visible pinned memory, the kernel wrote there
+        HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
     HIP_OK(hipEventRecord(L->topk_done, st), "event");
     L->topk_pending = true;
     return 0;
@@ -324,6 +411,16 @@ extern "C" int infllm_layer_wait_topk(void *layer) {
     return 0;
 }
 
+extern "C" int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_miss_row, const int32_t *h_miss_slot,
+                                  const int32_t *h_miss_unit, const void *const *h_miss_src, void *stream, void *copy_stream) {
+    INFLLM_REQUIRE(layer && n_miss >= 0, "block_fetch: bad arguments");
+    Layer *L = (Layer *)layer;
+    INFLLM_REQUIRE(n_miss <= L->d.B * L->d.topk, "block_fetch: %d misses exceed what a block can select", n_miss);
+    int rc = do_fetch(L, n_miss, h_miss_row, h_miss_slot, h_miss_unit, h_miss_src, (hipStream_t)stream, (hipStream_t)copy_stream);
+    if (rc == 0) L->fetch_issued = true;
+    return rc;
+}
+
 extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream) {
     INFLLM_REQUIRE(layer && a, "block_back: null argument");
     Layer *L = (Layer *)layer;
@@ -335,7 +432,6 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     INFLLM_REQUIRE(a->n_miss >= 0 && a->n_miss <= d.B * a->n_sel && a->init_len >= 0 && a->init_len <= d.init_cap,
                    "block_back: bad miss / init counts");
     INFLLM_REQUIRE(a->n_sel == 0 || a->h_sel_slots, "block_back: null slot list");
-    INFLLM_REQUIRE(a->n_miss == 0 || (a->h_miss_row && a->h_miss_slot && a->h_miss_src && a->h_miss_unit), "block_back: null miss list");
     INFLLM_REQUIRE(a->d_out && a->cursor >= 0 && a->init_take >= 0 && a->n_carve >= 0 && a->n_carve <= d.max_carve,
                    "block_back: bad output / carve arguments");
     INFLLM_REQUIRE(a->n_units >= 0, "block_back: negative unit count");
@@ -344,41 +440,47 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     const int64_t slot_elems = 2 * unit_elems;
     const int cur = L->cur_slot;
 
-    // ---- 1. fetch missed units into their slots (copy stream)
-    if (a->n_miss > 0) {
-        if (side && L->has_global) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "block_back: wait global");
-        // a missed unit that is still waiting for its copy to the host must land there first
-        if (L->off.pending) {
-            bool hit = false;
-            for (int i = 0; i < a->n_miss && !hit; ++i)
-                hit = a->h_miss_unit[i] >= L->off.first_unit && a->h_miss_unit[i] < L->off.first_unit + L->off.count;
-            if (hit) {
-                int orc = issue_offload(L, cs);
-                if (orc) return orc;
-            }
-        }
-        L->fetch_dst.resize(a->n_miss);
-        for (int i = 0; i < a->n_miss; ++i) {
-            const int u = a->h_miss_row[i], slot = a->h_miss_slot[i];
-            INFLLM_REQUIRE(u >= 0 && u < d.B && slot >= 0 && slot < d.max_cached && a->h_miss_src[i], "block_back: bad miss entry");
-            L->fetch_dst[i] = (bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + slot) * slot_elems;
-        }
-        int frc = infllm_fetch_units(a->h_miss_src, L->fetch_dst.data(), a->n_miss, slot_elems * (int64_t)sizeof(bf16_t), copy_stream);
+    // ---- 1. fetch missed units into their slots (copy stream), unless infllm_block_fetch already did
+    if (!L->fetch_issued) {
+        int frc = do_fetch(L, a->n_miss, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src, st, cs);
         if (frc) return frc;
-        if (side) {
-            HIP_OK(hipEventRecord(L->fetch_done, cs), "block_back: event");
-            HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
-        }
     }
-
-    if (L->off.pending) {
-        int orc = issue_offload(L, cs);
-        if (orc) return orc;
+    L->fetch_issued = false;
+    if (L->fetch_wait) {
+        HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
+        L->fetch_wait = false;
     }
 
     // ---- 2. page table of the global stage: units | init | overflow remainder
     const int64_t overflow_end = b1 - d.n_local > a->cursor ? b1 - d.n_local : a->cursor;
     int n_pages = 0;
+    if (d.B * a->n_sel <= kPageJobSlots) {
+        PageJob j{};
+        j.B = d.B; j.Hkv = d.Hkv; j.bs = bs; j.max_cached = d.max_cached; j.n_sel = a->n_sel; j.init_len = a->init_len;
+        j.n_unit_pages = a->n_sel * ((bs + kTile - 1) / kTile);
+        j.n_init_pages = (a->init_len + kTile - 1) / kTile;
+        int n_over = 0;
+        for (int64_t pos = a->cursor; pos < overflow_end; ++n_over) {
+            const int64_t row = pos % d.ring_cap;
+            int64_t len = overflow_end - pos;
+            if (len > kTile) len = kTile;
+            if (len > d.ring_cap - row) len = d.ring_cap - row;
+            pos += len;
+        }
+        j.n_pages = n_pages = j.n_unit_pages + j.n_init_pages + n_over;
+        INFLLM_REQUIRE(n_pages <= d.max_pages, "block_back: %d pages exceed the table (%d)", n_pages, d.max_pages);
+        j.cursor = a->cursor; j.overflow_end = overflow_end; j.ring_cap = d.ring_cap; j.init_cap = d.init_cap;
+        j.slab = (const bf16_t *)d.d_slab; j.init_kv = (const bf16_t *)d.d_init_kv;
+        j.ring_k = (const bf16_t *)d.d_ring_k_raw; j.ring_v = (const bf16_t *)d.d_ring_v;
+        for (int i = 0; i < d.B * a->n_sel; ++i) {
+            INFLLM_REQUIRE(a->h_sel_slots[i] >= 0 && a->h_sel_slots[i] < d.max_cached, "block_back: slot %d out of range", a->h_sel_slots[i]);
+            j.slots[i] = a->h_sel_slots[i];
+        }
+        if (n_pages > 0) {
+            hipLaunchKernelGGL(build_pages_kernel, dim3((n_pages + 63) / 64, d.B), dim3(64), 0, st, j, d.d_pages);
+            INFLLM_CHECK_LAUNCH("build_pages");
+        }
+    } else
     {
         const int slot = L->page_cur;
         L->page_cur = (slot + 1) % d.page_slots;
