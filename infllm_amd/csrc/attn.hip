@@ -24,8 +24,6 @@ constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * kWave;
 constexpr int kQTile = 32;                 // queries per wave
 constexpr int kBig = 1 << 29;              // clamp for mask distances held in int32
-constexpr int kKPad = kD + 8;              // LDS row of K (bf16 elements)
-constexpr int kVPad = kD + 16;             // LDS row of V (bf16 elements)
 
 struct StageRange {
     int64_t lo, hi;   // key index range [lo, hi) visible to a span of queries
@@ -45,25 +43,33 @@ __device__ __forceinline__ StageRange visible_range(const infllm_attn_args &a, i
 
 __device__ __forceinline__ int floordiv64(int64_t x) { return (int)(x >> 6); }   // arithmetic shift = floor
 
-// LDS layouts (both free of bank conflicts for the 16-byte MFMA operand reads):
-//   Ks[buf][row][kKPad]  row = key with bits 2 and 3 swapped inside each 32-key half, so that the
-//                        lane holding MFMA row r reads LDS row r; 272-byte rows rotate the banks.
-//   Vs[buf][key][kVPad]  natural rows; the V^T operand of the second MFMA is formed by the transposing
-//                        LDS read ds_read_b64_tr_b16: in a group of 16 lanes, lane 4*j + q supplies the
-//                        address of 4 consecutive d of key j, and lane i receives element i of key
-//                        j = 0..3, i.e. 4 consecutive keys at one d.  288-byte rows keep the 4 rows of a
-//                        read on disjoint banks.
+// LDS layouts.  Tiles go from global memory straight into LDS (global_load_lds_dwordx4: lane l of a
+// wave deposits its 16 bytes at base + 16*l, so one instruction fills 4 rows of 256 bytes), which leaves
+// no staging registers; which 16-byte chunk of which row a lane FETCHES is free, and that is where the
+// layout is decided:
+//   Ks[buf][R][16 chunks]  LDS row R holds key k_lds_row(R) (bits 2 and 3 swapped inside each 32-key
+//                          half, so the lane that owns MFMA row r reads LDS row r); chunk c of the row
+//                          sits at position c ^ swz(R), so the 8 rows read together hit 8 bank groups.
+//   Vs[buf][R][16 chunks]  natural rows, same swizzle; the V^T operand of the second MFMA is formed by
+//                          the transposing read ds_read_b64_tr_b16: in a group of 16 lanes, lane 4*j + q
+//                          supplies the address of 4 consecutive d of key j, and lane i receives element
+//                          i of keys j = 0..3, i.e. 4 consecutive keys at one d.
 __device__ __forceinline__ int k_lds_row(int key) { return (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1); }
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ s16x4 lds_read_tr(const bf16_t *p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
 }
+__device__ __forceinline__ void load_to_lds16(const bf16_t *g, bf16_t *lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                     (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+}
 
 template <bool PAGED>
 __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[2][kTile][kKPad];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[2][kTile][kVPad];
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[2][kTile][kD];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[2][kTile][kD];
     __shared__ int wg_lo[kWaves], wg_hi[kWaves];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -124,12 +130,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         }
     }
 
-    // ---- cooperative tile loads: thread -> (rows, 16-byte chunk)
-    const int ld_chunk = tid & 15;            // 8 head_dim elements
-    const int ld_row = tid >> 4;              // 0..15
-    u32x4 kbuf[4], vbuf[4];                   // K and V rows ld_row + 16*i
-
-    auto load_tile = [&](int t) {
+    // ---- tile loads: wave w, instruction i fills LDS rows 16*w + 4*i .. +3; lane -> (row, position)
+    const int ld_pos = lane & 15, ld_sub = lane >> 4;
+    auto load_tile = [&](int t, int buf) {
         const bf16_t *kbase, *vbase;
         int64_t k_sl, v_sl;
         int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
@@ -152,19 +155,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            int r = ld_row + 16 * i;
-            kbuf[i] = (r >= row_lo && r < row_hi) ? *(const u32x4 *)(kbase + (int64_t)r * k_sl + ld_chunk * 8)
-                                                 : u32x4{0, 0, 0, 0};
-            vbuf[i] = (r >= row_lo && r < row_hi) ? *(const u32x4 *)(vbase + (int64_t)r * v_sl + ld_chunk * 8)
-                                                 : u32x4{0, 0, 0, 0};
+            const int R0 = 16 * wave + 4 * i, R = R0 + ld_sub;
+            const int chunk = ld_pos ^ swz(R);
+            const int kkey = k_lds_row(R);
+            // rows outside the source keep whatever the buffer held (finite values): their keys are masked
+            if (kkey >= row_lo && kkey < row_hi) load_to_lds16(kbase + (int64_t)kkey * k_sl + chunk * 8, &Ks[buf][R0][0]);
+            if (R >= row_lo && R < row_hi) load_to_lds16(vbase + (int64_t)R * v_sl + chunk * 8, &Vs[buf][R0][0]);
         }
     };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *(u32x4 *)&Ks[buf][k_lds_row(ld_row + 16 * i)][ld_chunk * 8] = kbuf[i];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *(u32x4 *)&Vs[buf][ld_row + 16 * i][ld_chunk * 8] = vbuf[i];
-    };
+    // LDS starts as zeros so that rows never written hold finite values (0 * stale must stay 0)
+    for (int e = tid; e < 2 * kTile * kD / 8; e += kThreads) {
+        ((u32x4 *)&Ks[0][0][0])[e] = u32x4{0, 0, 0, 0};
+        ((u32x4 *)&Vs[0][0][0])[e] = u32x4{0, 0, 0, 0};
+    }
+    __syncthreads();
 
     // ---- running softmax state of this lane's query (max kept in raw logit units)
     float m_run = -INFINITY, l_run = 0.f;
@@ -176,14 +180,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
 
     const float scale = a.softmax_scale * 1.4426950408889634f;
 
-    if (g_t1 > g_t0) {
-        load_tile(g_t0);
-        store_tile(0);
-        if (g_t0 + 1 < g_t1) load_tile(g_t0 + 1);
-    }
+    if (g_t1 > g_t0) load_tile(g_t0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     for (int t = g_t0; t < g_t1; ++t) {
         const int cur = (t - g_t0) & 1;
+        if (t + 1 < g_t1) load_tile(t + 1, cur ^ 1);   // lands while this tile is computed; that buffer was
+                                                       // last read before the barrier that ended tile t-1
         if (t >= w_t0 && t < w_t1) {           // wave-uniform; the barrier stays outside
             f32x16 s[2];
 #pragma unroll
@@ -192,17 +195,28 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                 for (int r = 0; r < 16; ++r) s[ks][r] = 0.f;
             }
             {
-                bf16x8 ka[2][kD / 16];             // all 16 K operands are requested before the first MFMA
+                // 16 K operands in groups of 4: a group is requested from LDS while the MFMAs of the
+                // previous group run (scheduling fences keep the compiler from serialising read -> MFMA)
+                bf16x8 ka[4][4];
+                auto k_operand = [&](int i) {          // i = ks * 8 + kk
+                    return *(const bf16x8 *)&Ks[cur][(i >> 3) * 32 + col][((((i & 7) * 2) + grp) ^ swz(col)) * 8];
+                };
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
+                for (int j = 0; j < 4; ++j) ka[0][j] = k_operand(j);
 #pragma unroll
-                    for (int kk = 0; kk < kD / 16; ++kk)
-                        ka[ks][kk] = *(const bf16x8 *)&Ks[cur][ks * 32 + col][grp * 8 + kk * 16];
+                for (int gi = 0; gi < 4; ++gi) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (gi < 3) {
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
+                        for (int j = 0; j < 4; ++j) ka[gi + 1][j] = k_operand((gi + 1) * 4 + j);
+                    }
 #pragma unroll
-                    for (int kk = 0; kk < kD / 16; ++kk)
-                        s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks][kk], qreg[kk], s[ks], 0, 0, 0);
+                    for (int j = 0; j < 4; ++j) {
+                        const int i = gi * 4 + j;
+                        s[i >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[gi][j], qreg[i & 7], s[i >> 3], 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
             // ---- mask (only tiles that touch a boundary); distances are clamped into int32
             bool need_mask;
@@ -272,34 +286,39 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             {
                 // V^T operands: lane -> (4 keys j, 4 d) address pattern of the transposing read
                 const int lam = lane & 15, g16 = lane >> 4;
-                const bf16_t *vrow = &Vs[cur][8 * (g16 >> 1) + (lam >> 2)][16 * (g16 & 1) + 4 * (lam & 3)];
-                s16x4 va[4][kD / 32][2];           // [ks*2+mm][dt][key half]
-#pragma unroll
-                for (int gi = 0; gi < 4; ++gi)
+                const int vr = 8 * (g16 >> 1) + (lam >> 2);              // row inside a 16-key step (second read: +4)
+                const int vc = 2 * (g16 & 1) + ((lam & 3) >> 1);         // 16-byte chunk inside a 32-d tile
+                const int vh = 4 * (lam & 1);                            // element offset inside the chunk
+                // 4 groups (16 keys each) of 4 MFMAs; the operands of a group are requested from LDS while
+                // the MFMAs of the previous group run
+                s16x4 va[2][kD / 32][2];           // [group parity][dt][key half]
+                auto v_operands = [&](int gi, s16x4 (*dst)[2]) {
 #pragma unroll
                     for (int dt = 0; dt < kD / 32; ++dt) {
-                        const bf16_t *p0 = vrow + (gi * 16) * kVPad + dt * 32;
-                        va[gi][dt][0] = lds_read_tr(p0);
-                        va[gi][dt][1] = lds_read_tr(p0 + 4 * kVPad);
+                        const int r0 = gi * 16 + vr, r1 = r0 + 4;
+                        dst[dt][0] = lds_read_tr(&Vs[cur][r0][((dt * 4 + vc) ^ swz(r0)) * 8 + vh]);
+                        dst[dt][1] = lds_read_tr(&Vs[cur][r1][((dt * 4 + vc) ^ swz(r1)) * 8 + vh]);
                     }
+                };
+                v_operands(0, va[0]);
 #pragma unroll
                 for (int gi = 0; gi < 4; ++gi) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (gi < 3) v_operands(gi + 1, va[(gi + 1) & 1]);
                     const int ks = gi >> 1, mm = gi & 1;
                     u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
                     bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
 #pragma unroll
                     for (int dt = 0; dt < kD / 32; ++dt) {
                         typedef short s16x8 __attribute__((ext_vector_type(8)));
-                        s16x8 v8 = __builtin_shufflevector(va[gi][dt][0], va[gi][dt][1], 0, 1, 2, 3, 4, 5, 6, 7);
+                        s16x8 v8 = __builtin_shufflevector(va[gi & 1][dt][0], va[gi & 1][dt][1], 0, 1, 2, 3, 4, 5, 6, 7);
                         oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, v8), pb, oacc[dt], 0, 0, 0);
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (t + 1 < g_t1) {
-            store_tile(cur ^ 1);                // the other buffer was last read one barrier ago
-            if (t + 2 < g_t1) load_tile(t + 2);  // in flight during the next tile's math
-        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
