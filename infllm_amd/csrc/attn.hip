@@ -66,10 +66,18 @@ __device__ __forceinline__ void load_to_lds16(const bf16_t *g, bf16_t *lds_wave_
                                      (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
 
+constexpr int kTileBytes = kTile * kD * 2;        // one K (or V) tile in LDS
+constexpr float kLazyLog2 = 8.f;                  // the running max may lag the true max by 2^8
+
+template <int N>
+struct IntC {
+    static constexpr int value = N;
+};
+
 template <bool PAGED>
 __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[2][kTile][kD];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[2][kTile][kD];
+    __shared__ __attribute__((aligned(16))) char Ks[2 * kTileBytes];
+    __shared__ __attribute__((aligned(16))) char Vs[2 * kTileBytes];
     __shared__ int wg_lo[kWaves], wg_hi[kWaves];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -79,6 +87,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     const int split = blockIdx.z;
     const int n_qtiles = (a.Lq + kQTile - 1) / kQTile;
     const int n_tasks = n_qtiles * G;
+#ifdef INFLLM_PHASES
+    long long *ph = (long long *)a.d_lse_part + 1024 * 1024;     // debug build only: stamps beyond the lse partials
+    int ph_n = 0;
+    const bool ph_on = blockIdx.x == 3 && blockIdx.y == 1 && blockIdx.z == 1 && tid == 0;
+#define PH_STAMP() do { if (ph_on && ph_n < 512) ph[ph_n++] = clock64(); } while (0)
+#else
+#define PH_STAMP() do { } while (0)
+#endif
+    PH_STAMP();
 
     // ---- this wave's task and the tiles it needs
     const int task = blockIdx.x * kWaves + wave;
@@ -105,6 +122,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         wg_lo[wave] = w_t1 > w_t0 ? w_t0 : INT32_MAX;
         wg_hi[wave] = w_t1 > w_t0 ? w_t1 : INT32_MIN;
     }
+    // LDS starts as zeros so that rows never written hold finite values (0 * stale must stay 0)
+    for (int e = tid; e < 2 * kTileBytes / 16; e += kThreads) {
+        ((u32x4 *)Ks)[e] = u32x4{0, 0, 0, 0};
+        ((u32x4 *)Vs)[e] = u32x4{0, 0, 0, 0};
+    }
     __syncthreads();
     int g_t0 = min(min(wg_lo[0], wg_lo[1]), min(wg_lo[2], wg_lo[3]));
     int g_t1 = max(max(wg_hi[0], wg_hi[1]), max(wg_hi[2], wg_hi[3]));
@@ -130,48 +152,82 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         }
     }
 
-    // ---- tile loads: wave w, instruction i fills LDS rows 16*w + 4*i .. +3; lane -> (row, position)
-    const int ld_pos = lane & 15, ld_sub = lane >> 4;
+    // ---- per-lane LDS byte offsets of the MFMA operands (inside one tile buffer)
+    uint32_t k_off[kD / 16];                  // K operand kk of sub-tile 0 (sub-tile 1: + 32 rows)
+#pragma unroll
+    for (int kk = 0; kk < kD / 16; ++kk) k_off[kk] = col * 256 + (((kk * 2 + grp) ^ swz(col)) * 16);
+    uint32_t v_off[kD / 32][2];               // V^T operand of d-tile dt, key half e, of 16-key step 0 (step gi: + 16*gi rows)
+    {
+        const int lam = lane & 15, g16 = lane >> 4;
+        const int vr = 8 * (g16 >> 1) + (lam >> 2);              // lane 4*j + q addresses key j ...
+        const int vc = 2 * (g16 & 1) + ((lam & 3) >> 1);         // ... at 4 consecutive d: 16-byte chunk
+        const int vh = 8 * (lam & 1);                            //     and byte offset inside it
+#pragma unroll
+        for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) v_off[dt][e] = (vr + 4 * e) * 256 + (((dt * 4 + vc) ^ swz(vr + 4 * e)) * 16) + vh;
+    }
+
+    // ---- tile loads: wave w, instruction i fills LDS rows 16*w + 4*i .. +3; lane -> (row, position).
+    //      The wave-uniform tile base advances with the loop; the per-lane offsets are loop invariant.
+    uint32_t gk_off[4], gv_off[4];            // element offsets inside a tile
+    int gk_row[4], gv_row[4];
+    {
+        const int ld_pos = lane & 15, ld_sub = lane >> 4;
+        const int64_t k_sl = PAGED ? kD : a.k_sl, v_sl = PAGED ? kD : a.v_sl;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int R = 16 * wave + 4 * i + ld_sub, chunk = ld_pos ^ swz(R);
+            gk_row[i] = k_lds_row(R);
+            gv_row[i] = R;
+            gk_off[i] = (uint32_t)(gk_row[i] * k_sl + chunk * 8);
+            gv_off[i] = (uint32_t)(R * v_sl + chunk * 8);
+        }
+    }
+    const bf16_t *k_head = nullptr, *v_head = nullptr;          // linear source: row 0 of this kv head
+    int64_t ring_row = 0;                                        // ring row of the tile to load next
+    if (!PAGED) {
+        k_head = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh;
+        v_head = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh;
+        ring_row = ((int64_t)g_t0 * kTile) % a.cap;
+    }
     auto load_tile = [&](int t, int buf) {
         const bf16_t *kbase, *vbase;
-        int64_t k_sl, v_sl;
         int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
         if (PAGED) {
             const infllm_page pg = a.d_pages[(int64_t)b * a.n_pages + t];
             kbase = (const bf16_t *)pg.k + (int64_t)g * pg.head_stride;
             vbase = (const bf16_t *)pg.v + (int64_t)g * pg.head_stride;
-            k_sl = v_sl = kD;
             row_lo = 0;
             row_hi = pg.n_valid;
         } else {
             const int64_t j0 = (int64_t)t * kTile;
-            const int64_t r0 = j0 % a.cap;    // cap is a multiple of the tile, so a tile never wraps
-            kbase = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh + r0 * a.k_sl;
-            vbase = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh + r0 * a.v_sl;
-            k_sl = a.k_sl;
-            v_sl = a.v_sl;
+            kbase = k_head + ring_row * a.k_sl;       // cap is a multiple of the tile, so a tile never wraps
+            vbase = v_head + ring_row * a.v_sl;
+            ring_row += kTile;
+            if (ring_row >= a.cap) ring_row -= a.cap;
             row_lo = (int)max((int64_t)0, a.j_lo - j0);
             row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
         }
+        char *kdst = Ks + buf * kTileBytes + wave * 4096, *vdst = Vs + buf * kTileBytes + wave * 4096;
+        if (row_lo == 0 && row_hi == kTile) {          // the common case: no per-lane predicate
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int R0 = 16 * wave + 4 * i, R = R0 + ld_sub;
-            const int chunk = ld_pos ^ swz(R);
-            const int kkey = k_lds_row(R);
-            // rows outside the source keep whatever the buffer held (finite values): their keys are masked
-            if (kkey >= row_lo && kkey < row_hi) load_to_lds16(kbase + (int64_t)kkey * k_sl + chunk * 8, &Ks[buf][R0][0]);
-            if (R >= row_lo && R < row_hi) load_to_lds16(vbase + (int64_t)R * v_sl + chunk * 8, &Vs[buf][R0][0]);
+            for (int i = 0; i < 4; ++i) {
+                load_to_lds16(kbase + gk_off[i], (bf16_t *)(kdst + i * 1024));
+                load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // rows outside the source keep whatever the buffer held (finite values): their keys are masked
+                if (gk_row[i] >= row_lo && gk_row[i] < row_hi) load_to_lds16(kbase + gk_off[i], (bf16_t *)(kdst + i * 1024));
+                if (gv_row[i] >= row_lo && gv_row[i] < row_hi) load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
+            }
         }
     };
-    // LDS starts as zeros so that rows never written hold finite values (0 * stale must stay 0)
-    for (int e = tid; e < 2 * kTile * kD / 8; e += kThreads) {
-        ((u32x4 *)&Ks[0][0][0])[e] = u32x4{0, 0, 0, 0};
-        ((u32x4 *)&Vs[0][0][0])[e] = u32x4{0, 0, 0, 0};
-    }
-    __syncthreads();
 
-    // ---- running softmax state of this lane's query (max kept in raw logit units)
-    float m_run = -INFINITY, l_run = 0.f;
+    // ---- running softmax state of this lane's query (max kept in raw logit units, allowed to lag)
+    float m_run = -INFINITY, l_run = 0.f, neg_ms = 0.f;
     f32x16 oacc[kD / 32];
 #pragma unroll
     for (int dt = 0; dt < kD / 32; ++dt)
@@ -179,149 +235,166 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         for (int r = 0; r < 16; ++r) oacc[dt][r] = 0.f;
 
     const float scale = a.softmax_scale * 1.4426950408889634f;
+    const float lazy = kLazyLog2 / scale;
+
+    auto tile_math = [&](auto buf_c, int t) {
+        constexpr int BUF = decltype(buf_c)::value;
+        const char *kb = Ks + BUF * kTileBytes, *vb = Vs + BUF * kTileBytes;
+        f32x16 s[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[ks][r] = 0.f;
+        {
+            // 16 K operands in groups of 4 (kk pair x both sub-tiles): a group is requested from LDS while the
+            // MFMAs of the previous one run; scheduling fences keep the compiler from serialising read -> MFMA
+            bf16x8 ka[4][4];
+            auto k_operand = [&](int i) {          // i = kk * 2 + ks
+                return *(const bf16x8 *)(kb + (i & 1) * 32 * 256 + k_off[i >> 1]);
+            };
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ka[0][j] = k_operand(j);
+#pragma unroll
+            for (int gi = 0; gi < 4; ++gi) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (gi < 3) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) ka[gi + 1][j] = k_operand((gi + 1) * 4 + j);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = gi * 4 + j;
+                    s[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[gi][j], qreg[i >> 1], s[i & 1], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // ---- mask (only tiles that touch a boundary); distances are clamped into int32
+        bool need_mask;
+        int row_lo = 0, row_hi = kTile;
+        int d0 = 0;                            // dist of (this lane's query, key 0 of the tile)
+        if (PAGED) {
+            row_hi = a.d_pages[(int64_t)b * a.n_pages + t].n_valid;
+            need_mask = row_hi < kTile;
+        } else {
+            const int64_t j0 = (int64_t)t * kTile;
+            row_lo = (int)max((int64_t)0, a.j_lo - j0);
+            row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
+            need_mask = row_lo > 0 || row_hi < kTile;
+            const int64_t e0 = (int64_t)i0 + a.offset - j0;       // dist(query i0, key j0)
+            if (a.mask == INFLLM_MASK_WINDOW) {
+                need_mask |= (e0 < kTile - 1) || (e0 + (i1 - i0) >= a.window);
+            } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
+                need_mask |= (e0 - (kTile - 1) < a.window);
+            }
+            d0 = (int)min(max(e0, (int64_t)-kBig), (int64_t)kBig) + col;
+        }
+        if (need_mask) {
+            const int win = (int)min(a.window, (int64_t)2 * kBig);
+            const int lo_l = row_lo - 8 * grp, hi_l = row_hi - 8 * grp;      // bounds on kc for this lane
+            const int dl = d0 - 8 * grp;                                       // dist = dl - kc
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    // key of register r: ko = kc + 8*grp with the compile-time part kc; everything is
+                    // expressed relative to the per-lane bases so that no per-register value is kept
+                    const int kc = ks * 32 + 16 * (r >> 3) + (r & 7);
+                    bool vis = (kc >= lo_l) && (kc < hi_l);
+                    if (!PAGED) {
+                        if (a.mask == INFLLM_MASK_WINDOW) vis = vis && (kc <= dl) && (kc > dl - win);
+                        if (a.mask == INFLLM_MASK_COMPLEMENT) vis = vis && (kc <= dl - win);
+                    }
+                    s[ks][r] = vis ? s[ks][r] : -INFINITY;
+                }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[ks][r]);
+        tmax = fmaxf(tmax, wave_xor32(tmax));
+        // lazy running max: it only moves when a score would exceed it by more than 2^kLazyLog2 after scaling,
+        // so the rescale of the output accumulators is rare; probabilities stay below 2^kLazyLog2
+        const bool moved = tmax > m_run + lazy;
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+            const float m_new = moved ? tmax : m_run;
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale);      // exp2(-inf) = 0 on the first move
+            const float al = moved ? alpha : 1.f;
+            l_run *= al;
+#pragma unroll
+            for (int dt = 0; dt < kD / 32; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[dt][r] *= al;
+            m_run = m_new;
+            neg_ms = (m_run == -INFINITY) ? 0.f : -m_run * scale;
+        }
+        float psum = 0.f;
+        uint32_t pw[2][8];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r], scale, neg_ms));
+                float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r + 1], scale, neg_ms));
+                psum += p0 + p1;
+                pw[ks][r >> 1] = pack_bf16x2(p0, p1);
+            }
+        l_run += psum;
+        {
+            // 4 steps of 16 keys, 4 MFMAs each; the V^T operands of a step are requested from LDS while the
+            // MFMAs of the previous step run
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            s16x8 va[2][kD / 32];
+            auto v_operands = [&](int gi, s16x8 *dst) {
+#pragma unroll
+                for (int dt = 0; dt < kD / 32; ++dt) {
+                    dst[dt].lo = lds_read_tr((const bf16_t *)(vb + gi * 16 * 256 + v_off[dt][0]));
+                    dst[dt].hi = lds_read_tr((const bf16_t *)(vb + gi * 16 * 256 + v_off[dt][1]));
+                }
+            };
+            v_operands(0, va[0]);
+#pragma unroll
+            for (int gi = 0; gi < 4; ++gi) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (gi < 3) {
+                    v_operands(gi + 1, va[(gi + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                const int ks = gi >> 1, mm = gi & 1;
+                u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
+                bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+#pragma unroll
+                for (int dt = 0; dt < kD / 32; ++dt)
+                    oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[gi & 1][dt]), pb, oacc[dt], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
 
     if (g_t1 > g_t0) load_tile(g_t0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int t = g_t0; t < g_t1; ++t) {
-        const int cur = (t - g_t0) & 1;
-        if (t + 1 < g_t1) load_tile(t + 1, cur ^ 1);   // lands while this tile is computed; that buffer was
-                                                       // last read before the barrier that ended tile t-1
-        if (t >= w_t0 && t < w_t1) {           // wave-uniform; the barrier stays outside
-            f32x16 s[2];
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) s[ks][r] = 0.f;
-            }
-            {
-                // 16 K operands in groups of 4: a group is requested from LDS while the MFMAs of the
-                // previous group run (scheduling fences keep the compiler from serialising read -> MFMA)
-                bf16x8 ka[4][4];
-                auto k_operand = [&](int i) {          // i = ks * 8 + kk
-                    return *(const bf16x8 *)&Ks[cur][(i >> 3) * 32 + col][((((i & 7) * 2) + grp) ^ swz(col)) * 8];
-                };
-#pragma unroll
-                for (int j = 0; j < 4; ++j) ka[0][j] = k_operand(j);
-#pragma unroll
-                for (int gi = 0; gi < 4; ++gi) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (gi < 3) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) ka[gi + 1][j] = k_operand((gi + 1) * 4 + j);
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const int i = gi * 4 + j;
-                        s[i >> 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[gi][j], qreg[i & 7], s[i >> 3], 0, 0, 0);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // ---- mask (only tiles that touch a boundary); distances are clamped into int32
-            bool need_mask;
-            int row_lo = 0, row_hi = kTile;
-            int d0 = 0;                            // dist of (this lane's query, key 0 of the tile)
-            if (PAGED) {
-                row_hi = a.d_pages[(int64_t)b * a.n_pages + t].n_valid;
-                need_mask = row_hi < kTile;
-            } else {
-                const int64_t j0 = (int64_t)t * kTile;
-                row_lo = (int)max((int64_t)0, a.j_lo - j0);
-                row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
-                need_mask = row_lo > 0 || row_hi < kTile;
-                const int64_t e0 = (int64_t)i0 + a.offset - j0;       // dist(query i0, key j0)
-                if (a.mask == INFLLM_MASK_WINDOW) {
-                    need_mask |= (e0 < kTile - 1) || (e0 + (i1 - i0) >= a.window);
-                } else if (a.mask == INFLLM_MASK_COMPLEMENT) {
-                    need_mask |= (e0 - (kTile - 1) < a.window);
-                }
-                d0 = (int)min(max(e0, (int64_t)-kBig), (int64_t)kBig) + col;
-            }
-            if (need_mask) {
-                const int win = (int)min(a.window, (int64_t)2 * kBig);
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int ko = ks * 32 + 16 * (r >> 3) + 8 * grp + (r & 7);
-                        bool vis = ko >= row_lo && ko < row_hi;
-                        if (!PAGED) {
-                            const int dist = d0 - ko;
-                            if (a.mask == INFLLM_MASK_WINDOW) vis = vis && dist >= 0 && dist < win;
-                            if (a.mask == INFLLM_MASK_COMPLEMENT) vis = vis && dist >= win;
-                        }
-                        s[ks][r] = vis ? s[ks][r] : -INFINITY;
-                    }
-            }
-            float tmax = -INFINITY;
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[ks][r]);
-            tmax = fmaxf(tmax, wave_xor32(tmax));
-            const float m_new = fmaxf(m_run, tmax);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale);
-            const float neg_ms = -m_use * scale;
-            float psum = 0.f;
-            uint32_t pw[2][8];
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int r = 0; r < 16; r += 2) {
-                    float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r], scale, neg_ms));
-                    float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r + 1], scale, neg_ms));
-                    psum += p0 + p1;
-                    pw[ks][r >> 1] = pack_bf16x2(p0, p1);
-                }
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {     // some query of the wave moved its max
-#pragma unroll
-                for (int dt = 0; dt < kD / 32; ++dt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[dt][r] *= alpha;
-            }
-            {
-                // V^T operands: lane -> (4 keys j, 4 d) address pattern of the transposing read
-                const int lam = lane & 15, g16 = lane >> 4;
-                const int vr = 8 * (g16 >> 1) + (lam >> 2);              // row inside a 16-key step (second read: +4)
-                const int vc = 2 * (g16 & 1) + ((lam & 3) >> 1);         // 16-byte chunk inside a 32-d tile
-                const int vh = 4 * (lam & 1);                            // element offset inside the chunk
-                // 4 groups (16 keys each) of 4 MFMAs; the operands of a group are requested from LDS while
-                // the MFMAs of the previous group run
-                s16x4 va[2][kD / 32][2];           // [group parity][dt][key half]
-                auto v_operands = [&](int gi, s16x4 (*dst)[2]) {
-#pragma unroll
-                    for (int dt = 0; dt < kD / 32; ++dt) {
-                        const int r0 = gi * 16 + vr, r1 = r0 + 4;
-                        dst[dt][0] = lds_read_tr(&Vs[cur][r0][((dt * 4 + vc) ^ swz(r0)) * 8 + vh]);
-                        dst[dt][1] = lds_read_tr(&Vs[cur][r1][((dt * 4 + vc) ^ swz(r1)) * 8 + vh]);
-                    }
-                };
-                v_operands(0, va[0]);
-#pragma unroll
-                for (int gi = 0; gi < 4; ++gi) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (gi < 3) v_operands(gi + 1, va[(gi + 1) & 1]);
-                    const int ks = gi >> 1, mm = gi & 1;
-                    u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
-                    bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
-#pragma unroll
-                    for (int dt = 0; dt < kD / 32; ++dt) {
-                        typedef short s16x8 __attribute__((ext_vector_type(8)));
-                        s16x8 v8 = __builtin_shufflevector(va[gi & 1][dt][0], va[gi & 1][dt][1], 0, 1, 2, 3, 4, 5, 6, 7);
-                        oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, v8), pb, oacc[dt], 0, 0, 0);
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
+    // two tiles per trip so that the LDS buffer index is a compile-time constant; a tile is loaded into the
+    // buffer that was last read before the previous barrier, and lands while the current tile is computed
+    for (int t = g_t0; t < g_t1; t += 2) {
+        PH_STAMP();
+        if (t + 1 < g_t1) load_tile(t + 1, 1);
+        PH_STAMP();
+        if (t >= w_t0 && t < w_t1) tile_math(IntC<0>{}, t);          // wave-uniform; barriers stay outside
+        PH_STAMP();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PH_STAMP();
+        __syncthreads();
+        if (t + 1 >= g_t1) break;
+        if (t + 2 < g_t1) load_tile(t + 2, 0);
+        if (t + 1 >= w_t0 && t + 1 < w_t1) tile_math(IntC<1>{}, t + 1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
+    PH_STAMP();
     // ---- epilogue: normalised partial + base-2 log-sum-exp
     if (!live) return;
     const float l_tot = l_run + wave_xor32(l_run);
@@ -339,6 +412,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             *(f32x4 *)(orow + dt * 32 + 8 * q4 + 4 * grp) = o4;
         }
     if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run * scale + log2f(l_tot) : -INFINITY;
+    PH_STAMP();
 }
 
 // one thread per (row, 4 dims): P partials -> bf16 output row + final lse
