@@ -20,7 +20,8 @@
 
 namespace {
 
-constexpr int kWaves = 4;
+constexpr int kWaves = 8;                  // 2 per SIMD inside ONE workgroup: a K/V tile in LDS feeds 256 query rows
+constexpr int kStages = 4;                 // K/V tiles resident in LDS (up to 3 in flight ahead of the math)
 constexpr int kThreads = kWaves * kWave;
 constexpr int kQTile = 32;                 // queries per wave
 constexpr int kBig = 1 << 29;              // clamp for mask distances held in int32
@@ -76,8 +77,8 @@ struct IntC {
 
 template <bool PAGED>
 __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a) {
-    __shared__ __attribute__((aligned(16))) char Ks[2 * kTileBytes];
-    __shared__ __attribute__((aligned(16))) char Vs[2 * kTileBytes];
+    extern __shared__ __attribute__((aligned(16))) char lds_dyn[];      // kStages K tiles, then kStages V tiles
+    char *const Ks = lds_dyn, *const Vs = lds_dyn + kStages * kTileBytes;
     __shared__ int wg_lo[kWaves], wg_hi[kWaves];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -123,13 +124,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         wg_hi[wave] = w_t1 > w_t0 ? w_t1 : INT32_MIN;
     }
     // LDS starts as zeros so that rows never written hold finite values (0 * stale must stay 0)
-    for (int e = tid; e < 2 * kTileBytes / 16; e += kThreads) {
-        ((u32x4 *)Ks)[e] = u32x4{0, 0, 0, 0};
-        ((u32x4 *)Vs)[e] = u32x4{0, 0, 0, 0};
-    }
+    for (int e = tid; e < 2 * kStages * kTileBytes / 16; e += kThreads) ((u32x4 *)lds_dyn)[e] = u32x4{0, 0, 0, 0};
     __syncthreads();
-    int g_t0 = min(min(wg_lo[0], wg_lo[1]), min(wg_lo[2], wg_lo[3]));
-    int g_t1 = max(max(wg_hi[0], wg_hi[1]), max(wg_hi[2], wg_hi[3]));
+    int g_t0 = INT32_MAX, g_t1 = INT32_MIN;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        g_t0 = min(g_t0, wg_lo[w]);
+        g_t1 = max(g_t1, wg_hi[w]);
+    }
     if (g_t1 <= g_t0) g_t0 = g_t1 = 0;
     {
         int64_t n = g_t1 - g_t0;
@@ -168,16 +170,17 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             for (int e = 0; e < 2; ++e) v_off[dt][e] = (vr + 4 * e) * 256 + (((dt * 4 + vc) ^ swz(vr + 4 * e)) * 16) + vh;
     }
 
-    // ---- tile loads: wave w, instruction i fills LDS rows 16*w + 4*i .. +3; lane -> (row, position).
+    // ---- tile loads: wave w, instruction i fills LDS rows 8*w + 4*i .. +3; lane -> (row, position).
     //      The wave-uniform tile base advances with the loop; the per-lane offsets are loop invariant.
-    uint32_t gk_off[4], gv_off[4];            // element offsets inside a tile
-    int gk_row[4], gv_row[4];
+    constexpr int kLd = kTile / (4 * kWaves);  // load instructions per wave and tile, for K and for V
+    uint32_t gk_off[kLd], gv_off[kLd];        // element offsets inside a tile
+    int gk_row[kLd], gv_row[kLd];
     {
         const int ld_pos = lane & 15, ld_sub = lane >> 4;
         const int64_t k_sl = PAGED ? kD : a.k_sl, v_sl = PAGED ? kD : a.v_sl;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int R = 16 * wave + 4 * i + ld_sub, chunk = ld_pos ^ swz(R);
+        for (int i = 0; i < kLd; ++i) {
+            const int R = 4 * kLd * wave + 4 * i + ld_sub, chunk = ld_pos ^ swz(R);
             gk_row[i] = k_lds_row(R);
             gv_row[i] = R;
             gk_off[i] = (uint32_t)(gk_row[i] * k_sl + chunk * 8);
@@ -191,6 +194,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         v_head = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh;
         ring_row = ((int64_t)g_t0 * kTile) % a.cap;
     }
+    int partial_in_flight = 0;
     auto load_tile = [&](int t, int buf) {
         const bf16_t *kbase, *vbase;
         int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
@@ -209,16 +213,17 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             row_lo = (int)max((int64_t)0, a.j_lo - j0);
             row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
         }
-        char *kdst = Ks + buf * kTileBytes + wave * 4096, *vdst = Vs + buf * kTileBytes + wave * 4096;
+        char *kdst = Ks + buf * kTileBytes + wave * (kLd * 1024), *vdst = Vs + buf * kTileBytes + wave * (kLd * 1024);
         if (row_lo == 0 && row_hi == kTile) {          // the common case: no per-lane predicate
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < kLd; ++i) {
                 load_to_lds16(kbase + gk_off[i], (bf16_t *)(kdst + i * 1024));
                 load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
             }
         } else {
+            partial_in_flight = kStages;          // not every wave issues every load: wait for all of them for a while
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < kLd; ++i) {
                 // rows outside the source keep whatever the buffer held (finite values): their keys are masked
                 if (gk_row[i] >= row_lo && gk_row[i] < row_hi) load_to_lds16(kbase + gk_off[i], (bf16_t *)(kdst + i * 1024));
                 if (gv_row[i] >= row_lo && gv_row[i] < row_hi) load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
@@ -237,9 +242,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     const float scale = a.softmax_scale * 1.4426950408889634f;
     const float lazy = kLazyLog2 / scale;
 
-    auto tile_math = [&](auto buf_c, int t) {
-        constexpr int BUF = decltype(buf_c)::value;
-        const char *kb = Ks + BUF * kTileBytes, *vb = Vs + BUF * kTileBytes;
+    auto tile_math = [&](int buf, int t) {
+        const char *kb = Ks + buf * kTileBytes, *vb = Vs + buf * kTileBytes;
         f32x16 s[2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
@@ -309,6 +313,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                     s[ks][r] = vis ? s[ks][r] : -INFINITY;
                 }
         }
+#ifdef INFLLM_DBG_STAMP_INNER
+        PH_STAMP();
+#endif
         float tmax = -INFINITY;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
@@ -342,6 +349,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                 pw[ks][r >> 1] = pack_bf16x2(p0, p1);
             }
         l_run += psum;
+#ifdef INFLLM_DBG_STAMP_INNER
+        PH_STAMP();
+#endif
         {
             // 4 steps of 16 keys, 4 MFMAs each; the V^T operands of a step are requested from LDS while the
             // MFMAs of the previous step run
@@ -373,24 +383,32 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         }
     };
 
-    if (g_t1 > g_t0) load_tile(g_t0, 0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // kStages - 1 tiles are requested ahead; tile t lives in buffer (t - g_t0) % kStages, and the buffer a
+    // new tile goes to was last read before the previous barrier
+    for (int p = 0; p < kStages - 1; ++p)
+        if (g_t0 + p < g_t1) load_tile(g_t0 + p, p);
+    auto wait_tile = [&](int t) {           // returns once tile t has landed (loads complete in order)
+        const int ahead = min(g_t1 - 1 - t, kStages - 2);       // tiles requested after t
+        if (partial_in_flight > 0 || ahead <= 0) {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else if (ahead == 1) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLd) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * kLd) : "memory");
+        }
+    };
+    if (g_t1 > g_t0) wait_tile(g_t0);
     __syncthreads();
-    // two tiles per trip so that the LDS buffer index is a compile-time constant; a tile is loaded into the
-    // buffer that was last read before the previous barrier, and lands while the current tile is computed
-    for (int t = g_t0; t < g_t1; t += 2) {
+    for (int t = g_t0; t < g_t1; ++t) {
+        const int buf = (t - g_t0) % kStages;
         PH_STAMP();
-        if (t + 1 < g_t1) load_tile(t + 1, 1);
+        if (t + kStages - 1 < g_t1) load_tile(t + kStages - 1, (buf + kStages - 1) % kStages);
+        if (partial_in_flight > 0) --partial_in_flight;
         PH_STAMP();
-        if (t >= w_t0 && t < w_t1) tile_math(IntC<0>{}, t);          // wave-uniform; barriers stay outside
+        if (t >= w_t0 && t < w_t1) tile_math(buf, t);          // wave-uniform; barriers stay outside
         PH_STAMP();
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (t + 1 < g_t1) wait_tile(t + 1);
         PH_STAMP();
-        __syncthreads();
-        if (t + 1 >= g_t1) break;
-        if (t + 2 < g_t1) load_tile(t + 2, 0);
-        if (t + 1 >= w_t0 && t + 1 < w_t1) tile_math(IntC<1>{}, t + 1);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
@@ -457,9 +475,16 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
     const int G = a->H / a->Hkv;
     const int n_tasks = ((a->Lq + kQTile - 1) / kQTile) * G;
     dim3 grid((n_tasks + kWaves - 1) / kWaves, a->B * a->Hkv, a->nsplit);
+    constexpr size_t lds_bytes = 2 * kStages * kTileBytes;
+    static bool lds_set[2] = {false, false};           // dynamic LDS above 64 KiB must be enabled once per kernel
     if (a->d_pages) {
         INFLLM_REQUIRE(a->n_pages >= 0, "attn_stage: negative page count");
-        hipLaunchKernelGGL(attn_stage_kernel<true>, grid, dim3(kThreads), 0, (hipStream_t)stream, *a);
+        if (!lds_set[1]) {
+            hipError_t e = hipFuncSetAttribute((const void *)attn_stage_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
+            lds_set[1] = true;
+        }
+        hipLaunchKernelGGL(attn_stage_kernel<true>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a);
     } else {
         INFLLM_REQUIRE(a->j_hi <= a->j_lo || (a->d_k && a->d_v), "attn_stage: null k / v pointer");
         INFLLM_REQUIRE(a->cap > 0 && a->cap % kTile == 0, "attn_stage: cap %lld is not a positive multiple of %d",
@@ -469,7 +494,12 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
         INFLLM_REQUIRE(a->mask >= 0 && a->mask <= 2, "attn_stage: unknown mask %d", a->mask);
         INFLLM_REQUIRE((a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8 | a->v_sl % 8 | a->v_sh % 8 | a->v_sb % 8) == 0,
                        "attn_stage: k/v strides must be multiples of 8");
-        hipLaunchKernelGGL(attn_stage_kernel<false>, grid, dim3(kThreads), 0, (hipStream_t)stream, *a);
+        if (!lds_set[0]) {
+            hipError_t e = hipFuncSetAttribute((const void *)attn_stage_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
+            lds_set[0] = true;
+        }
+        hipLaunchKernelGGL(attn_stage_kernel<false>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a);
     }
     INFLLM_CHECK_LAUNCH("attn_stage");
     return 0;

@@ -53,8 +53,8 @@ struct Layer {
 
 int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
     const int G = d.H / d.Hkv;
-    const int wgs = (((n_queries + 31) / 32) * G + 3) / 4 * d.Hkv * d.B;
-    int want = (2 * d.num_cus + wgs - 1) / wgs;
+    const int wgs = (((n_queries + 31) / 32) * G + 7) / 8 * d.Hkv * d.B;      // 8 wave tasks per workgroup
+    int want = (d.num_cus + wgs - 1) / wgs;                                      // one workgroup per CU (LDS bound)
     int cap = n_tiles / 8;
     int s = want < d.max_splits ? want : d.max_splits;
     if (s > cap) s = cap;
