@@ -436,6 +436,67 @@ class ContextManager:
             out = out.view(batch_size, heads, input_length, -1)
         return out
 
+    # ------------------------------------------------------- state in / out
+    # The reference keeps its state only in the live object (SURVEY appendix B lists the fields); these two
+    # methods let a harness start from a prepared memory (e.g. 8192 units with representatives) or resume.
+    def export_state(self):
+        """Snapshot after an append(): everything a fresh ContextManager needs to continue the stream."""
+        torch.cuda.synchronize()
+        T, cur, cap = self.length, self.cursor, self.ring_cap
+        rows = torch.arange(cur, T, device=self.device) % cap
+        units = [self.host_unit(u).clone() for u in range(self.num_global_block)]
+        return dict(length=T, n_units=self.num_global_block, init_len=self.init_len,
+                    tail_k=self.ring_k_raw[:, :, rows].clone(), tail_v=self.ring_v[:, :, rows].clone(),
+                    tail_score=self.ring_score[:, :, rows].clone(),
+                    init_k=self.init_kv[:, 0, :, :self.init_len].clone(), init_v=self.init_kv[:, 1, :, :self.init_len].clone(),
+                    units=torch.stack(units) if units else None,
+                    reps=self.reps[:, :self.num_global_block].clone())
+
+    def load_state(self, state):
+        """Start from a prepared memory.  ``state``: length T; tail_k/tail_v [B,Hkv,T-cursor,D] (un-rotated,
+        the tokens not carved yet, which include the local window); tail_score [B,H,T-cursor] fp32 or None;
+        init_k/init_v [B,Hkv,init_len,D]; units [n_units,B,2,Hkv,bs,D] (any device) or None; reps
+        [B,n_units,H*D].  The counts must satisfy the stream's closed forms (context_manager.py:614-679):
+        init_len = min(n_init, max(T-n_local, 0)), n_units = max(0, (T-n_init-n_local)//block_size)."""
+        from .. import ops
+        assert not self.initialized and self.length == 0, "load_state needs a fresh ContextManager"
+        tail_k, tail_v = state["tail_k"], state["tail_v"]
+        T = int(state["length"])
+        B, Hkv, n_tail, D = tail_k.shape
+        reps = state["reps"]
+        H = reps.shape[2] // D if reps is not None and reps.numel() else state["num_heads"]
+        init_len = min(self.n_init, max(T - self.n_local, 0))
+        n_units = max(0, (T - self.n_init - self.n_local) // self.block_size)
+        cursor = init_len + n_units * self.block_size
+        assert n_tail == T - cursor, f"tail holds {n_tail} tokens, the stream state needs {T - cursor}"
+        assert state["init_k"].shape[2] == init_len and (n_units == 0 or state["units"].shape[0] == n_units)
+        q_like = torch.empty((B, H, 1, D), dtype=torch.bfloat16, device=tail_k.device)
+        self._init(q_like, tail_k[:, :, :1])
+        self._bind_reps()
+        self.length, self.cursor, self.init_len = T, cursor, init_len
+        if init_len:
+            self.init_kv[:, 0, :, :init_len] = state["init_k"]
+            self.init_kv[:, 1, :, :init_len] = state["init_v"]
+        if n_units:
+            self._grow_reps(n_units) if n_units > self.reps.shape[1] else None
+            self.reps[:, :n_units] = reps
+            for u in range(n_units):
+                self._host_unit_addr(u)                        # allocates the pinned chunk
+                self.host_unit(u).copy_(state["units"][u])
+            self.num_global_block = n_units
+        # tail -> rings (RoPE at the absolute positions) in pieces of one execution block
+        zq = torch.zeros((B, H, self.exc_block_size, D), dtype=torch.bfloat16, device=self.device)
+        for st in range(0, n_tail, self.exc_block_size):
+            n = min(self.exc_block_size, n_tail - st)
+            ops.ingest(zq[:, :, :n], tail_k[:, :, st:st + n], tail_v[:, :, st:st + n], cursor + st, self.n_local - 1,
+                       self.inv_freq, float(self.position_embedding.distance_scale), self.ring_k_raw, self.ring_k_rot,
+                       self.ring_v, self.ring_score, self.q_loc[0], self.q_glb[0])
+        if state.get("tail_score") is not None:
+            rows = torch.arange(cursor, T, device=self.device) % self.ring_cap
+            self.ring_score[:, :, rows] = state["tail_score"].to(torch.float32)
+        torch.cuda.synchronize()
+        return self
+
     # ----------------------------------------------------------------- tracing
     def trace_repr_indices(self):
         """{unit: int tensor [B, H, repr_topk]} of the keys chosen as representatives (needs record_trace)."""

@@ -155,6 +155,37 @@ def test_call_splitting_cache_size_and_side_stream_do_not_change_results():
     assert torch.equal(ref, fifo)
 
 
+def test_state_export_and_injection_resume_the_stream_exactly():
+    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
+    T0, T1 = 900, 333
+    q, k, v = _stream(T0 + T1, 8, 2, 13)
+    full, cm1 = _run_gpu(q, k, v, [T0, T1], 1e4, **SMALL)
+    _, cm_a = _run_gpu(q[:, :, :T0], k[:, :, :T0], v[:, :, :T0], [T0], 1e4, **SMALL)
+    state = cm_a.export_state()
+    assert state["n_units"] == (T0 - SMALL["n_init"] - SMALL["n_local"]) // SMALL["block_size"]
+    assert torch.equal(state["init_k"].cpu(), k[:, :, :SMALL["n_init"]])
+    assert torch.equal(state["tail_k"].cpu(), k[:, :, T0 - state["tail_k"].shape[2]:T0])
+    u3 = state["units"][3]                                    # unit 3 = tokens [n_init + 3*bs, n_init + 4*bs)
+    lo = SMALL["n_init"] + 3 * SMALL["block_size"]
+    assert torch.equal(u3[0, 0], k[0, :, lo:lo + SMALL["block_size"]]) and torch.equal(u3[0, 1], v[0, :, lo:lo + SMALL["block_size"]])
+    rope = RotaryEmbeddingESM(D, base=1e4, device="cuda")
+    cm_b = ContextManager(rope, SMALL["n_init"], SMALL["n_local"], SMALL["block_size"], SMALL["max_cached_block"],
+                          SMALL["topk"], SMALL["exc_block_size"], None, False, SMALL["repr_topk"]).load_state(state)
+    assert cm_b.length == T0 and cm_b.num_global_block == state["n_units"]
+    sl = slice(T0, T0 + T1)
+    qd, kd, vd = q[:, :, sl].cuda(), k[:, :, sl].cuda(), v[:, :, sl].cuda()
+    resumed = cm_b.append(qd, kd, vd, qd, kd, vd).cpu()
+    assert torch.equal(resumed, full[:, :, sl])
+    assert cm_b.length == T0 + T1 == cm1.length and cm_b.num_global_block == cm1.num_global_block
+
+
+def test_decode_steps_follow_oracle():
+    """Single-token appends over a prepared memory (the decode shape): retrieval, fetch and attention per step."""
+    calls = [1200] + [1] * 48
+    cm, ora, fol = _compare(sum(calls), calls, H=8, Hkv=2, base=1e4, seed=21, **SMALL)
+    assert cm.stats["blocks"] == len(ora.block_trace)
+
+
 def test_attention_type_forward_contract():
     """ATTN_FORWRAD['inf-llm'] closure: projections in, (output, ContextManager) out (inf_llm.py:20-77)."""
     from infllm_amd.attention import ATTN_FORWRAD, ContextManager, RotaryEmbeddingESM
