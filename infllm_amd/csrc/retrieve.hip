@@ -14,7 +14,7 @@ __device__ __forceinline__ float wave_sum(float x) {
 }
 
 // ---------------------------------------------------------------- unit scores (GEMV)
-// one wave per representative row; the mean query sits in LDS as fp32
+// Generic shape: one wave per representative row; the mean query sits in LDS as fp32.
 __global__ __launch_bounds__(256) void unit_scores_kernel(const bf16_t *reps, int64_t rep_stride, int N, int C,
                                                           const float *qbar, float *scores) {
     extern __shared__ float qs[];
@@ -39,6 +39,76 @@ __global__ __launch_bounds__(256) void unit_scores_kernel(const bf16_t *reps, in
         acc = wave_sum(acc);
         if (lane == 0) scores[n] = acc;
     }
+}
+
+// Rows of CPL*512 elements: a lane owns CPL 16-byte chunks of every row and keeps its slice of the mean
+// query in registers, so the row loop is nothing but CPL independent loads followed by FMAs.  The first
+// row's loads are issued before the query is staged, and a wave walks its rows with a fixed stride so
+// that all waves of the chip stream disjoint rows at once.
+template <int CPL, int ROWS>
+__global__ __launch_bounds__(256) void unit_scores_rows_kernel(const bf16_t *reps, int64_t rep_stride, int N,
+                                                                const float *qbar, float *scores) {
+    extern __shared__ float qs[];
+    constexpr int C = CPL * 512;
+    const int lane = threadIdx.x & 63;
+    const int waves_per_wg = blockDim.x >> 6;
+    const int n_waves = gridDim.x * waves_per_wg;
+    int n = blockIdx.x * waves_per_wg + (threadIdx.x >> 6);     // rows n, n + n_waves, ... belong to this wave
+    u32x4 w[ROWS][CPL];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+        if (n + r * n_waves < N) {
+            const bf16_t *row = reps + (int64_t)(n + r * n_waves) * rep_stride + lane * 8;
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) w[r][j] = __builtin_nontemporal_load((const u32x4 *)(row + j * 512));
+        }
+    for (int e = threadIdx.x * 4; e < C; e += blockDim.x * 4) *(f32x4 *)(qs + e) = *(const f32x4 *)(qbar + e);
+    __syncthreads();
+    float q[CPL][8];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) {
+        const f32x4 lo = *(const f32x4 *)(qs + j * 512 + lane * 8), hi = *(const f32x4 *)(qs + j * 512 + lane * 8 + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) q[j][i] = lo[i], q[j][4 + i] = hi[i];
+    }
+    while (n < N) {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const int cur = n + r * n_waves;
+            if (cur >= N) break;
+            float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc0 += bf16_bits_to_f32(w[r][j][i] & 0xffffu) * q[j][2 * i];
+                    acc1 += bf16_bits_to_f32(w[r][j][i] >> 16) * q[j][2 * i + 1];
+                }
+            }
+            const int nxt = cur + ROWS * n_waves;
+            if (nxt < N) {
+                const bf16_t *row = reps + (int64_t)nxt * rep_stride + lane * 8;
+#pragma unroll
+                for (int j = 0; j < CPL; ++j) w[r][j] = __builtin_nontemporal_load((const u32x4 *)(row + j * 512));
+            }
+            const float acc = wave_sum(acc0 + acc1);
+            if (lane == 0) scores[cur] = acc;
+        }
+        n += ROWS * n_waves;
+    }
+}
+
+// At most 512 workgroups (two per CU, all resident at once: a second round of workgroups costs more than
+// it gains); long tables keep two rows per wave in flight.
+template <int CPL>
+void launch_unit_scores_rows(const bf16_t *reps, int64_t rep_stride, int N, const float *qbar, float *scores, hipStream_t st) {
+    constexpr int kRowsDeep = CPL <= 8 ? 2 : 1;
+    const bool deep = kRowsDeep > 1 && N >= 4096;
+    const int per_wg = 4 * (deep ? kRowsDeep : 1);
+    int wgs = (N + per_wg - 1) / per_wg;
+    if (wgs > 512) wgs = 512;
+    auto kern = deep ? unit_scores_rows_kernel<CPL, kRowsDeep> : unit_scores_rows_kernel<CPL, 1>;
+    hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), (size_t)CPL * 512 * sizeof(float), st, reps, rep_stride, N, qbar, scores);
 }
 
 // ---------------------------------------------------------------- top-k (radix select)
@@ -121,6 +191,99 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
     }
 }
 
+// Tables of up to 16384 scores: every thread keeps its R consecutive keys in registers, so the scores are read
+// once.  Three digit passes (12, 12 and 8 bits from the top; 4096 bins spread the keys of one binade over
+// many LDS counters) find the key of the k-th largest; a pass whose bucket is wanted whole ends the search.
+// Output contract as above: indices ascending, lowest indices among keys equal to the k-th.
+template <int R>
+__global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *scores, int N, int k, int32_t *idx_out) {
+    __shared__ __align__(16) int hist[4096];
+    __shared__ int wave_tot[kSelThreads / 64];
+    __shared__ uint32_t sh_prefix;
+    __shared__ int sh_need, sh_done;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_valid = min(max(N - tid * R, 0), R);
+    uint32_t key[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) key[j] = j < n_valid ? order_key(scores[tid * R + j]) : 0u;
+
+    uint32_t prefix = 0, pmask = 0;
+    int need = k;
+    bool done = false;
+    for (int p = 0; p < 3 && !done; ++p) {
+        const int shift = p == 0 ? 20 : p == 1 ? 8 : 0;
+        const uint32_t dmask = p == 2 ? 255u : 4095u;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) hist[tid + i * kSelThreads] = 0;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < R; ++j)
+            if (j < n_valid && (key[j] & pmask) == prefix) atomicAdd(&hist[dmask - ((key[j] >> shift) & dmask)], 1);
+        __syncthreads();
+        // bins are stored from the largest digit down; thread t owns bins 4t..4t+3
+        const int h0 = hist[4 * tid], h1 = hist[4 * tid + 1], h2 = hist[4 * tid + 2], h3 = hist[4 * tid + 3];
+        const int s = h0 + h1 + h2 + h3;
+        int incl = s;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += up;
+        }
+        if (lane == 63) wave_tot[wave] = incl;
+        __syncthreads();
+        int excl = incl - s;
+        for (int w = 0; w < kSelThreads / 64; ++w) excl += w < wave ? wave_tot[w] : 0;
+        if (excl < need && excl + s >= need) {                 // exactly one thread holds the bucket of the k-th
+            const int hv[4] = {h0, h1, h2, h3};
+            int e = excl, bin = 0;
+#pragma unroll
+            for (int i = 0; i < 3; ++i)
+                if (e + hv[bin] < need) e += hv[bin], ++bin;
+            sh_prefix = prefix | ((dmask - (uint32_t)(4 * tid + bin)) << shift);
+            sh_need = need - e;
+            sh_done = hv[bin] == need - e;
+        }
+        __syncthreads();
+        prefix = sh_prefix;
+        need = sh_need;
+        done = sh_done != 0;
+        pmask |= dmask << shift;
+    }
+    // keys above the prefix are all taken; of those equal to it (under pmask) the first `need` by index
+    int cg = 0, ce = 0;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const uint32_t mk = key[j] & pmask;
+        cg += (j < n_valid && mk > prefix) ? 1 : 0;
+        ce += (j < n_valid && mk == prefix) ? 1 : 0;
+    }
+    const int packed = (ce << 16) | cg;                        // cg < k <= 1024 and ce <= 16384: no carry between the fields
+    int incl = packed;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    __syncthreads();                                           // wave_tot of the last pass fully read
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    int excl = incl - packed;
+    for (int w = 0; w < kSelThreads / 64; ++w) excl += w < wave ? wave_tot[w] : 0;
+    int g_before = excl & 0xffff, e_before = excl >> 16;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        if (j >= n_valid) break;
+        const uint32_t mk = key[j] & pmask;
+        if (mk > prefix) {
+            idx_out[g_before + min(e_before, need)] = tid * R + j;
+            ++g_before;
+        } else if (mk == prefix) {
+            if (e_before < need) idx_out[g_before + e_before] = tid * R + j;
+            ++e_before;
+        }
+    }
+}
+
 // ---------------------------------------------------------------- representative keys
 constexpr int kMaxUnit = 2048;             // largest supported unit (block_size)
 
@@ -181,9 +344,18 @@ extern "C" int infllm_unit_scores(const void *d_reps, int64_t rep_stride, int32_
                    first, count, C);
     INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "unit_scores: row stride %lld", (long long)rep_stride);
     if (count == 0) return 0;
-    const int wgs = count < 4 * 2048 ? (count + 3) / 4 : 2048;
-    hipLaunchKernelGGL(unit_scores_kernel, dim3(wgs), dim3(256), (size_t)C * sizeof(float), (hipStream_t)stream,
-                       (const bf16_t *)d_reps + (int64_t)first * rep_stride, rep_stride, count, C, d_qbar, d_scores + first);
+    const bf16_t *rows = (const bf16_t *)d_reps + (int64_t)first * rep_stride;
+    float *out = d_scores + first;
+    switch (C % 512 == 0 ? C / 512 : 0) {
+#define ROWS_CASE(n) case n: launch_unit_scores_rows<n>(rows, rep_stride, count, d_qbar, out, (hipStream_t)stream); break
+        ROWS_CASE(1); ROWS_CASE(2); ROWS_CASE(4); ROWS_CASE(5); ROWS_CASE(6); ROWS_CASE(8); ROWS_CASE(10); ROWS_CASE(12); ROWS_CASE(16);
+#undef ROWS_CASE
+    default: {
+        const int wgs = count < 4 * 2048 ? (count + 3) / 4 : 2048;
+        hipLaunchKernelGGL(unit_scores_kernel, dim3(wgs), dim3(256), (size_t)C * sizeof(float), (hipStream_t)stream, rows,
+                           rep_stride, count, C, d_qbar, out);
+    }
+    }
     INFLLM_CHECK_LAUNCH("unit_scores");
     return 0;
 }
@@ -191,7 +363,21 @@ extern "C" int infllm_unit_scores(const void *d_reps, int64_t rep_stride, int32_
 extern "C" int infllm_topk(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, void *stream) {
     INFLLM_REQUIRE(d_scores && d_idx, "topk: null pointer");
     INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && k <= 1024, "topk: k=%d with N=%d", k, N);
-    hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, (hipStream_t)stream, d_scores, N, k, d_idx);
+    const hipStream_t st = (hipStream_t)stream;
+    switch (N <= 16384 ? (N + kSelThreads - 1) / kSelThreads : 0) {       // keys per thread
+#define REGS_CASE(r) hipLaunchKernelGGL(topk_regs_kernel<r>, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx); break
+    case 1: REGS_CASE(1);
+    case 2: REGS_CASE(2);
+    case 3: REGS_CASE(3);
+    case 4: REGS_CASE(4);
+    case 5: case 6: REGS_CASE(6);
+    case 7: case 8: REGS_CASE(8);
+    case 9: case 10: REGS_CASE(10);
+    case 11: case 12: REGS_CASE(12);
+    case 13: case 14: case 15: case 16: REGS_CASE(16);
+#undef REGS_CASE
+    default: hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx);
+    }
     INFLLM_CHECK_LAUNCH("topk");
     return 0;
 }

@@ -158,6 +158,11 @@ def score_topk(reps, n, qbar, k, scores, idx):
           "infllm_score_topk")
 
 
+def topk(scores, n, k, idx):
+    """idx[:k] = ascending indices of the k largest of scores[:n] (lowest indices among equal scores)."""
+    check(_lib.load().infllm_topk(scores.data_ptr(), n, k, idx.data_ptr(), _stream()), "infllm_topk")
+
+
 def repr_keys(ring_score, ring_k_raw, t0, bs, n_units, repr_topk, rep_out, rep_sb, rep_su, idx_out=None):
     B, H, cap = ring_score.shape
     Hkv = ring_k_raw.shape[1]

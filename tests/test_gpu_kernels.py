@@ -238,7 +238,8 @@ def test_operator_class_protocol():
 
 
 # ----------------------------------------------------------------- retrieval
-@pytest.mark.parametrize("N,k", [(17, 16), (991, 16), (8192, 16), (5000, 64), (40, 1)])
+@pytest.mark.parametrize("N,k", [(17, 16), (991, 16), (8192, 16), (5000, 64), (40, 1), (8194, 16), (16384, 64), (20000, 16),
+                                 (3000, 1024), (1024, 1024), (2049, 3)])
 def test_score_topk_matches_bruteforce(N, k):
     ops = _ops()
     C = 32 * D
@@ -277,6 +278,22 @@ def test_topk_with_exact_ties_takes_lowest_indices():
     neg = (-reps).cuda()
     ops.score_topk(neg, N, qbar.cuda(), 4, scores, idx)
     assert idx.cpu().tolist()[:4] == [0, 1, 2, 3]
+
+
+@pytest.mark.parametrize("N,k,levels", [(6000, 16, 5), (1000, 100, 3), (12000, 300, 40), (70, 70, 2), (16384, 1, 1),
+                                        (30000, 50, 7)])
+def test_topk_on_heavily_tied_scores_is_the_stable_descending_prefix(N, k, levels):
+    """Few distinct score values (negative, zero and positive): the selection must be the first k of a stable
+    descending sort, returned in ascending index order, whichever digit pass the search stops in."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(N + k)
+    vals = torch.randint(0, levels, (N,), generator=g).float() - levels // 2
+    vals = vals * (1.0 + 2.0 ** -20)                      # differences in the lowest mantissa bits as well
+    scores = vals.cuda()
+    idx = torch.full((k,), -1, dtype=torch.int32, device="cuda")
+    ops.topk(scores, N, k, idx)
+    order = sorted(range(N), key=lambda i: (-float(vals[i]), i))
+    assert idx.cpu().tolist() == sorted(order[:k])
 
 
 @pytest.mark.parametrize("bs,r,H,Hkv", [(128, 4, 32, 8), (8, 2, 4, 2), (100, 1, 3, 3), (64, 64, 2, 1)])
