@@ -155,6 +155,9 @@ def main():
                     help="prefill = the headline 128K-token stream (config 2); decode = config 3 (own JSON line)")
     ap.add_argument("--decode-units", type=int, default=8192)
     ap.add_argument("--decode-steps", type=int, default=256)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="first run three elementwise passes over 256 MiB (reads 256 MiB, writes 256 MiB each): the known-size "
+                         "kernel that hardware byte counters of a profiled run are scaled by")
     ap.add_argument("--max-cached-block", type=int, default=KNOBS["max_cached_block"],
                     help="GPU unit-cache slots (the headline number uses the reference's 32)")
     args = ap.parse_args()
@@ -164,6 +167,13 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.copy_calibration:
+        src = torch.ones((128 << 20,), dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.neg(src, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     if args.workload == "decode":
         decode_workload(args, dev)
         return

@@ -84,14 +84,28 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
     const int G = a.H / a.Hkv;
-    const int b = blockIdx.y / a.Hkv, g = blockIdx.y % a.Hkv;
-    const int split = blockIdx.z;
+    // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  Renumber so that
+    // one XCD runs a contiguous run of ids: the workgroups that share a (kv head, split) K/V range then sit
+    // behind one L2 and that range leaves HBM once instead of once per XCD.
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    {
+        const int gx = gridDim.x, gy = gridDim.y, total = gx * gy * (int)gridDim.z;
+        if ((total & 7) == 0) {
+            const int lin = bx + gx * (by + gy * bz);
+            const int id = (lin & 7) * (total >> 3) + (lin >> 3);
+            bx = id % gx;
+            by = (id / gx) % gy;
+            bz = id / (gx * gy);
+        }
+    }
+    const int b = by / a.Hkv, g = by % a.Hkv;
+    const int split = bz;
     const int n_qtiles = (a.Lq + kQTile - 1) / kQTile;
     const int n_tasks = n_qtiles * G;
 #ifdef INFLLM_PHASES
     long long *ph = (long long *)a.d_lse_part + 1024 * 1024;     // debug build only: stamps beyond the lse partials
     int ph_n = 0;
-    const bool ph_on = blockIdx.x == 3 && blockIdx.y == 1 && blockIdx.z == 1 && tid == 0;
+    const bool ph_on = bx == 3 && by == 1 && bz == 1 && tid == 0;
 #define PH_STAMP() do { if (ph_on && ph_n < 512) ph[ph_n++] = clock64(); } while (0)
 #else
 #define PH_STAMP() do { } while (0)
@@ -99,7 +113,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     PH_STAMP();
 
     // ---- this wave's task and the tiles it needs
-    const int task = blockIdx.x * kWaves + wave;
+    const int task = bx * kWaves + wave;
     const bool live = task < n_tasks;
     const int qt = live ? task / G : 0, hg = live ? task % G : 0;
     const int h = g * G + hg;
