@@ -56,6 +56,13 @@ def run_stream(q, k, v, chunk, timing=False):
     return cm, out
 
 
+# HBM bytes per launch from hardware counters (FETCH_SIZE, WRITE_SIZE; one profiler run per counter, each scaled by
+# what the counter reads for a 256 MiB elementwise pass: x2.0 and x1.0).  The summaries of those runs sit in
+# profiles/*.hbm_bytes.txt; the figures hold for the default geometry only.
+LOCAL_STAGE_HBM_BYTES = int((20207.5 * 2.0 + 46020.4) * 1024)      # steady-state local stage: 39.5 MiB read + 44.9 MiB written
+UNIT_SCORES_HBM_BYTES = int((32868.1 * 2.0 + 64.0) * 1024)         # 8194 x 4096 representatives: 64.2 MiB read
+
+
 def decode_workload(args, dev):
     """BASELINE config 3: 256 single-token steps over a prepared memory of 8192 units (1,048,576 past tokens)
     with precomputed representatives.  Prints its own JSON line; not the headline metric."""
@@ -120,7 +127,7 @@ def decode_workload(args, dev):
         "n_gpus": 1, "steps": steps, "ms_per_step": dt / steps * 1e3, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"config 3: {steps} single-token steps, {N} units x {bs} tokens, topk {topk}, n_local {n_local}, "
                                f"max_cached {KNOBS['max_cached_block']}"},
-        "roofline": {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None,
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": UNIT_SCORES_HBM_BYTES,
                      "kernel": f"unit_scores_kernel ({N} x {H * D} bf16 representatives, {N * H * D * 2 / 2 ** 20:.1f} MiB per retrieval)",
                      "avg_launch_ms": ms},
         "cache": cm.stats}))
@@ -210,7 +217,7 @@ def main():
                                f"n_init128 n_local4096 bs128 topk16 repr_topk4 max_cached{KNOBS['max_cached_block']} lru, GMM keys",
                    "append_chunk": args.chunk},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": LOCAL_STAGE_HBM_BYTES,
                      "kernel": "attn_stage_kernel<false> (local stage, 512 q x 4096 visible keys x 32 heads)",
                      "avg_launch_ms": avg_ms, "launches_timed": len(steady),
                      "global_stage_avg_ms": sum(glob) / max(len(glob), 1)},
