@@ -79,6 +79,12 @@ int infllm_reduce_partials(const float *d_parts, int32_t B, int32_t n_parts, int
  * block j covers rows [j*exc, min((j+1)*exc, n)). */
 int infllm_block_mean(const void *d_q_glb, int32_t B, int32_t H, int32_t n, int32_t exc,
                       float *d_qbar, void *stream);
+/* The same means for a whole chunk of un-rotated input rows q [B,H,n,128] (strides in elements), as
+ * get_batched_topk needs them (context_manager.py:548-612, with the one-angle rotation of :744-746):
+ * d_qbar fp32 [B, n_blocks, H*128] = RoPE(mean of the block's rows, angle glb_pos). */
+int infllm_chunk_qbar(const void *d_q, int64_t q_sb, int64_t q_sh, int64_t q_sl, int32_t B, int32_t H,
+                      int32_t n, int32_t exc, const float *d_inv_freq, double distance_scale,
+                      int64_t glb_pos, float *d_qbar, void *stream);
 
 /* ---------------------------------------------------------------------------
  * One stage of the multi-stage attention (bf16 MFMA flash kernel).
@@ -290,11 +296,14 @@ typedef struct {
     float *d_unit_scores;                             /* [B, >= n_units] */
     int64_t unit_scores_sb;
     const void *d_q_next, *d_k_next, *d_v_next;       /* rows of the next block (same strides), or NULL */
-    int32_t n_next, reserved;
+    int32_t n_next, flags;                            /* INFLLM_NO_RETRIEVAL: the caller supplies the selection */
 } infllm_front_args;
 int infllm_block_front(void *layer, const infllm_front_args *a, void *stream);
 int infllm_layer_wait_topk(void *layer);
 
+/* flags of infllm_front_args / infllm_back_args: skip mean query, unit scores and top-k (the selection was made
+ * elsewhere, e.g. for a whole chunk at once: context_manager.py:548-612, 749-770) */
+enum { INFLLM_NO_RETRIEVAL = 1 };
 typedef struct {
     int32_t n, n_sel;                                 /* queries; selected units per batch row */
     int64_t b0;
@@ -311,11 +320,17 @@ typedef struct {
     int64_t rep_sb, rep_su;
     int32_t *d_repr_idx;                              /* optional [B,n_carve,H,repr_topk] */
     void *const *h_carve_dst;                         /* host [n_carve]: pinned [B,2,Hkv,block_size,128] */
-    int32_t n_units, reserved;                        /* units before this block's carving */
+    int32_t n_units, flags;                           /* units before this block's carving; INFLLM_NO_RETRIEVAL */
     const void *d_reps;                               /* [B, rows, H*128] (rep_sb / rep_su above) */
     float *d_unit_scores;                             /* [B, >= n_units + n_carve] */
     int64_t unit_scores_sb;
+    /* Optional (NULL = off), for cache_strategy "lru-s" (context_manager.py:454-470, 529-543): d_unit_mass
+     * [B,n_sel] fp32, device-visible, receives for every selected unit the sum over heads, queries and the
+     * unit's tokens of the block's final attention probabilities; d_mass_scratch fp32 [B,n_sel,H,block_size].
+     * infllm_layer_wait_mass blocks the host until the last such result is written. */
+    float *d_unit_mass, *d_mass_scratch;
 } infllm_back_args;
+int infllm_layer_wait_mass(void *layer);
 /* Optional: issue the fetch of infllm_block_back ahead of it, as soon as the misses are known (the rest of
  * the host's bookkeeping then overlaps the transfer); infllm_block_back must follow with the same lists. */
 int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_miss_row, const int32_t *h_miss_slot,

@@ -86,7 +86,7 @@ class FrontArgs(C.Structure):
         ("n", c_i32), ("n_units", c_i32), ("b0", c_i64),
         ("d_reps", c_vp), ("rep_sb", c_i64), ("rep_su", c_i64),
         ("d_unit_scores", c_vp), ("unit_scores_sb", c_i64),
-        ("d_q_next", c_vp), ("d_k_next", c_vp), ("d_v_next", c_vp), ("n_next", c_i32), ("reserved", c_i32),
+        ("d_q_next", c_vp), ("d_k_next", c_vp), ("d_v_next", c_vp), ("n_next", c_i32), ("flags", c_i32),
     ]
 
 
@@ -100,9 +100,12 @@ class BackArgs(C.Structure):
         ("init_take", c_i32), ("n_carve", c_i32),
         ("d_rep_out", c_vp), ("rep_sb", c_i64), ("rep_su", c_i64),
         ("d_repr_idx", c_vp), ("h_carve_dst", c_vp),
-        ("n_units", c_i32), ("reserved", c_i32), ("d_reps", c_vp), ("d_unit_scores", c_vp), ("unit_scores_sb", c_i64),
+        ("n_units", c_i32), ("flags", c_i32), ("d_reps", c_vp), ("d_unit_scores", c_vp), ("unit_scores_sb", c_i64),
+        ("d_unit_mass", c_vp), ("d_mass_scratch", c_vp),
     ]
 
+
+NO_RETRIEVAL = 1            # INFLLM_NO_RETRIEVAL
 
 # name -> (restype, argtypes); every symbol include/infllm_hip.h declares
 SYMBOLS = {
@@ -111,6 +114,7 @@ SYMBOLS = {
     "infllm_ingest": (c_i32, [C.POINTER(IngestArgs), c_vp]),
     "infllm_reduce_partials": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_f32, c_vp, c_vp]),
     "infllm_block_mean": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
+    "infllm_chunk_qbar": (c_i32, [c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_i32, c_vp, C.c_double, c_i64, c_vp, c_vp]),
     "infllm_attn_stage": (c_i32, [C.POINTER(AttnArgs), c_vp]),
     "infllm_attn_merge": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
     "infllm_local_score": (c_i32, [C.POINTER(ScoreArgs), c_vp]),
@@ -127,6 +131,7 @@ SYMBOLS = {
     "infllm_layer_destroy": (c_i32, [c_vp]),
     "infllm_block_front": (c_i32, [c_vp, C.POINTER(FrontArgs), c_vp]),
     "infllm_layer_wait_topk": (c_i32, [c_vp]),
+    "infllm_layer_wait_mass": (c_i32, [c_vp]),
     "infllm_block_fetch": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "infllm_block_back": (c_i32, [c_vp, C.POINTER(BackArgs), c_vp, c_vp]),
     "infllm_layer_flush": (c_i32, [c_vp, c_vp]),

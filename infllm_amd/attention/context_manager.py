@@ -55,6 +55,7 @@ class CachePolicy:
         self.clock = 0
         self.slot_of = {}
         self.free = list(range(capacity - 1, -1, -1))
+        self.evicted_log = None             # set to a list to record the evictions of every block
 
     def touch(self, selected):
         """Returns (misses, evicted) and updates values; slots of evicted units are freed."""
@@ -86,6 +87,8 @@ class CachePolicy:
         assert len(cached) <= self.capacity, "topk exceeds max_cached_block"
         for b in misses:
             self.slot_of[b] = self.free.pop()
+        if self.evicted_log is not None:
+            self.evicted_log.append(evicted)
         return misses, evicted
 
     def add_scores(self, units, unit_scores):
@@ -104,9 +107,9 @@ class ContextManager:
         if faiss:
             raise NotImplementedError("the faiss representative store is not available in this build")
         if cache_strategy == "lru-s":
-            raise NotImplementedError("cache_strategy='lru-s' needs the per-unit global score kernel (not built yet)")
+            assert score_decay is not None, "cache_strategy='lru-s' needs score_decay"
         if chunk_topk_calc is not None:
-            raise NotImplementedError("chunk_topk_calc is not implemented yet")
+            assert chunk_topk_calc >= exc_block_size, "chunk_topk_calc must cover at least one execution block"
         self.length = 0
         self.position_embedding = position_embedding
         self.n_init, self.n_local = n_init, n_local
@@ -125,6 +128,7 @@ class ContextManager:
         self.stats = dict(blocks=0, hits=0, misses=0, evictions=0)
         self._layer = None
         self._timing_cap = 0
+        self._mass_units = None                # lru-s: selections of the block whose unit masses are still on the device
         global _SIDE_STREAM
         if async_global_stream and _SIDE_STREAM is None and torch.cuda.is_available():
             _SIDE_STREAM = torch.cuda.Stream()
@@ -170,6 +174,9 @@ class ContextManager:
         self.unit_scores = torch.empty((B, 16), **f32)
         self.host_chunks, self._host_base, self._host_dev_base = [], [], []
         self.policy = [CachePolicy(self.max_cached_block, self.cache_strategy, self.score_decay) for _ in range(B)]
+        if self.record_trace:
+            for pol in self.policy:
+                pol.evicted_log = []
         self.cursor = 0
         self.init_len = 0
         self.num_global_block = 0
@@ -237,6 +244,14 @@ class ContextManager:
         ba.h_miss_row, ba.h_miss_slot = ctypes.addressof(self._miss_row), ctypes.addressof(self._miss_slot)
         ba.h_miss_unit = ctypes.addressof(self._miss_unit)
         ba.h_miss_src, ba.h_carve_dst = ctypes.addressof(self._miss_src), ctypes.addressof(self._carve_dst)
+        if self.cache_strategy == "lru-s":
+            # context_manager.py:454-470: per-unit attention mass of every block, read back by the host
+            self.mass_host = torch.zeros((B, max(topk, 1)), dtype=torch.float32, pin_memory=True)
+            self.mass_scratch = torch.empty((B, max(topk, 1), H, bs), **f32)
+            ba.d_unit_mass = self._lib.infllm_host_device_pointer(self.mass_host.data_ptr())
+            if not ba.d_unit_mass:
+                raise _lib.InfLLMHipError("pinned host memory is not device-mapped: " + (self._lib.infllm_last_error() or b"").decode())
+            ba.d_mass_scratch = self.mass_scratch.data_ptr()
         self._fa_ref, self._ba_ref = ctypes.byref(self._fa), ctypes.byref(self._ba)
         self.initialized = True
 
@@ -280,7 +295,7 @@ class ContextManager:
         return [(ms[i], nq[i], nk[i]) for i in range(n)]
 
     # -------------------------------------------------------- one exec block
-    def _block(self, st, n, out_ptr, n_next):
+    def _block(self, st, n, out_ptr, n_next, preselected=None):
         lib, layer, fa, ba = self._lib, self._layer, self._fa, self._ba
         B, bs, topk = self.num_units, self.block_size, self.topk
         b0 = self.length + st
@@ -291,6 +306,7 @@ class ContextManager:
         fa.d_v = self._v_ptr + st * self._v_step
         fa.n, fa.n_units, fa.b0 = n, N, b0
         fa.n_next = n_next
+        fa.flags = ba.flags = _lib.NO_RETRIEVAL if preselected is not None else 0
         if n_next:
             fa.d_q_next = fa.d_q + n * self._q_step
             fa.d_k_next = fa.d_k + n * self._k_step
@@ -299,7 +315,9 @@ class ContextManager:
         if rc:
             check(rc, "infllm_block_front")
         # ---- retrieval result (context_manager.py:366-383)
-        if N <= topk:
+        if preselected is not None:                          # chosen for the whole chunk (context_manager.py:381-382)
+            selected = preselected
+        elif N <= topk:
             selected = [list(range(N))] * B
         else:
             rc = lib.infllm_layer_wait_topk(layer)           # the one host wait of a block
@@ -310,6 +328,12 @@ class ContextManager:
         n_sel = len(selected[0])
         n_miss = 0
         stats = self.stats
+        if self._mass_units is not None:                     # lru-s: the previous block's masses decide this eviction
+            check(lib.infllm_layer_wait_mass(layer), "infllm_layer_wait_mass")
+            masses = self.mass_host.tolist()
+            for u in range(B):
+                self.policy[u].add_scores(self._mass_units[u], masses[u][:len(self._mass_units[u])])
+            self._mass_units = None
         for u in range(B):
             pol = self.policy[u]
             misses, evicted = pol.touch(selected[u])
@@ -358,6 +382,8 @@ class ContextManager:
         rc = lib.infllm_block_back(layer, self._ba_ref, self._main_raw, self._copy_raw)
         if rc:
             check(rc, "infllm_block_back")
+        if self.cache_strategy == "lru-s" and n_sel:
+            self._mass_units = selected
         if self.record_trace:
             self.trace_blocks.append(dict(b0=b0, b1=b1, selected=[sorted(s) for s in selected], n_units=N, init_len=init_len))
             if c:
@@ -366,6 +392,28 @@ class ContextManager:
         self.init_len = init_len + take
         self.cursor = cursor + take + c * bs
         self.num_global_block = N + c
+
+    def _chunk_topk(self, q, c0, c1):
+        """Selections of every execution block of q[:, :, c0:c1] against the units that exist now
+        (get_batched_topk, context_manager.py:548-612); one host wait for the whole chunk."""
+        B, N, topk, exc = self.num_units, self.num_global_block, self.topk, self.exc_block_size
+        n_blocks = -(-(c1 - c0) // exc)
+        if N <= topk:
+            return [[list(range(N))] * B for _ in range(n_blocks)]
+        C = self.unit_size * self.dim_head
+        qbar = torch.empty((B, n_blocks, C), dtype=torch.float32, device=self.device)
+        check(self._lib.infllm_chunk_qbar(q.data_ptr() + c0 * q.stride(2) * 2, q.stride(0), q.stride(1), q.stride(2), B,
+                                          self.unit_size, c1 - c0, exc, self.inv_freq.data_ptr(),
+                                          float(self.position_embedding.distance_scale), self.n_local - 1,
+                                          qbar.data_ptr(), self._main_raw), "infllm_chunk_qbar")
+        scores = torch.empty((N,), dtype=torch.float32, device=self.device)
+        idx = torch.empty((n_blocks, B, topk), dtype=torch.int32, device=self.device)
+        for j in range(n_blocks):
+            for u in range(B):
+                check(self._lib.infllm_score_topk(self.reps[u].data_ptr(), self.reps.stride(1), N, C, qbar[u, j].data_ptr(),
+                                                  topk, scores.data_ptr(), idx[j, u].data_ptr(), self._main_raw),
+                      "infllm_score_topk")
+        return idx.cpu().tolist()
 
     def _grow_reps(self, need):
         B, N = self.num_units, self.num_global_block
@@ -427,9 +475,23 @@ class ContextManager:
         self._copy_raw = _SIDE_STREAM.cuda_stream if self.async_global_stream else self._main_raw
         out_ptr, out_step = out.data_ptr(), out.stride(2) * 2
         exc = self.exc_block_size
+        use_chunks = self.chunk_topk_calc is not None and input_length > 1      # context_manager.py:749-760
+        if use_chunks:
+            per_chunk = self.chunk_topk_calc // exc
+            cuts = [i * exc for i in range(0, input_length // exc + 1, per_chunk)]
+            if cuts[-1] < input_length:
+                cuts.append(input_length)
+            cut_i, plan, plan_pos = -1, None, 0
         for st in range(0, input_length, exc):
             n = min(exc, input_length - st)
-            self._block(st, n, out_ptr + st * out_step, min(exc, input_length - st - n))
+            chosen = None
+            if use_chunks:
+                if cuts[cut_i + 1] < st + n:
+                    cut_i += 1
+                    plan, plan_pos = self._chunk_topk(q, cuts[cut_i], cuts[cut_i + 1]), 0
+                chosen = plan[plan_pos]
+                plan_pos += 1
+            self._block(st, n, out_ptr + st * out_step, min(exc, input_length - st - n), chosen)
         self.length += input_length
         check(self._lib.infllm_layer_flush(self._layer, self._copy_raw), "infllm_layer_flush")
         if self.perhead:

@@ -169,6 +169,49 @@ __global__ __launch_bounds__(kMeanThreads) void block_mean_kernel(const bf16_t *
     }
 }
 
+// Mean global query of every execution block of a chunk, straight from the un-rotated input rows: the global
+// query is rotated by ONE angle (rope.py:93-104), and a rotation is linear, so the mean is taken first (fp32)
+// and rotated once.  One workgroup per (block, head, batch row).
+__global__ __launch_bounds__(kMeanThreads) void chunk_qbar_kernel(const bf16_t *q, int64_t q_sb, int64_t q_sh, int64_t q_sl,
+                                                                 int H, int n, int exc, const float *inv_freq,
+                                                                 double distance_scale, int64_t glb_pos, float *qbar,
+                                                                 int n_blocks) {
+    __shared__ float2 part[kMeanThreads / 64][64];
+    __shared__ float mean[kD];
+    const int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int r0 = blk * exc, r1 = min(r0 + exc, n);
+    const bf16_t *src = q + (int64_t)b * q_sb + (int64_t)h * q_sh;
+    float s0 = 0.f, s1 = 0.f;
+    for (int r = r0 + grp; r < r1; r += kMeanThreads / 64) {
+        uint32_t w = *(const uint32_t *)(src + (int64_t)r * q_sl + lane * 2);
+        s0 += bf16_bits_to_f32(w & 0xffffu);
+        s1 += bf16_bits_to_f32(w >> 16);
+    }
+    part[grp][lane] = make_float2(s0, s1);
+    __syncthreads();
+    if (grp == 0) {
+        float t0 = 0.f, t1 = 0.f;
+        for (int g = 0; g < kMeanThreads / 64; ++g) {
+            t0 += part[g][lane].x;
+            t1 += part[g][lane].y;
+        }
+        const float inv = 1.f / (float)(r1 - r0);
+        mean[lane * 2] = t0 * inv;
+        mean[lane * 2 + 1] = t1 * inv;
+    }
+    __syncthreads();
+    if (threadIdx.x < kD / 2) {
+        const int f = threadIdx.x;
+        double sn, cs;
+        sincos((double)glb_pos * distance_scale * (double)inv_freq[f], &sn, &cs);
+        const float c = (float)cs, sgn = (float)sn, lo = mean[f], hi = mean[f + kD / 2];
+        float *dst = qbar + (((int64_t)b * n_blocks + blk) * H + h) * kD;
+        dst[f] = lo * c - hi * sgn;
+        dst[f + kD / 2] = hi * c + lo * sgn;
+    }
+}
+
 __global__ __launch_bounds__(256) void gather_rows_kernel(const bf16_t *ring, int64_t ring_cap, int Hkv, int64_t t0,
                                                           int n, int unit_rows, bf16_t *out, int64_t out_sb,
                                                           int64_t out_su, int64_t out_sh) {
@@ -222,6 +265,19 @@ extern "C" int infllm_block_mean(const void *d_q_glb, int32_t B, int32_t H, int3
     hipLaunchKernelGGL(block_mean_kernel, dim3(n_blocks, H, B), dim3(kMeanThreads), 0, (hipStream_t)stream,
                        (const bf16_t *)d_q_glb, H, n, exc, d_qbar, n_blocks);
     INFLLM_CHECK_LAUNCH("block_mean");
+    return 0;
+}
+
+extern "C" int infllm_chunk_qbar(const void *d_q, int64_t q_sb, int64_t q_sh, int64_t q_sl, int32_t B, int32_t H, int32_t n,
+                                 int32_t exc, const float *d_inv_freq, double distance_scale, int64_t glb_pos, float *d_qbar,
+                                 void *stream) {
+    INFLLM_REQUIRE(d_q && d_inv_freq && d_qbar, "chunk_qbar: null pointer");
+    INFLLM_REQUIRE(B > 0 && H > 0 && n > 0 && exc > 0, "chunk_qbar: bad sizes B=%d H=%d n=%d exc=%d", B, H, n, exc);
+    INFLLM_REQUIRE(q_sl % 2 == 0 && q_sh % 2 == 0 && q_sb % 2 == 0 && (uintptr_t)d_q % 4 == 0, "chunk_qbar: q rows must be 4-byte aligned");
+    const int n_blocks = (n + exc - 1) / exc;
+    hipLaunchKernelGGL(chunk_qbar_kernel, dim3(n_blocks, H, B), dim3(kMeanThreads), 0, (hipStream_t)stream, (const bf16_t *)d_q,
+                       q_sb, q_sh, q_sl, H, n, exc, d_inv_freq, distance_scale, glb_pos, d_qbar, n_blocks);
+    INFLLM_CHECK_LAUNCH("chunk_qbar");
     return 0;
 }
 

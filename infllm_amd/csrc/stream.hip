@@ -34,6 +34,8 @@ struct Layer {
         std::vector<void *> dst;
     } off;
     int page_cur = 0, carve_cur = 0;
+    hipEvent_t mass_done = nullptr;
+    bool mass_pending = false;
     bool has_global = false;
     bool topk_pending = false;
     int slot = 0;                         // workspace slot written last
@@ -50,6 +52,21 @@ struct Layer {
         hipError_t e_ = (call);                                                         \
         if (e_ != hipSuccess) return infllm_fail(-2, "%s: %s", what, hipGetErrorString(e_)); \
     } while (0)
+
+// out[b, i] = sum of the `count` floats at scratch[(b * n_sel + i) * count ...]: the attention mass of one selected unit
+// (context_manager.py:457-460: sum over the unit's tokens, then over the heads)
+__global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, int count, float *out) {
+    __shared__ float red[4];
+    const int idx = blockIdx.y * gridDim.x + blockIdx.x;
+    const float *src = scratch + (int64_t)idx * count;
+    float acc = 0.f;
+    for (int e = threadIdx.x; e < count; e += 256) acc += src[e];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) out[idx] = (red[0] + red[1]) + (red[2] + red[3]);
+}
 
 int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
     const int G = d.H / d.Hkv;
@@ -204,7 +221,8 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
     bool ok = hipEventCreateWithFlags(&L->topk_done, hipEventDisableTiming) == hipSuccess &&
               hipEventCreateWithFlags(&L->global_done, hipEventDisableTiming) == hipSuccess &&
               hipEventCreateWithFlags(&L->fetch_done, hipEventDisableTiming) == hipSuccess &&
-              hipEventCreateWithFlags(&L->carve_ready, hipEventDisableTiming) == hipSuccess;
+              hipEventCreateWithFlags(&L->carve_ready, hipEventDisableTiming) == hipSuccess &&
+              hipEventCreateWithFlags(&L->mass_done, hipEventDisableTiming) == hipSuccess;
     L->page_evt.resize(d.page_slots, nullptr);
     L->carve_evt.resize(d.carve_slots, nullptr);
     L->page_busy.assign(d.page_slots, 0);
@@ -222,7 +240,7 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
 extern "C" int infllm_layer_destroy(void *layer) {
     if (!layer) return 0;
     Layer *L = (Layer *)layer;
-    for (hipEvent_t e : {L->topk_done, L->global_done, L->fetch_done, L->carve_ready})
+    for (hipEvent_t e : {L->topk_done, L->global_done, L->fetch_done, L->carve_ready, L->mass_done})
         if (e) (void)hipEventDestroy(e);
     for (hipEvent_t e : L->page_evt)
         if (e) (void)hipEventDestroy(e);
@@ -349,7 +367,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     // ---- this block's prologue and retrieval, unless the previous block prepared them
     if (!(L->prepared && L->prepared_b0 == a->b0 && L->prepared_n == a->n)) {
         L->slot ^= 1;
-        const bool retrieve = a->n_units > d.topk;
+        const bool retrieve = a->n_units > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL);
         rc = run_ingest(L, a, a->d_q, a->d_k, a->d_v, a->n, a->b0, L->slot, retrieve, stream);
         if (rc) return rc;
         L->topk_pending = false;
@@ -390,7 +408,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
         L->slot ^= 1;
         rc = run_ingest(L, a, a->d_q_next, a->d_k_next, a->d_v_next, a->n_next, b1, L->slot, true, stream);
         if (rc) return rc;
-        if (a->n_units > 0) {
+        if (a->n_units > 0 && !(a->flags & INFLLM_NO_RETRIEVAL)) {
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
             rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->slot, stream);
             if (rc) return rc;
@@ -408,6 +426,15 @@ extern "C" int infllm_layer_wait_topk(void *layer) {
     if (!L->topk_pending) return 0;
     HIP_OK(hipEventSynchronize(L->topk_done), "layer_wait_topk");
     L->topk_pending = false;
+    return 0;
+}
+
+extern "C" int infllm_layer_wait_mass(void *layer) {
+    INFLLM_REQUIRE(layer, "layer_wait_mass: null layer");
+    Layer *L = (Layer *)layer;
+    if (!L->mass_pending) return 0;
+    HIP_OK(hipEventSynchronize(L->mass_done), "layer_wait_mass");
+    L->mass_pending = false;
     return 0;
 }
 
@@ -559,6 +586,31 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, d.d_lse, stream);
     if (rc) return rc;
 
+    // ---- 3b. attention mass each selected unit received (only the score-decay policy asks for it)
+    if (a->d_unit_mass && a->n_sel > 0) {
+        INFLLM_REQUIRE(a->d_mass_scratch, "block_back: unit mass without scratch");
+        for (int u = 0; u < d.B; ++u)
+            for (int i = 0; i < a->n_sel; ++i) {
+                infllm_score_args sc{};
+                sc.d_q = (const bf16_t *)d.d_q_glb + (int64_t)cur * d.B * d.H * d.exc * kD + (int64_t)u * d.H * a->n * kD;
+                sc.q_sl = kD; sc.q_sh = (int64_t)a->n * kD; sc.q_sb = 0;
+                sc.B = 1; sc.H = d.H; sc.Hkv = d.Hkv; sc.Lq = a->n;
+                sc.d_k = (const bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + a->h_sel_slots[u * a->n_sel + i]) * slot_elems;
+                sc.k_sl = kD; sc.k_sh = (int64_t)bs * kD; sc.k_sb = 0;
+                sc.cap = bs; sc.j_lo = 0; sc.j_hi = bs;
+                sc.mask = INFLLM_MASK_NONE; sc.accumulate = 0;
+                sc.d_lse = d.d_lse + (int64_t)u * d.H * a->n; sc.softmax_scale = d.softmax_scale;
+                sc.d_score = a->d_mass_scratch + ((int64_t)u * a->n_sel + i) * d.H * bs;
+                sc.score_sh = bs; sc.score_sb = 0; sc.score_cap = bs;
+                rc = infllm_local_score(&sc, stream);
+                if (rc) return rc;
+            }
+        hipLaunchKernelGGL(unit_mass_kernel, dim3(a->n_sel, d.B), dim3(256), 0, st, a->d_mass_scratch, d.H * bs, a->d_unit_mass);
+        INFLLM_CHECK_LAUNCH("unit_mass");
+        HIP_OK(hipEventRecord(L->mass_done, st), "block_back: event");
+        L->mass_pending = true;
+    }
+
     // ---- 4. what the next block's retrieval waits for: scores of the tokens that leave the ring now,
     //         init peeling, representatives of the new units
     const int64_t new_cursor = a->cursor + a->init_take + (int64_t)a->n_carve * bs;
@@ -586,7 +638,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     // ---- 5. the next block's retrieval (its prologue ran in block_front)
     L->topk_pending = false;
     const int n_units_next = a->n_units + a->n_carve;
-    if (L->prepared && n_units_next > d.topk) {
+    if (L->prepared && n_units_next > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL)) {
         INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_back: null representative / score buffer");
         rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->slot,
                              stream);

@@ -93,8 +93,9 @@ class UnitCacheModel:
 class StreamOracle:
     def __init__(self, rope, n_init, n_local, block_size, max_cached_block, topk,
                  exc_block_size, score_decay=None, repr_topk=1, cache_strategy="lru",
-                 perhead=False, topk_hook=None, repr_hook=None):
+                 perhead=False, topk_hook=None, repr_hook=None, chunk_topk_calc=None):
         assert exc_block_size <= n_local                      # context_manager.py:219
+        self.chunk_topk_calc = chunk_topk_calc
         self.rope = rope
         self.n_init, self.n_local = n_init, n_local
         self.block_size, self.topk = block_size, topk
@@ -107,6 +108,7 @@ class StreamOracle:
         self.topk_hook, self.repr_hook = topk_hook, repr_hook
         self.length = 0
         self.ready = False
+        self._chunk_plan = None
         self.block_trace = []     # one dict per execution block
         self.unit_trace = []      # one dict per carved unit
 
@@ -137,7 +139,35 @@ class StreamOracle:
         return x.repeat_interleave(self.H // self.Hkv, dim=1)
 
     # -------------------------------------------------------------- retrieval
+    def _retrieve_chunk(self, gq_chunk):
+        """context_manager.py:548-612: the selections of every execution block of a chunk, all against the
+        units that exist when the chunk starts.  The score is the head MEAN of q-bar_h . rep_h (a positive
+        multiple of the per-block score of :159-163, so the same ranking)."""
+        n_blocks = -(-gq_chunk.shape[2] // self.exc_block_size)
+        out = []
+        for j in range(n_blocks):
+            blk = gq_chunk[:, :, j * self.exc_block_size:(j + 1) * self.exc_block_size]
+            if self.n_units <= self.topk:
+                out.append(([list(range(self.n_units)) for _ in range(self.B)], [None] * self.B))
+                continue
+            mean_q = blk.mean(dim=2)                                           # [B, H, D]
+            chosen, scores = [], []
+            for u in range(self.B):
+                reps = torch.stack(self.reps[u]).reshape(self.n_units, self.H, self.D)
+                sc = torch.einsum("nhd,hd->nh", reps, mean_q[u]).mean(dim=1)
+                pick = sorted(sc.topk(self.topk).indices.tolist())
+                if self.topk_hook is not None:
+                    other = self.topk_hook(len(self.block_trace) + j, u, sc * self.H)
+                    if other is not None:
+                        pick = sorted(other)
+                chosen.append(pick)
+                scores.append(sc * self.H)
+            out.append((chosen, scores))
+        return out
+
     def _retrieve(self, gq_block):
+        if self._chunk_plan is not None:                                       # :366-383, the cached branch
+            return self._chunk_plan[self._chunk_pos]
         if self.n_units <= self.topk:
             chosen = [list(range(self.n_units)) for _ in range(self.B)]
             scores = [None] * self.B
@@ -254,15 +284,31 @@ class StreamOracle:
         self.rem_score = torch.cat((self.rem_score, torch.zeros(self.B, self.H, L, dtype=k.dtype)), dim=-1)
         gq = self.rope.one_angle(q, self.n_local)
 
+        # context_manager.py:749-770: chunk boundaries at multiples of chunk_topk_calc, plus the tail
+        use_chunks = self.chunk_topk_calc is not None and L > 1
+        self._chunk_plan = None
+        if use_chunks:
+            per_chunk = self.chunk_topk_calc // self.exc_block_size
+            cuts = [i * self.exc_block_size for i in range(0, L // self.exc_block_size + 1, per_chunk)]
+            if cuts[-1] < L:
+                cuts.append(L)
+            cut_i = -1
+
         outs = []
         for st in range(0, L, self.exc_block_size):
             ed = min(st + self.exc_block_size, L)
+            if use_chunks and cuts[cut_i + 1] < ed:
+                cut_i += 1
+                self._chunk_plan = self._retrieve_chunk(gq[:, :, cuts[cut_i]:cuts[cut_i + 1]])
+                self._chunk_pos = 0
             kv_st = max(kv_len + st - L - self.n_local, 0)
             kv_ed = kv_len + ed - L
             o, ls = self._block(q[:, :, st:ed], self.win_k[:, :, kv_st:kv_ed],
                                 self.win_v[:, :, kv_st:kv_ed], gq[:, :, st:ed], cur_st, cur_ed)
             outs.append(o)
             cur_st, cur_ed = self._after_block(ed - st, kv_ed - kv_st, ls, cur_st, cur_ed)
+            if use_chunks:
+                self._chunk_pos += 1
 
         self.length += L
         if self.win_k.shape[-2] >= self.n_local:

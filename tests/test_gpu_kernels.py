@@ -105,6 +105,27 @@ def test_block_mean():
         assert torch.allclose(qbar[:, j], want, atol=1e-5)
 
 
+def test_chunk_qbar_is_the_mean_of_the_one_angle_rotation():
+    """infllm_chunk_qbar means first and rotates once; the oracle rotates every row (rope.py:93-104) and then
+    means (context_manager.py:571-576).  Strided input rows (a slice of a longer call)."""
+    from infllm_amd import _lib
+    lib = _lib.load()
+    B, H, n, exc, n_local = 2, 3, 150, 64, 48
+    full = _rand((B, H, n + 20, D), 5)
+    q = full[:, :, 7:7 + n]
+    rope = RopeOracle(D, base=1e4)
+    inv_freq = rope.inv_freq.float().cuda()
+    qd = full.cuda()[:, :, 7:7 + n]
+    qbar = torch.zeros((B, 3, H * D), dtype=torch.float32, device="cuda")
+    _lib.check(lib.infllm_chunk_qbar(qd.data_ptr(), qd.stride(0), qd.stride(1), qd.stride(2), B, H, n, exc, inv_freq.data_ptr(),
+                                     1.0, n_local - 1, qbar.data_ptr(), torch.cuda.current_stream().cuda_stream), "infllm_chunk_qbar")
+    rot = rope.one_angle(q.float(), n_local)
+    for j, (a, b) in enumerate(((0, 64), (64, 128), (128, 150))):
+        want = rot[:, :, a:b].mean(dim=2).reshape(B, H * D)
+        assert torch.allclose(qbar[:, j].cpu(), want, atol=2e-5), float((qbar[:, j].cpu() - want).abs().max())
+    assert lib.infllm_chunk_qbar(None, 0, 0, 0, B, H, n, exc, inv_freq.data_ptr(), 1.0, 0, qbar.data_ptr(), None) != 0
+
+
 # ----------------------------------------------------------------- attention
 def _oracle_two_stage(q, stages):
     a = MultiStageOracle(q.shape)

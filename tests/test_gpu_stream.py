@@ -39,7 +39,7 @@ def _run_gpu(q, k, v, calls, base, **kw):
     rope = RotaryEmbeddingESM(D, base=base, device="cuda")
     cm = ContextManager(rope, kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"], kw["topk"],
                         kw["exc_block_size"], kw.get("score_decay"), False, kw.get("repr_topk", 1),
-                        kw.get("cache_strategy", "lru"), None, kw.get("async_global_stream", False), False, False,
+                        kw.get("cache_strategy", "lru"), kw.get("chunk_topk_calc"), kw.get("async_global_stream", False), False, False,
                         kw.get("perhead", False))
     cm.record_trace = True
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
@@ -94,7 +94,8 @@ def _compare(T, calls, H, Hkv, base, seed, B=1, **kw):
     fol = Follower(cm, kw["topk"], kw.get("repr_topk", 1))
     ora = StreamOracle(RopeOracle(D, base=base), kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"],
                        kw["topk"], kw["exc_block_size"], repr_topk=kw.get("repr_topk", 1), perhead=kw.get("perhead", False),
-                       topk_hook=fol.topk_hook, repr_hook=fol.repr_hook)
+                       topk_hook=fol.topk_hook, repr_hook=fol.repr_hook, cache_strategy=kw.get("cache_strategy", "lru"),
+                       score_decay=kw.get("score_decay"), chunk_topk_calc=kw.get("chunk_topk_calc"))
     outs, pos = [], 0
     for L in calls:
         sl = slice(pos, pos + L)
@@ -120,6 +121,27 @@ SMALL = dict(n_init=16, n_local=256, block_size=32, max_cached_block=8, topk=4, 
 def test_small_geometry_follows_oracle(calls):
     cm, ora, fol = _compare(sum(calls), calls, H=8, Hkv=2, base=1e4, seed=len(calls), **SMALL)
     assert cm.num_global_block > SMALL["topk"]            # retrieval was exercised
+
+
+def test_score_decay_policy_follows_oracle():
+    """cache_strategy lru-s: evictions are decided by the decayed attention mass each cached unit received
+    (context_manager.py:454-470), which the device computes and the host reads back once per block."""
+    kw = dict(SMALL, cache_strategy="lru-s", score_decay=0.1, max_cached_block=6)
+    cm, ora, _ = _compare(1500, [700, 1, 1, 798], H=8, Hkv=2, base=1e4, seed=31, B=2, **kw)
+    assert cm.stats["evictions"] > 20
+    for u in range(2):
+        gpu_events = [sorted(e) for e in cm.policy[u].evicted_log]
+        assert gpu_events == [sorted(e["evicted"]) for e in ora.cache[u].events]
+        assert list(cm.policy[u].cached) == list(ora.cache[u].cached)      # same residents, same dict order
+    # unit masses: every block's mass is a share of the H * n probabilities of that block
+    assert 0.0 < float(cm.mass_host.sum()) <= 2 * 8 * 64 + 1e-3
+
+
+@pytest.mark.parametrize("chunk", [64, 192, 4096])
+def test_chunked_retrieval_follows_oracle(chunk):
+    kw = dict(SMALL, chunk_topk_calc=chunk)
+    cm, ora, _ = _compare(1334, [1000, 1, 333], H=8, Hkv=2, base=1e4, seed=33, B=2, **kw)
+    assert cm.num_global_block > SMALL["topk"]
 
 
 def test_unaligned_geometry_and_batch():

@@ -217,3 +217,59 @@ def test_cache_model_ties_break_in_insertion_order_and_selected_are_kept():
     assert s.events[-1]["evicted"] == [0]
     with pytest.raises(AssertionError):
         UnitCacheModel(1, "lru").touch([0, 1])
+
+
+# ------------------------------------------------------------- chunked retrieval (context_manager.py:548-612, 749-770)
+def test_chunked_retrieval_with_one_block_per_chunk_is_the_plain_path():
+    calls = [96, 40, 1, 64, 23]
+    q, k, v = _stream(sum(calls), seed=21)
+    plain, cm0 = _run(q, k, v, calls)
+    chunked, cm1 = _run(q, k, v, calls, chunk_topk_calc=GEOM["exc_block_size"])
+    assert [b["selected"] for b in cm0.block_trace] == [b["selected"] for b in cm1.block_trace]
+    assert torch.equal(plain, chunked)
+
+
+def test_chunked_retrieval_freezes_the_unit_set_at_each_chunk_start():
+    exc, chunk = GEOM["exc_block_size"], 3 * GEOM["exc_block_size"]
+    calls = [150, 1, 70]                                    # 150 = 3 chunks + a ragged tail; single tokens bypass chunks
+    q, k, v = _stream(sum(calls), seed=22)
+    out, cm = _run(q, k, v, calls, chunk_topk_calc=chunk)
+    # replay: which units exist at each block / at the start of its chunk (closed form of the carving)
+    n_units_at = lambda T: max(0, (T - GEOM["n_init"] - GEOM["n_local"]) // GEOM["block_size"])
+    rope = RopeOracle(q.shape[-1], base=10000)
+    pos, bi = 0, 0
+    for L in calls:
+        gq = rope.one_angle(q[:, :, pos:pos + L], GEOM["n_local"])
+        for st in range(0, L, exc):
+            blk = cm.block_trace[bi]
+            chunk_start = pos + (st // chunk) * chunk if L > 1 else pos + st
+            frozen = n_units_at(chunk_start)
+            if L > 1:
+                assert all(u < frozen for u in blk["selected"][0]) and blk["n_units"] >= frozen
+            if frozen > GEOM["topk"]:
+                # brute force in fp64: sum over heads of mean-query . representative, over the frozen units only
+                mean_q = gq[0, :, st:st + exc].double().mean(dim=1).reshape(-1)
+                reps = torch.stack(cm.reps[0][:frozen]).double()
+                want = sorted(torch.topk(reps @ mean_q, GEOM["topk"]).indices.tolist())
+                assert blk["selected"][0] == want
+            bi += 1
+        pos += L
+    # results still equal an un-chunked run whenever the selections happen to agree block by block
+    assert bi == len(cm.block_trace) and out.shape[2] == sum(calls)
+
+
+def test_chunked_retrieval_changes_selections_but_not_the_attention_rule():
+    """A chunk that spans several blocks may select differently from the plain path (new units are invisible
+    until the next chunk); forcing the plain path to the same selections reproduces the output exactly.
+    The stream is warmed up with single-token calls (which never use chunks) until more than topk units exist,
+    so that the plain path consults its hook in every later block."""
+    calls = [1] * 70 + [160]
+    q, k, v = _stream(sum(calls), seed=23)
+    out_c, cm_c = _run(q, k, v, calls, chunk_topk_calc=4 * GEOM["exc_block_size"])
+    picks = [b["selected"] for b in cm_c.block_trace]
+    assert cm_c.block_trace[70]["n_units"] > GEOM["topk"]
+    hook = lambda block, row, scores: picks[block][row]
+    out_p, cm_p = _run(q, k, v, calls, topk_hook=hook)
+    assert [b["selected"] for b in cm_p.block_trace] == picks
+    assert torch.equal(out_c, out_p)
+    assert [b["selected"] for b in _run(q, k, v, calls)[1].block_trace] != picks      # and the chunking mattered here
