@@ -86,6 +86,14 @@ int infllm_chunk_qbar(const void *d_q, int64_t q_sb, int64_t q_sh, int64_t q_sl,
                       int32_t n, int32_t exc, const float *d_inv_freq, double distance_scale,
                       int64_t glb_pos, float *d_qbar, void *stream);
 
+/* RoPE of plain rows, for the attention types that rotate tensors themselves (stream_llm.py:62-73,
+ * infinite_lm.py:59-66, origin.py:36; rope.py:27-47, 93-112): x [B,H,L,128] bf16 with element strides
+ * sb/sh/sl -> d_out [B,H,L,128] contiguous, row r rotated by the angle of position pos0 + r*pos_step
+ * (pos_step 1: consecutive positions; 0: one angle for every row).  Angles in fp64. */
+int infllm_rope_rows(const void *d_x, int64_t sb, int64_t sh, int64_t sl, int32_t B, int32_t H, int32_t L,
+                     int64_t pos0, int32_t pos_step, const float *d_inv_freq, double distance_scale,
+                     void *d_out, void *stream);
+
 /* ---------------------------------------------------------------------------
  * One stage of the multi-stage attention (bf16 MFMA flash kernel).
  * Replaces MultiStageDotProductionAttention.append

@@ -115,6 +115,7 @@ SYMBOLS = {
     "infllm_reduce_partials": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_f32, c_vp, c_vp]),
     "infllm_block_mean": (c_i32, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "infllm_chunk_qbar": (c_i32, [c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_i32, c_vp, C.c_double, c_i64, c_vp, c_vp]),
+    "infllm_rope_rows": (c_i32, [c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_i64, c_i32, c_vp, C.c_double, c_vp, c_vp]),
     "infllm_attn_stage": (c_i32, [C.POINTER(AttnArgs), c_vp]),
     "infllm_attn_merge": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
     "infllm_local_score": (c_i32, [C.POINTER(ScoreArgs), c_vp]),

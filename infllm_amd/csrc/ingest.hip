@@ -212,6 +212,25 @@ __global__ __launch_bounds__(kMeanThreads) void chunk_qbar_kernel(const bf16_t *
     }
 }
 
+// RoPE of plain rows (rope.py:27-47, 93-104): out[b,h,r,:] = x[b,h,r,:] rotated by the angle of position
+// pos0 + r * pos_step (pos_step 0: every row by the same angle).  One wave per row, a lane owns the pair
+// (d, d + 64); the angle is formed in fp64 like in the stream prologue.
+__global__ __launch_bounds__(256) void rope_rows_kernel(const bf16_t *x, int64_t sb, int64_t sh, int64_t sl, int H, int L,
+                                                        int64_t pos0, int pos_step, const float *inv_freq,
+                                                        double distance_scale, bf16_t *out) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6), h = blockIdx.y, b = blockIdx.z;
+    if (r >= L) return;
+    const bf16_t *src = x + (int64_t)b * sb + (int64_t)h * sh + (int64_t)r * sl;
+    bf16_t *dst = out + (((int64_t)b * H + h) * L + r) * kD;
+    double sn, cs;
+    sincos((double)(pos0 + (int64_t)r * pos_step) * distance_scale * (double)inv_freq[lane], &sn, &cs);
+    const float c = (float)cs, s = (float)sn;
+    const float lo = bf16_bits_to_f32(((const uint16_t *)src)[lane]), hi = bf16_bits_to_f32(((const uint16_t *)src)[lane + kD / 2]);
+    ((uint16_t *)dst)[lane] = (uint16_t)(pack_bf16x2(lo * c - hi * s, 0.f) & 0xffffu);
+    ((uint16_t *)dst)[lane + kD / 2] = (uint16_t)(pack_bf16x2(hi * c + lo * s, 0.f) & 0xffffu);
+}
+
 __global__ __launch_bounds__(256) void gather_rows_kernel(const bf16_t *ring, int64_t ring_cap, int Hkv, int64_t t0,
                                                           int n, int unit_rows, bf16_t *out, int64_t out_sb,
                                                           int64_t out_su, int64_t out_sh) {
@@ -278,6 +297,17 @@ extern "C" int infllm_chunk_qbar(const void *d_q, int64_t q_sb, int64_t q_sh, in
     hipLaunchKernelGGL(chunk_qbar_kernel, dim3(n_blocks, H, B), dim3(kMeanThreads), 0, (hipStream_t)stream, (const bf16_t *)d_q,
                        q_sb, q_sh, q_sl, H, n, exc, d_inv_freq, distance_scale, glb_pos, d_qbar, n_blocks);
     INFLLM_CHECK_LAUNCH("chunk_qbar");
+    return 0;
+}
+
+extern "C" int infllm_rope_rows(const void *d_x, int64_t sb, int64_t sh, int64_t sl, int32_t B, int32_t H, int32_t L, int64_t pos0,
+                                int32_t pos_step, const float *d_inv_freq, double distance_scale, void *d_out, void *stream) {
+    INFLLM_REQUIRE(B >= 0 && H >= 0 && L >= 0 && pos0 >= 0 && (pos_step == 0 || pos_step == 1), "rope_rows: bad sizes B=%d H=%d L=%d", B, H, L);
+    if (B == 0 || H == 0 || L == 0) return 0;
+    INFLLM_REQUIRE(d_x && d_inv_freq && d_out, "rope_rows: null pointer");
+    hipLaunchKernelGGL(rope_rows_kernel, dim3((L + 3) / 4, H, B), dim3(256), 0, (hipStream_t)stream, (const bf16_t *)d_x, sb, sh, sl,
+                       H, L, pos0, pos_step, d_inv_freq, distance_scale, (bf16_t *)d_out);
+    INFLLM_CHECK_LAUNCH("rope_rows");
     return 0;
 }
 

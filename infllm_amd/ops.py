@@ -84,6 +84,17 @@ def reduce_partials(parts, scale, out):
           "infllm_reduce_partials")
 
 
+def rope_rows(x, inv_freq, distance_scale, pos0, consecutive=True):
+    """x [B,H,L,128] bf16 (any strides with unit last stride) -> contiguous rows rotated at pos0 + r (or all at pos0)."""
+    B, H, L, D = x.shape
+    assert x.dtype == torch.bfloat16 and D == 128 and (L == 0 or x.stride(3) == 1)
+    out = torch.empty((B, H, L, D), dtype=torch.bfloat16, device=x.device)
+    check(_lib.load().infllm_rope_rows(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2), B, H, L, int(pos0),
+                                       1 if consecutive else 0, inv_freq.data_ptr(), float(distance_scale), out.data_ptr(),
+                                       _stream()), "infllm_rope_rows")
+    return out
+
+
 def block_mean(q_glb, B, H, n, exc, qbar):
     check(_lib.load().infllm_block_mean(q_glb.data_ptr(), B, H, n, exc, qbar.data_ptr(), _stream()), "infllm_block_mean")
 
