@@ -21,7 +21,7 @@
 namespace {
 
 constexpr int kWaves = 8;                  // 2 per SIMD inside ONE workgroup: a K/V tile in LDS feeds 256 query rows
-constexpr int kStages = 4;                 // K/V tiles resident in LDS (up to 3 in flight ahead of the math)
+constexpr int kStages = 4;                 // K/V tiles resident in LDS: the pair being multiplied and the pair in flight
 constexpr int kThreads = kWaves * kWave;
 constexpr int kQTile = 32;                 // queries per wave
 constexpr int kBig = 1 << 29;              // clamp for mask distances held in int32
@@ -137,8 +137,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         wg_lo[wave] = w_t1 > w_t0 ? w_t0 : INT32_MAX;
         wg_hi[wave] = w_t1 > w_t0 ? w_t1 : INT32_MIN;
     }
-    // LDS starts as zeros so that rows never written hold finite values (0 * stale must stay 0)
-    for (int e = tid; e < 2 * kStages * kTileBytes / 16; e += kThreads) ((u32x4 *)lds_dyn)[e] = u32x4{0, 0, 0, 0};
     __syncthreads();
     int g_t0 = INT32_MAX, g_t1 = INT32_MIN;
 #pragma unroll
@@ -155,18 +153,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         g_t1 = t_end;
     }
 
-    // ---- Q as the B operand: lane = (query col, k-group)
-    bf16x8 qreg[kD / 16];
-    {
-        const int qi = i0 + col;
-        const bool ok = live && qi < a.Lq;
-        const bf16_t *qrow = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qi * a.q_sl;
-#pragma unroll
-        for (int kk = 0; kk < kD / 16; ++kk) {
-            u32x4 raw = ok ? *(const u32x4 *)(qrow + kk * 16 + grp * 8) : u32x4{0, 0, 0, 0};
-            qreg[kk] = __builtin_bit_cast(bf16x8, raw);
-        }
-    }
+    bf16x8 qreg[kD / 16];                     // Q as the B operand: lane = (query col, k-group); loaded behind the first tiles
 
     // ---- per-lane LDS byte offsets of the MFMA operands (inside one tile buffer)
     uint32_t k_off[kD / 16];                  // K operand kk of sub-tile 0 (sub-tile 1: + 32 rows)
@@ -208,7 +195,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         v_head = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh;
         ring_row = ((int64_t)g_t0 * kTile) % a.cap;
     }
-    int partial_in_flight = 0;
     auto load_tile = [&](int t, int buf) {
         const bf16_t *kbase, *vbase;
         int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
@@ -235,12 +221,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                 load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
             }
         } else {
-            partial_in_flight = kStages;          // not every wave issues every load: wait for all of them for a while
 #pragma unroll
             for (int i = 0; i < kLd; ++i) {
-                // rows outside the source keep whatever the buffer held (finite values): their keys are masked
+                // rows outside the source are written as zeros: their keys are masked, but 0 * stale must stay 0
                 if (gk_row[i] >= row_lo && gk_row[i] < row_hi) load_to_lds16(kbase + gk_off[i], (bf16_t *)(kdst + i * 1024));
+                else *(u32x4 *)(kdst + i * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
                 if (gv_row[i] >= row_lo && gv_row[i] < row_hi) load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
+                else *(u32x4 *)(vdst + i * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
             }
         }
     };
@@ -397,52 +384,70 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         }
     };
 
-    // kStages - 1 tiles are requested ahead; tile t lives in buffer (t - g_t0) % kStages, and the buffer a
-    // new tile goes to was last read before the previous barrier
-    for (int p = 0; p < kStages - 1; ++p)
+    // Tiles are handled in pairs: one barrier per two tiles.  While the pair (t, t+1) is multiplied, the next
+    // pair is on its way into the other two buffers, which were last read before the previous barrier; the
+    // loads of a pair are the only ones outstanding, so landing = vmcnt(0).
+    static_assert(kStages == 4, "two buffer pairs");
+    for (int p = 0; p < 2; ++p)
         if (g_t0 + p < g_t1) load_tile(g_t0 + p, p);
-    auto wait_tile = [&](int t) {           // returns once tile t has landed (loads complete in order)
-        const int ahead = min(g_t1 - 1 - t, kStages - 2);       // tiles requested after t
-        if (partial_in_flight > 0 || ahead <= 0) {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        } else if (ahead == 1) {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLd) : "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * kLd) : "memory");
+    {
+        const int qi = i0 + col;
+        const bool ok = live && qi < a.Lq;
+        const bf16_t *qrow = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qi * a.q_sl;
+#pragma unroll
+        for (int kk = 0; kk < kD / 16; ++kk) {
+            u32x4 raw = ok ? *(const u32x4 *)(qrow + kk * 16 + grp * 8) : u32x4{0, 0, 0, 0};
+            qreg[kk] = __builtin_bit_cast(bf16x8, raw);
         }
-    };
-    if (g_t1 > g_t0) wait_tile(g_t0);
+    }
+
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int t = g_t0; t < g_t1; ++t) {
-        const int buf = (t - g_t0) % kStages;
+    for (int t = g_t0; t < g_t1; t += 2) {
+        const int buf = (t - g_t0) & 3;                          // 0 or 2
         PH_STAMP();
-        if (t + kStages - 1 < g_t1) load_tile(t + kStages - 1, (buf + kStages - 1) % kStages);
-        if (partial_in_flight > 0) --partial_in_flight;
+        if (t + 2 < g_t1) load_tile(t + 2, buf ^ 2);
+        if (t + 3 < g_t1) load_tile(t + 3, (buf ^ 2) + 1);
         PH_STAMP();
         if (t >= w_t0 && t < w_t1) tile_math(buf, t);          // wave-uniform; barriers stay outside
+        if (t + 1 < g_t1 && t + 1 >= w_t0 && t + 1 < w_t1) tile_math(buf + 1, t + 1);
         PH_STAMP();
-        if (t + 1 < g_t1) wait_tile(t + 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         PH_STAMP();
         __syncthreads();
     }
 
     PH_STAMP();
-    // ---- epilogue: normalised partial + base-2 log-sum-exp
+    // ---- epilogue: normalised partial + base-2 log-sum-exp.  The accumulators hold O^T (a lane owns a query and
+    //      scattered 4-float pieces of its row); they go through this wave's 16 KB of the now idle tile buffers so
+    //      that every store instruction writes two whole 512-byte rows.
     if (!live) return;
     const float l_tot = l_run + wave_xor32(l_run);
     const int qi = i0 + col;
-    if (qi >= a.Lq) return;
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int64_t row = (((int64_t)split * a.B + b) * a.H + h) * a.Lq + qi;
-    float *orow = a.d_o_part + row * kD;
+    const int64_t row0 = (((int64_t)split * a.B + b) * a.H + h) * a.Lq + i0;      // row of this wave's first query
+    const int64_t row = row0 + col;
+    {
+        char *stage = lds_dyn + wave * (kQTile * kD * 4);
 #pragma unroll
-    for (int dt = 0; dt < kD / 32; ++dt)
+        for (int dt = 0; dt < kD / 32; ++dt)
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            f32x4 o4{oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv, oacc[dt][4 * q4 + 2] * inv,
-                     oacc[dt][4 * q4 + 3] * inv};
-            *(f32x4 *)(orow + dt * 32 + 8 * q4 + 4 * grp) = o4;
+            for (int q4 = 0; q4 < 4; ++q4) {
+                f32x4 o4{oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv, oacc[dt][4 * q4 + 2] * inv,
+                         oacc[dt][4 * q4 + 3] * inv};
+                const int chunk = dt * 8 + 2 * q4 + grp;                           // 16-byte piece of the row
+                *(f32x4 *)(stage + col * (kD * 4) + ((chunk ^ col) & 31) * 16) = o4;
+            }
+        const int rows_left = a.Lq - i0;                                           // valid queries of this tile
+        const int piece = lane & 31;
+#pragma unroll
+        for (int k2 = 0; k2 < kQTile / 2; ++k2) {
+            const int qr = 2 * k2 + (lane >> 5);
+            const f32x4 o4 = *(const f32x4 *)(stage + qr * (kD * 4) + ((piece ^ qr) & 31) * 16);
+            if (qr < rows_left) *(f32x4 *)(a.d_o_part + (row0 + qr) * kD + piece * 4) = o4;
         }
+    }
+    if (qi >= a.Lq) return;
     if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run * scale + log2f(l_tot) : -INFINITY;
     PH_STAMP();
 }
