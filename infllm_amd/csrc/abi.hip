@@ -42,43 +42,45 @@ extern "C" int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int
 namespace {
 
 constexpr int kFetchMax = 64;          // units per launch
-constexpr int kFetchChunk = 16384;     // bytes moved by one workgroup iteration (256 threads x 4 x 16 B)
 
 struct FetchList {
     const uint4 *src[kFetchMax];
     uint4 *dst[kFetchMax];
 };
 
-// A small, fixed number of workgroups walks all (unit, chunk) pairs: reads that cross PCIe stay
-// outstanding for microseconds, and spreading them over every CU stalls the memory pipelines of the
-// kernels running beside the fetch.  4 independent 16-byte loads per thread keep the link busy.
+// A fixed number of workgroups walks all (unit, piece) pairs.  Reads that cross PCIe stay outstanding for
+// microseconds and slow down whatever else runs on the chip in proportion to how many are in flight, so the
+// launch is shaped for just enough of them to keep the link busy: 128 single-wave workgroups with one 16-byte
+// load per lane (128 KiB in flight) measured best for the whole stream.  U independent loads per thread.
+template <int U>
 __global__ __launch_bounds__(256) void unit_fetch_kernel(FetchList list, int n_units, int64_t nbytes) {
-    const int chunks_per_unit = (int)((nbytes + kFetchChunk - 1) / kFetchChunk);
-    const int total = n_units * chunks_per_unit;
+    const int piece = (int)blockDim.x * U * 16;              // bytes moved by one workgroup iteration
+    const int pieces_per_unit = (int)((nbytes + piece - 1) / piece);
+    const int total = n_units * pieces_per_unit;
+    const int64_t end = nbytes / 16;
     for (int w = blockIdx.x; w < total; w += gridDim.x) {
-        const int unit = w / chunks_per_unit;
-        const int64_t begin = (int64_t)(w % chunks_per_unit) * kFetchChunk / 16;
-        const int64_t end = nbytes / 16;
+        const int unit = w / pieces_per_unit;
+        const int64_t begin = (int64_t)(w % pieces_per_unit) * (piece / 16);
         const uint4 *src = list.src[unit];
         uint4 *dst = list.dst[unit];
-        uint4 v[4];
+        uint4 v[U];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (begin + threadIdx.x + 256 * i < end) v[i] = src[begin + threadIdx.x + 256 * i];
+        for (int i = 0; i < U; ++i)
+            if (begin + threadIdx.x + blockDim.x * i < end) v[i] = src[begin + threadIdx.x + blockDim.x * i];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (begin + threadIdx.x + 256 * i < end) dst[begin + threadIdx.x + 256 * i] = v[i];
+        for (int i = 0; i < U; ++i)
+            if (begin + threadIdx.x + blockDim.x * i < end) dst[begin + threadIdx.x + blockDim.x * i] = v[i];
     }
 }
 
-int fetch_workgroups() {
-    static int n = [] {
-        const char *e = getenv("INFLLM_FETCH_WGS");
-        int v = e ? atoi(e) : 0;
-        return v > 0 ? v : 32;
-    }();
-    return n;
+int env_int(const char *name, int fallback) {
+    const char *e = getenv(name);
+    const int v = e ? atoi(e) : 0;
+    return v > 0 ? v : fallback;
 }
+int fetch_workgroups() { static int n = env_int("INFLLM_FETCH_WGS", 128); return n; }
+int fetch_threads() { static int n = env_int("INFLLM_FETCH_THREADS", 64); return n == 128 || n == 256 ? n : 64; }
+int fetch_unroll() { static int n = env_int("INFLLM_FETCH_UNROLL", 1); return n == 2 || n == 4 ? n : 1; }
 
 }  // namespace
 
@@ -96,9 +98,12 @@ extern "C" int infllm_fetch_units(const void *const *h_src, void *const *d_dst, 
             list.src[i] = (const uint4 *)h_src[first + i];
             list.dst[i] = (uint4 *)d_dst[first + i];
         }
-        const int64_t work = (int64_t)m * ((nbytes + kFetchChunk - 1) / kFetchChunk);
+        const int threads = fetch_threads(), unroll = fetch_unroll();
+        const int64_t piece = (int64_t)threads * unroll * 16;
+        const int64_t work = (int64_t)m * ((nbytes + piece - 1) / piece);
         const int wgs = work < fetch_workgroups() ? (int)work : fetch_workgroups();
-        hipLaunchKernelGGL(unit_fetch_kernel, dim3(wgs), dim3(256), 0, (hipStream_t)stream, list, m, nbytes);
+        auto kern = unroll == 1 ? unit_fetch_kernel<1> : unroll == 2 ? unit_fetch_kernel<2> : unit_fetch_kernel<4>;
+        hipLaunchKernelGGL(kern, dim3(wgs), dim3(threads), 0, (hipStream_t)stream, list, m, nbytes);
         INFLLM_CHECK_LAUNCH("unit_fetch");
     }
     return 0;
