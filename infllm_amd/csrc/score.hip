@@ -16,9 +16,12 @@ namespace {
 
 constexpr int kQStage = 64;                // queries per LDS stage
 constexpr int kQPad = kD + 8;              // LDS row of Q (bf16 elements): 272 bytes rotates the banks
-constexpr int kKeysPerWg = 4 * kTile;
 
+// KS = 32-key halves per wave: 2 for long key ranges; 1 halves the work of a wave per query stage, which is what
+// bounds the short launches that sit on the critical path between two blocks.
+template <int KS>
 __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a) {
+    constexpr int kWaveKeys = 32 * KS, kKeysPerWg = 4 * kWaveKeys;
     __shared__ __attribute__((aligned(16))) bf16_t Qs[2][kQStage][kQPad];
     __shared__ __attribute__((aligned(16))) float Ls[2][kQStage];
 
@@ -26,15 +29,15 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     const int col = lane & 31, grp = lane >> 5;
     const int G = a.H / a.Hkv;
     const int b = blockIdx.y / a.H, h = blockIdx.y % a.H, g = h / G;
-    const int64_t jg = ((a.j_lo >> 6) + (int64_t)blockIdx.x * 4) * kTile;   // first key of the workgroup
-    const int64_t j0 = jg + (int64_t)wave * kTile;                          // first key of this wave
+    const int64_t jg = (a.j_lo / kWaveKeys + (int64_t)blockIdx.x * 4) * kWaveKeys;   // first key of the workgroup
+    const int64_t j0 = jg + (int64_t)wave * kWaveKeys;                               // first key of this wave
     const float scale = a.softmax_scale * 1.4426950408889634f;
 
     // ---- this wave's 64 keys as the B operand (lane = key column)
-    bf16x8 kreg[2][kD / 16];
-    bool jok[2];
+    bf16x8 kreg[KS][kD / 16];
+    bool jok[KS];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < KS; ++ks) {
         const int64_t j = j0 + ks * 32 + col;
         jok[ks] = j >= a.j_lo && j < a.j_hi;
         const bf16_t *krow = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh + (j % a.cap) * a.k_sl;
@@ -64,7 +67,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     };
     int64_t g_lo, g_hi, w_lo, w_hi;
     query_range(jg, jg + kKeysPerWg - 1, g_lo, g_hi);
-    query_range(j0, j0 + kTile - 1, w_lo, w_hi);
+    query_range(j0, j0 + kWaveKeys - 1, w_lo, w_hi);
     const int st_lo = (int)(g_lo / kQStage), st_hi = g_hi > g_lo ? (int)((g_hi - 1) / kQStage) + 1 : st_lo;
 
     const bf16_t *qbase = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
         if (tid < kQStage) Ls[buf][tid] = lbuf;
     };
 
-    float colsum[2] = {0.f, 0.f};
+    float colsum[KS] = {};
     if (st_hi > st_lo) {
         load_stage(st_lo);
         store_stage(0);
@@ -109,14 +112,20 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
                 f32x4 l4[4];                                     // lse of rows 8*(r>>2) + 4*grp + (r&3)
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) l4[q4] = *(const f32x4 *)&Ls[cur][qs * 32 + 8 * q4 + 4 * grp];
+                // both key halves at once: two independent accumulator chains keep the matrix pipe busy
+                f32x16 sacc2[KS];
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    f32x16 sacc;
+                for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+                    for (int r = 0; r < 16; ++r) sacc2[ks][r] = 0.f;
 #pragma unroll
-                    for (int kk = 0; kk < kD / 16; ++kk)
-                        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[kk], kreg[ks][kk], sacc, 0, 0, 0);
+                for (int kk = 0; kk < kD / 16; ++kk)
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        sacc2[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[kk], kreg[ks][kk], sacc2[ks], 0, 0, 0);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const f32x16 sacc = sacc2[ks];
                     // dist(i, j) = i - j + offset for the first query row and this lane's key
                     const int64_t jk = j0 + ks * 32;
                     const int64_t e0 = iq - jk + a.offset;       // query iq, key jk
@@ -152,7 +161,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
         __syncthreads();
     }
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < KS; ++ks) {
         const float tot = colsum[ks] + wave_xor32(colsum[ks]);
         const int64_t j = j0 + ks * 32 + col;
         if (grp == 0 && jok[ks]) {
@@ -176,8 +185,13 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
     INFLLM_REQUIRE((a->q_sl % 8 | a->q_sh % 8 | a->q_sb % 8 | a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8) == 0,
                    "local_score: strides must be multiples of 8");
     if (a->j_hi <= a->j_lo) return 0;
-    const int64_t tiles = ((a->j_hi - 1) >> 6) - (a->j_lo >> 6) + 1;
-    hipLaunchKernelGGL(local_score_kernel, dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+    if (a->j_hi - a->j_lo > 1024) {
+        const int64_t tiles = (a->j_hi - 1) / 64 - a->j_lo / 64 + 1;
+        hipLaunchKernelGGL(local_score_kernel<2>, dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+    } else {
+        const int64_t tiles = (a->j_hi - 1) / 32 - a->j_lo / 32 + 1;
+        hipLaunchKernelGGL(local_score_kernel<1>, dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+    }
     INFLLM_CHECK_LAUNCH("local_score");
     return 0;
 }
