@@ -133,6 +133,62 @@ def decode_workload(args, dev):
         "cache": cm.stats}))
 
 
+def model_workload(args, dev):
+    """BASELINE config 4: a 32-layer decoder with the Llama-3-8B architecture and random weights, every attention
+    routed through the "inf-llm" type; chunked prefill (all but the last token in pieces of 8192, then the last
+    token) followed by greedy decode steps, driven by GreedySearch.  Prints its own JSON line; not the headline."""
+    import transformers
+    from infllm_amd.utils import GreedySearch, patch_hf
+    cfg = transformers.LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=args.model_layers,
+                                   num_attention_heads=32, num_key_value_heads=8, head_dim=128, vocab_size=128256,
+                                   rope_theta=500000.0, max_position_embeddings=8192, tie_word_embeddings=False)
+    torch.manual_seed(4)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            model = transformers.LlamaForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(old)
+    knobs = {k: KNOBS[k] for k in ("n_init", "n_local", "topk", "block_size", "max_cached_block", "exc_block_size", "repr_topk")}
+    model = patch_hf(model, "inf-llm", dict(knobs, fattn=False), base=500000.0).eval()
+
+    class Tok:                                      # token ids in, token ids out
+        eos_token_id = -1
+
+        def decode(self, ids):
+            return ids.tolist()
+
+    T, steps = args.model_tokens, args.model_decode_steps
+    ids = torch.randint(0, 128256, (T,), generator=torch.Generator().manual_seed(5))
+    gs = GreedySearch(model, Tok())
+    # time the prefill and the decode separately: a first generate() with no new token, then one more that decodes
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    first = gs.generate(input_ids=ids, max_length=0, chunk_size=8192)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    # the cache now holds the whole prompt; feed the token the prefill chose and keep decoding greedily
+    with torch.inference_mode():
+        logits, past = gs._step(ids[None, -1:].to(dev), torch.ones((1, T + 1), dtype=torch.long, device=dev), gs.past_kv)
+        word = logits[:, -1].argmax(dim=-1)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for _ in range(steps):
+            logits, past = gs._step(word.view(1, 1), torch.ones((1, 1), dtype=torch.long, device=dev), past)
+            word = logits[:, -1].argmax(dim=-1)
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+    cm = past[0]
+    print(json.dumps({
+        "metric": "InfLLM full decoder (Llama-3-8B architecture, random weights): prefill tokens/s", "value": T / (t1 - t0),
+        "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config 4: {args.model_layers} layers, {T}-token prefill in chunks of 8192 + last token, "
+                               f"then {steps} greedy steps; inf-llm knobs {knobs}"},
+        "prefill_s": t1 - t0, "decode_steps_per_s": steps / (t3 - t2), "decode_ms_per_step": (t3 - t2) / steps * 1e3,
+        "layer0_cache": cm.stats, "layer0_units": cm.num_global_block}))
+
+
 def cpu_baseline(tokens, threads):
     """The fp32 oracle (restating the reference's torch path) on the first `tokens` tokens of the same
     kind of stream, on the host cores."""
@@ -158,8 +214,12 @@ def main():
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--chunk", type=int, default=8192, help="tokens per append() call")
     ap.add_argument("--cpu-tokens", type=int, default=16384, help="0 disables the CPU baseline")
-    ap.add_argument("--workload", choices=["prefill", "decode"], default="prefill",
-                    help="prefill = the headline 128K-token stream (config 2); decode = config 3 (own JSON line)")
+    ap.add_argument("--workload", choices=["prefill", "decode", "model"], default="prefill",
+                    help="prefill = the headline 128K-token stream (config 2); decode = config 3, model = config 4 "
+                         "(each with its own JSON line)")
+    ap.add_argument("--model-layers", type=int, default=32)
+    ap.add_argument("--model-tokens", type=int, default=131072)
+    ap.add_argument("--model-decode-steps", type=int, default=128)
     ap.add_argument("--decode-units", type=int, default=8192)
     ap.add_argument("--decode-steps", type=int, default=256)
     ap.add_argument("--copy-calibration", action="store_true",
@@ -183,6 +243,9 @@ def main():
         del src, dst
     if args.workload == "decode":
         decode_workload(args, dev)
+        return
+    if args.workload == "model":
+        model_workload(args, dev)
         return
     T = args.tokens
     q, k, v = make_stream(T, 0, dev)
