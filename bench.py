@@ -29,15 +29,30 @@ ROPE_BASE = 1e6
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
-def make_stream(T, seed, device):
-    """q, v ~ N(0,1); keys from a 64-component Gaussian mixture per kv head (means N(0,1), std 0.3)."""
+def make_stream(T, seed, device, favour=0):
+    """q, v ~ N(0,1); keys from a 64-component Gaussian mixture per kv head (means N(0,1), std 0.3).
+    favour > 0 (BASELINE config 5): the queries of an execution block lean towards `favour` mixture components
+    drawn per block (q = that component's mean + N(0,1)), so consecutive blocks retrieve different units."""
     g = torch.Generator(device=device).manual_seed(seed)
-    q = torch.randn((1, H, T, D), generator=g, device=device, dtype=torch.float32).bfloat16()
-    v = torch.randn((1, HKV, T, D), generator=g, device=device, dtype=torch.float32).bfloat16()
     means = torch.randn((HKV, 64, D), generator=g, device=device)
-    comp = torch.randint(0, 64, (HKV, T), generator=g, device=device)
-    k = torch.gather(means, 1, comp[:, :, None].expand(-1, -1, D))
-    k = (k + 0.3 * torch.randn((HKV, T, D), generator=g, device=device))[None].bfloat16()
+    q = torch.empty((1, H, T, D), dtype=torch.bfloat16, device=device)
+    k = torch.empty((1, HKV, T, D), dtype=torch.bfloat16, device=device)
+    v = torch.empty((1, HKV, T, D), dtype=torch.bfloat16, device=device)
+    exc = KNOBS["exc_block_size"]
+    for t0 in range(0, T, 1 << 17):                     # in slices: the fp32 temporaries of a 1M-token stream are large
+        n = min(1 << 17, T - t0)
+        qs = torch.randn((H, n, D), generator=g, device=device)
+        if favour:
+            blocks = (n + exc - 1) // exc
+            pick = torch.randint(0, 64, (blocks, favour), generator=g, device=device)
+            which = torch.randint(0, favour, (n,), generator=g, device=device)
+            comp_q = pick[torch.arange(n, device=device) // exc, which]                      # [n]
+            qs += means[:, comp_q].repeat_interleave(H // HKV, dim=0)                         # [H, n, D]
+        q[0, :, t0:t0 + n] = qs.bfloat16()
+        v[0, :, t0:t0 + n] = torch.randn((HKV, n, D), generator=g, device=device).bfloat16()
+        comp = torch.randint(0, 64, (HKV, n), generator=g, device=device)
+        ks = torch.gather(means, 1, comp[:, :, None].expand(-1, -1, D)) + 0.3 * torch.randn((HKV, n, D), generator=g, device=device)
+        k[0, :, t0:t0 + n] = ks.bfloat16()
     return q, k, v
 
 
@@ -222,6 +237,8 @@ def main():
     ap.add_argument("--model-decode-steps", type=int, default=128)
     ap.add_argument("--decode-units", type=int, default=8192)
     ap.add_argument("--decode-steps", type=int, default=256)
+    ap.add_argument("--favour", type=int, default=0,
+                    help="queries of a block lean towards this many mixture components (config 5 uses 2 with --tokens 1048576)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run three elementwise passes over 256 MiB (reads 256 MiB, writes 256 MiB each): the known-size "
                          "kernel that hardware byte counters of a profiled run are scaled by")
@@ -248,7 +265,7 @@ def main():
         model_workload(args, dev)
         return
     T = args.tokens
-    q, k, v = make_stream(T, 0, dev)
+    q, k, v = make_stream(T, 0, dev, args.favour)
     torch.cuda.synchronize()
 
     for _ in range(args.warmup):
@@ -276,8 +293,9 @@ def main():
         "value": T * args.steps / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"config 2: one InfLLM layer, {T}-token stream, exc 512, H32/Hkv8/D128, "
-                               f"n_init128 n_local4096 bs128 topk16 repr_topk4 max_cached{KNOBS['max_cached_block']} lru, GMM keys",
+        "config": {"workload": f"{'config 5' if args.favour else 'config 2'}: one InfLLM layer, {T}-token stream, exc 512, H32/Hkv8/D128, "
+                               f"n_init128 n_local4096 bs128 topk16 repr_topk4 max_cached{KNOBS['max_cached_block']} lru, GMM keys"
+                               + (f", queries favour {args.favour} components per block" if args.favour else ""),
                    "append_chunk": args.chunk},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": LOCAL_STAGE_HBM_BYTES,

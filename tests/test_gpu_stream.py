@@ -149,6 +149,16 @@ def test_unaligned_geometry_and_batch():
     _compare(700, [333, 367], H=6, Hkv=3, base=1e4, seed=7, B=2, **kw)
 
 
+def test_many_batch_rows_take_the_host_built_page_table():
+    """More than 64 selected (row, unit) pairs per block: the page table no longer fits a kernel argument and
+    is staged through pinned memory instead."""
+    # repr_topk = block_size: the representative is the plain mean of the unit's keys, so this test exercises the
+    # page-table path without depending on near-ties among 16 noisy token scores
+    kw = dict(n_init=8, n_local=128, block_size=16, max_cached_block=16, topk=16, exc_block_size=32, repr_topk=16)
+    cm, ora, _ = _compare(600, [300, 300], H=4, Hkv=2, base=1e4, seed=18, B=5, **kw)
+    assert cm.num_global_block > kw["topk"] and cm.num_units * kw["topk"] > 64
+
+
 def test_no_gqa_and_perhead():
     kw = dict(SMALL, perhead=True)
     _compare(800, [800], H=2, Hkv=1, base=1e4, seed=8, **kw)
@@ -199,6 +209,61 @@ def test_state_export_and_injection_resume_the_stream_exactly():
     resumed = cm_b.append(qd, kd, vd, qd, kd, vd).cpu()
     assert torch.equal(resumed, full[:, :, sl])
     assert cm_b.length == T0 + T1 == cm1.length and cm_b.num_global_block == cm1.num_global_block
+
+
+def test_full_size_stream_one_block_against_the_oracle_from_exported_state():
+    """BASELINE config 2 at full size (131,072 tokens, Mistral geometry, mixture keys).  The whole stream is too long
+    for the CPU oracle, so: closed forms for the state, and ONE execution block (the last) recomputed on the CPU
+    in fp32 from the state exported just before it - its retrieval set by brute force over all 990 representatives,
+    its output through oracle.multistage with window-relative RoPE (small angles, as the reference forms them)."""
+    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
+    from oracle.multistage import MultiStageOracle
+    H, Hkv, T, exc, n_local, n_init, bs, topk = 32, 8, 131072, 512, 4096, 128, 128, 16
+    base = 1e6
+    q, k, v = _stream(T, H, Hkv, seed=100)
+    rope = RotaryEmbeddingESM(D, base=base, device="cuda")
+    cm = ContextManager(rope, n_init, n_local, bs, 32, topk, exc, None, False, 4, "lru", None, True)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    T0 = T - exc
+    for st in range(0, T0, 8192):
+        sl = slice(st, min(st + 8192, T0))
+        cm.append(qd[:, :, sl], kd[:, :, sl], vd[:, :, sl], qd[:, :, sl], kd[:, :, sl], vd[:, :, sl])
+    state = cm.export_state()
+    n_units = (T0 - n_init - n_local) // bs
+    assert state["n_units"] == n_units == cm.num_global_block and state["init_len"] == n_init
+    n_tail = state["tail_k"].shape[2]
+    assert n_tail == T0 - n_init - n_units * bs and n_local <= n_tail < n_local + bs
+    assert torch.equal(state["tail_k"].cpu(), k[:, :, T0 - n_tail:T0])
+    cm.record_trace = True
+    sl = slice(T0, T)
+    got = cm.append(qd[:, :, sl], kd[:, :, sl], vd[:, :, sl], qd[:, :, sl], kd[:, :, sl], vd[:, :, sl]).cpu()
+    chosen = cm.trace_blocks[-1]["selected"][0]
+    assert cm.length == T and cm.num_global_block == (T - n_init - n_local) // bs == 991
+
+    ora_rope = RopeOracle(D, base=base)
+    qb, kb, vb = q[:, :, sl].float(), k[:, :, sl].float(), v[:, :, sl].float()
+    gq = ora_rope.one_angle(qb, n_local)
+    # retrieval: top-16 of sum_h mean-query_h . representative_h over every unit (context_manager.py:366-383)
+    scores = state["reps"][0].float().cpu().double() @ gq[0].mean(dim=1).reshape(-1).double()
+    want = set(scores.topk(topk).indices.tolist())
+    kth = float(scores.topk(topk).values[-1])
+    assert all(abs(float(scores[i]) - kth) <= TIE_REL * abs(kth) for i in set(chosen) ^ want), (sorted(chosen), sorted(want))
+    # attention of the block: local window (relative RoPE) + [chosen units | init | overflow remainder] (un-rotated)
+    tail_k, tail_v = state["tail_k"].float().cpu(), state["tail_v"].float().cpu()
+    all_k, all_v = torch.cat((tail_k, kb), dim=2), torch.cat((tail_v, vb), dim=2)
+    win_k, win_v = all_k[:, :, -(n_local + exc):], all_v[:, :, -(n_local + exc):]
+    q_rot, k_rot = ora_rope.window(qb, win_k)
+    attn = MultiStageOracle(qb.shape)
+    attn.append(q_rot, k_rot, win_v, sliding_window=n_local)
+    overflow = max(n_tail + exc - n_local, 0)
+    units = state["units"]
+    glob_k = torch.cat([units[u][:, 0].float().cpu() for u in sorted(chosen)] + [state["init_k"].float().cpu(), tail_k[:, :, :overflow]], dim=2)
+    glob_v = torch.cat([units[u][:, 1].float().cpu() for u in sorted(chosen)] + [state["init_v"].float().cpu(), tail_v[:, :, :overflow]], dim=2)
+    assert glob_k.shape[2] == topk * bs + n_init + overflow
+    attn.append(gq, glob_k, glob_v, end=True, sliding_window=(n_local + glob_k.shape[2], n_local), complement_sliding_window=True)
+    want_out, _ = attn.get_result()
+    err = (got.float() - want_out).abs()
+    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (float(err.max()), float(err.mean()))
 
 
 def test_decode_steps_follow_oracle():
