@@ -499,7 +499,7 @@ class ContextManager:
         return out
 
     # ------------------------------------------------------- state in / out
-    # The reference keeps its state only in the live object (SURVEY appendix B lists the fields); these two
+    # The reference keeps its state only in the live object (context_manager.py:292-363); these two
     # methods let a harness start from a prepared memory (e.g. 8192 units with representatives) or resume.
     def export_state(self):
         """Snapshot after an append(): everything a fresh ContextManager needs to continue the stream."""
