@@ -288,6 +288,11 @@ typedef struct {
     double distance_scale;
     float softmax_scale;
     int32_t reserved;
+    /* Optional (both or neither): one pinned int32, as the device sees it and as the host sees it.  With
+     * h_topk_idx == NULL the selection kernel stores a sequence number there after the ids, and
+     * infllm_layer_wait_topk polls it instead of sleeping on an event (falls back to the event after 2 ms). */
+    int32_t *d_topk_flag;
+    const volatile int32_t *h_topk_flag;
 } infllm_layer_desc;
 
 void *infllm_layer_create(const infllm_layer_desc *desc);    /* NULL + infllm_last_error() on failure */

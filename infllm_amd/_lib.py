@@ -74,6 +74,7 @@ class LayerDesc(C.Structure):
         ("d_pages", c_vp), ("h_pages", c_vp), ("max_pages", c_i32), ("page_slots", c_i32),
         ("d_carve_stage", c_vp), ("max_carve", c_i32), ("carve_slots", c_i32),
         ("d_inv_freq", c_vp), ("distance_scale", c_f64), ("softmax_scale", c_f32), ("reserved", c_i32),
+        ("d_topk_flag", c_vp), ("h_topk_flag", c_vp),
     ]
 
 

@@ -219,6 +219,10 @@ class ContextManager:
         d.h_topk_idx = None
         if not d.d_topk_idx:
             d.d_topk_idx, d.h_topk_idx = self.topk_idx.data_ptr(), self.topk_idx_host.data_ptr()
+        else:                                      # the host polls a sequence number stored behind the ids
+            self.topk_flag_host = torch.zeros((16,), dtype=torch.int32, pin_memory=True)
+            d.d_topk_flag = self._lib.infllm_host_device_pointer(self.topk_flag_host.data_ptr())
+            d.h_topk_flag = self.topk_flag_host.data_ptr() if d.d_topk_flag else None
         d.d_pages, d.h_pages = self.pages_dev.data_ptr(), self.pages_host.data_ptr()
         d.max_pages, d.page_slots = self.max_pages, _PAGE_SLOTS
         d.d_carve_stage, d.max_carve, d.carve_slots = self.carve_stage.data_ptr(), self.max_carve, _CARVE_SLOTS

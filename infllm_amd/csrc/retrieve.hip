@@ -141,7 +141,18 @@ __device__ int block_exclusive_scan(int v, int *wave_tot, int *total) {
     return base + incl - v;
 }
 
-__global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, int N, int k, int32_t *idx_out) {
+// Both selection kernels can end by publishing a sequence number next to the ids (flag may be NULL): every
+// thread fences its id stores to system scope, the workgroup meets, then one thread stores the number.  A host
+// that polls the (pinned) flag sees the ids no later than the number.
+__device__ __forceinline__ void publish(int32_t *flag, int32_t value) {
+    if (!flag) return;
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+__global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *flag,
+                                                           int32_t flag_value) {
     __shared__ int hist[256];
     __shared__ int wave_tot[kSelThreads / 64];
     __shared__ uint32_t sh_prefix;
@@ -189,6 +200,7 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
         eq_base += tot_eq;
         out_base += tot_sel;
     }
+    publish(flag, flag_value);
 }
 
 // Tables of up to 16384 scores: every thread keeps its R consecutive keys in registers, so the scores are read
@@ -196,7 +208,8 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
 // many LDS counters) find the key of the k-th largest; a pass whose bucket is wanted whole ends the search.
 // Output contract as above: indices ascending, lowest indices among keys equal to the k-th.
 template <int R>
-__global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *scores, int N, int k, int32_t *idx_out) {
+__global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *flag,
+                                                                int32_t flag_value) {
     __shared__ __align__(16) int hist[4096];
     __shared__ int wave_tot[kSelThreads / 64];
     __shared__ uint32_t sh_prefix;
@@ -282,6 +295,7 @@ __global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *sco
             ++e_before;
         }
     }
+    publish(flag, flag_value);
 }
 
 // ---------------------------------------------------------------- representative keys
@@ -360,12 +374,19 @@ extern "C" int infllm_unit_scores(const void *d_reps, int64_t rep_stride, int32_
     return 0;
 }
 
+int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+
 extern "C" int infllm_topk(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, void *stream) {
+    return infllm_topk_publish(d_scores, N, k, d_idx, nullptr, 0, stream);
+}
+
+// library-internal: the selection followed by `*d_flag = flag_value` (system scope) once the ids are written
+int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream) {
     INFLLM_REQUIRE(d_scores && d_idx, "topk: null pointer");
     INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && k <= 1024, "topk: k=%d with N=%d", k, N);
     const hipStream_t st = (hipStream_t)stream;
     switch (N <= 16384 ? (N + kSelThreads - 1) / kSelThreads : 0) {       // keys per thread
-#define REGS_CASE(r) hipLaunchKernelGGL(topk_regs_kernel<r>, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx); break
+#define REGS_CASE(r) hipLaunchKernelGGL(topk_regs_kernel<r>, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_flag, flag_value); break
     case 1: REGS_CASE(1);
     case 2: REGS_CASE(2);
     case 3: REGS_CASE(3);
@@ -376,7 +397,7 @@ extern "C" int infllm_topk(const float *d_scores, int32_t N, int32_t k, int32_t 
     case 11: case 12: REGS_CASE(12);
     case 13: case 14: case 15: case 16: REGS_CASE(16);
 #undef REGS_CASE
-    default: hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx);
+    default: hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_flag, flag_value);
     }
     INFLLM_CHECK_LAUNCH("topk");
     return 0;

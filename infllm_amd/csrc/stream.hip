@@ -2,6 +2,8 @@
 // (inf_llm/attention/context_manager.py:474-545, 614-679): the launches of a block are
 // issued natively, back to back, so that the host interpreter is not on the GPU's
 // critical path.  Decisions (which units are cached, what gets carved) stay with the caller.
+#include <atomic>
+#include <chrono>
 #include <vector>
 
 #include "common.h"
@@ -36,6 +38,7 @@ struct Layer {
     int page_cur = 0, carve_cur = 0;
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
+    int32_t topk_seq = 0;
     bool has_global = false;
     bool topk_pending = false;
     int slot = 0;                         // workspace slot written last
@@ -67,6 +70,10 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
     __syncthreads();
     if (threadIdx.x == 0) out[idx] = (red[0] + red[1]) + (red[2] + red[3]);
 }
+
+}  // namespace
+int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+namespace {
 
 int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
     const int G = d.H / d.Hkv;
@@ -325,8 +332,13 @@ int run_unit_scores(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_su, 
 int run_topk(Layer *L, const float *scores, int64_t scores_sb, int n_units, void *stream) {
     const infllm_layer_desc &d = L->d;
     hipStream_t st = (hipStream_t)stream;
+    // the last row's kernel also publishes a sequence number the host can poll (kernels of a stream finish in order)
+    const bool poll = d.d_topk_flag && d.h_topk_flag && !d.h_topk_idx;
+    if (poll) ++L->topk_seq;
     for (int u = 0; u < d.B; ++u) {
-        int rc = infllm_topk(scores + (int64_t)u * scores_sb, n_units, d.topk, d.d_topk_idx + (int64_t)u * d.topk, stream);
+        const bool last = poll && u == d.B - 1;
+        int rc = infllm_topk_publish(scores + (int64_t)u * scores_sb, n_units, d.topk, d.d_topk_idx + (int64_t)u * d.topk,
+                                     last ? d.d_topk_flag : nullptr, L->topk_seq, stream);
         if (rc) return rc;
     }
     if (d.h_topk_idx)      // NULL: d_topk_idx is itself host-visible pinned memory, the kernel wrote there
@@ -424,6 +436,21 @@ extern "C" int infllm_layer_wait_topk(void *layer) {
     INFLLM_REQUIRE(layer, "layer_wait_topk: null layer");
     Layer *L = (Layer *)layer;
     if (!L->topk_pending) return 0;
+    if (L->d.d_topk_flag && L->d.h_topk_flag && !L->d.h_topk_idx) {
+        // poll the pinned sequence number for a while: waking up from an event wait costs tens of microseconds,
+        // and this wait sits on the chain from one block's selection to the next
+        const volatile int32_t *flag = L->d.h_topk_flag;
+        const auto t0 = std::chrono::steady_clock::now();
+        for (uint32_t spins = 0; *flag != L->topk_seq; ++spins) {
+            if ((spins & 1023u) == 1023u && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) break;
+            __builtin_ia32_pause();
+        }
+        if (*flag == L->topk_seq) {
+            std::atomic_thread_fence(std::memory_order_acquire);
+            L->topk_pending = false;
+            return 0;
+        }
+    }
     HIP_OK(hipEventSynchronize(L->topk_done), "layer_wait_topk");
     L->topk_pending = false;
     return 0;
