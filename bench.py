@@ -218,7 +218,7 @@ def cpu_baseline(tokens, threads):
     ora.append(q, k, v)
     dt = time.perf_counter() - t0
     return dict(value=tokens / dt, unit="tokens/s", cores=threads, kind="port",
-                sample=f"first {tokens} tokens of the same stream shape (config 1 size), fp32 oracle, {dt:.1f} s")
+                sample=f"first {tokens} tokens of the same stream shape (config 1 is 16384), fp32 oracle, {dt:.1f} s")
 
 
 def main():
@@ -228,7 +228,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--chunk", type=int, default=8192, help="tokens per append() call")
-    ap.add_argument("--cpu-tokens", type=int, default=16384, help="0 disables the CPU baseline")
+    ap.add_argument("--cpu-tokens", type=int, default=32768, help="0 disables the CPU baseline")
     ap.add_argument("--workload", choices=["prefill", "decode", "model"], default="prefill",
                     help="prefill = the headline 128K-token stream (config 2); decode = config 3, model = config 4 "
                          "(each with its own JSON line)")
