@@ -50,21 +50,29 @@ __device__ __forceinline__ int floordiv64(int64_t x) { return (int)(x >> 6); }  
 // layout is decided:
 //   Ks[buf][R][16 chunks]  LDS row R holds key k_lds_row(R) (bits 2 and 3 swapped inside each 32-key
 //                          half, so the lane that owns MFMA row r reads LDS row r); chunk c of the row
-//                          sits at position c ^ swz(R), so the 8 rows read together hit 8 bank groups.
+//                          sits at position c ^ swz(R).  The LDS serves 256 bytes per cycle from 64 banks: a
+//                          16-byte read is conflict free when the 16 lanes of a quarter wave hit 16 different
+//                          chunk positions, an 8-byte transposing read when the 32 lanes of a half wave hit 32
+//                          different 8-byte slots; swz() is a permutation of the 4 low row bits that gives both
+//                          (K: 16 consecutive rows, one chunk each; V: 4 rows x 4 chunks x 2 halves).
 //   Vs[buf][R][16 chunks]  natural rows, same swizzle; the V^T operand of the second MFMA is formed by
 //                          the transposing read ds_read_b64_tr_b16: in a group of 16 lanes, lane 4*j + q
 //                          supplies the address of 4 consecutive d of key j, and lane i receives element
 //                          i of keys j = 0..3, i.e. 4 consecutive keys at one d.
 __device__ __forceinline__ int k_lds_row(int key) { return (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1); }
-__device__ __forceinline__ int swz(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
+__device__ __forceinline__ int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ s16x4 lds_read_tr(const bf16_t *p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
 }
+// Issued as inline assembly on purpose.  With the builtin, the compiler tracks the transfer as an LDS store that
+// may alias every later LDS read and puts `s_waitcnt vmcnt(0)` in front of the first operand read of the tile being
+// multiplied - which waits for the tiles just requested for LATER and serialises load and math completely.  The
+// kernel orders the transfers itself: vmcnt(0) and a barrier before a buffer is read, a barrier before it is refilled.
 __device__ __forceinline__ void load_to_lds16(const bf16_t *g, bf16_t *lds_wave_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
-                                     (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+    const uint32_t lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(g) : "memory", "m0");
 }
 
 constexpr int kTileBytes = kTile * kD * 2;        // one K (or V) tile in LDS
@@ -195,11 +203,21 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         v_head = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh;
         ring_row = ((int64_t)g_t0 * kTile) % a.cap;
     }
+    // The page table is read through the constant address space: the index is wave-uniform, so these become scalar
+    // loads.  As vector loads they would share the vmcnt counter with the tile transfers, and waiting for a page
+    // entry would wait for every tile in flight.  The table is written by an earlier kernel and is read-only here.
+    const __attribute__((address_space(4))) infllm_page *page_table =
+        (const __attribute__((address_space(4))) infllm_page *)(uintptr_t)a.d_pages;
     auto load_tile = [&](int t, int buf) {
         const bf16_t *kbase, *vbase;
         int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
         if (PAGED) {
-            const infllm_page pg = a.d_pages[(int64_t)b * a.n_pages + t];
+            const __attribute__((address_space(4))) infllm_page *entry = page_table + ((int64_t)b * a.n_pages + t);
+            infllm_page pg;
+            pg.k = entry->k;
+            pg.v = entry->v;
+            pg.head_stride = entry->head_stride;
+            pg.n_valid = entry->n_valid;
             kbase = (const bf16_t *)pg.k + (int64_t)g * pg.head_stride;
             vbase = (const bf16_t *)pg.v + (int64_t)g * pg.head_stride;
             row_lo = 0;
@@ -280,7 +298,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         int row_lo = 0, row_hi = kTile;
         int d0 = 0;                            // dist of (this lane's query, key 0 of the tile)
         if (PAGED) {
-            row_hi = a.d_pages[(int64_t)b * a.n_pages + t].n_valid;
+            row_hi = page_table[(int64_t)b * a.n_pages + t].n_valid;
             need_mask = row_hi < kTile;
         } else {
             const int64_t j0 = (int64_t)t * kTile;
@@ -402,6 +420,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     }
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // The compiler does not know that the wait above also covered the query rows; passing them through an empty
+    // asm makes it place its own wait for them HERE rather than in front of their first use inside the loop,
+    // where a vmcnt(0) would wait for the tiles in flight.
+#pragma unroll
+    for (int kk = 0; kk < kD / 16; ++kk) asm volatile("" : "+v"(qreg[kk]));
     __syncthreads();
     for (int t = g_t0; t < g_t1; t += 2) {
         const int buf = (t - g_t0) & 3;                          // 0 or 2
