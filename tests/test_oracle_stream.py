@@ -273,3 +273,24 @@ def test_chunked_retrieval_changes_selections_but_not_the_attention_rule():
     assert [b["selected"] for b in cm_p.block_trace] == picks
     assert torch.equal(out_c, out_p)
     assert [b["selected"] for b in _run(q, k, v, calls)[1].block_trace] != picks      # and the chunking mattered here
+
+
+# ------------------------------------------------------------- frozen oracle outputs
+def test_oracle_still_produces_its_frozen_vectors():
+    """tests/golden/oracle_small.npz holds what the oracle computed on seeded inputs when its pins passed (they are
+    not reference outputs: the reference has none); an edit that changes the oracle's results must be deliberate."""
+    import importlib.util
+    import os
+    import numpy as np
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_vectors", os.path.join(here, "make_vectors.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    frozen = np.load(os.path.join(here, "oracle_small.npz"))
+    fresh = mod.vectors()
+    assert sorted(frozen.files) == sorted(fresh)
+    for name in frozen.files:
+        if fresh[name].dtype.kind == "f":
+            assert np.allclose(frozen[name], fresh[name], atol=1e-5), name
+        else:
+            assert np.array_equal(frozen[name], fresh[name]), name
