@@ -143,7 +143,8 @@ int infllm_attn_stage(const infllm_attn_args *a, void *stream);
 /* Joint softmax across stages/splits (torch_impl.py:15-36):
  * o = sum_p 2^(lse_p - LSE) o_p, LSE = log2 sum_p 2^lse_p.
  * d_o_part [P,B,H,Lq,128], d_lse_part [P,B,H,Lq] -> d_out bf16 [B,H,Lq,128]
- * (strides given), d_lse fp32 [B,H,Lq]. */
+ * (strides given), d_lse fp32 [B,H,Lq].  d_lse may be NULL (output only); d_out may be NULL (log-sum-exp
+ * only, a much smaller launch: the scores of infllm_local_score need nothing else). */
 int infllm_attn_merge(const float *d_o_part, const float *d_lse_part, int32_t P,
                       int32_t B, int32_t H, int32_t Lq,
                       void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl,

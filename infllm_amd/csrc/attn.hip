@@ -505,6 +505,18 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float *o_part, co
     if (c == 0 && lse_out) lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
 }
 
+// the log-sum-exp half of the merge alone: one thread per row
+__global__ __launch_bounds__(256) void attn_merge_lse_kernel(const float *lse_part, int P, int64_t rows, float *lse_out) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= rows) return;
+    float m = -INFINITY;
+    for (int p = 0; p < P; ++p) m = fmaxf(m, lse_part[p * rows + row]);
+    float den = 0.f;
+    if (m > -INFINITY)
+        for (int p = 0; p < P; ++p) den += __builtin_amdgcn_exp2f(lse_part[p * rows + row] - m);
+    lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
+}
+
 }  // namespace
 
 extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
@@ -550,9 +562,17 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
 extern "C" int infllm_attn_merge(const float *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
                                  int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
                                  void *stream) {
-    INFLLM_REQUIRE(d_o_part && d_lse_part && d_out, "attn_merge: null pointer");
+    INFLLM_REQUIRE(d_o_part && d_lse_part, "attn_merge: null pointer");
     INFLLM_REQUIRE(P >= 1 && B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes P=%d B=%d H=%d Lq=%d", P, B, H, Lq);
     INFLLM_REQUIRE((o_sl % 4 | o_sh % 4 | o_sb % 4) == 0, "attn_merge: output strides must be multiples of 4");
+    if (!d_out) {                                     // log-sum-exp only
+        INFLLM_REQUIRE(d_lse, "attn_merge: neither output nor lse requested");
+        const int64_t rows = (int64_t)B * H * Lq;
+        hipLaunchKernelGGL(attn_merge_lse_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d_lse_part, P,
+                           rows, d_lse);
+        INFLLM_CHECK_LAUNCH("attn_merge (lse)");
+        return 0;
+    }
     const int64_t threads = (int64_t)B * H * Lq * 32;
     hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                        d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);

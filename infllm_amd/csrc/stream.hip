@@ -610,7 +610,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         }
         parts += at.nsplit;
     }
-    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, d.d_lse, stream);
+    // only the joint log-sum-exp is needed by what follows on the way to the next selection; the output rows are
+    // merged once that selection is out (step 5b)
+    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, nullptr, 0, 0, 0, d.d_lse, stream);
     if (rc) return rc;
 
     // ---- 3b. attention mass each selected unit received (only the score-decay policy asks for it)
@@ -673,6 +675,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, n_units_next, stream);
         if (rc) return rc;
     }
+    // ---- 5b. the block's output rows
+    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, nullptr, stream);
+    if (rc) return rc;
     // ---- 6. off the critical path: the rest of the local score, new units to pinned host memory
     rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, stream);
     if (rc) return rc;
