@@ -484,16 +484,32 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float *o_part, co
     const int64_t row = e >> 5;
     const int c = (int)(e & 31);
     if (row >= rows) return;
+    // partials in batches of 8 so that the loads of a batch are in flight together (decode-sized blocks merge
+    // dozens of partials of very few rows: a chain of dependent loads would be all latency)
     float m = -INFINITY;
-    for (int p = 0; p < P; ++p) m = fmaxf(m, lse_part[p * rows + row]);
+    for (int p0 = 0; p0 < P; p0 += 8) {
+        float l8[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) l8[i] = p0 + i < P ? lse_part[(p0 + i) * rows + row] : -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m = fmaxf(m, l8[i]);
+    }
     f32x4 acc{0.f, 0.f, 0.f, 0.f};
     float den = 0.f;
     if (m > -INFINITY) {
-        for (int p = 0; p < P; ++p) {
-            float w = __builtin_amdgcn_exp2f(lse_part[p * rows + row] - m);
-            if (w > 0.f) {
-                f32x4 o = *(const f32x4 *)(o_part + (p * rows + row) * kD + c * 4);
-                acc += o * w;
+        for (int p0 = 0; p0 < P; p0 += 8) {
+            float l8[8];
+            f32x4 o8[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const bool on = p0 + i < P;
+                l8[i] = on ? lse_part[(p0 + i) * rows + row] : -INFINITY;
+                o8[i] = on ? *(const f32x4 *)(o_part + ((p0 + i) * rows + row) * kD + c * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float w = __builtin_amdgcn_exp2f(l8[i] - m);       // exp2(-inf) = 0: empty partials hold zeros
+                acc += o8[i] * w;
                 den += w;
             }
         }
@@ -509,11 +525,20 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float *o_part, co
 __global__ __launch_bounds__(256) void attn_merge_lse_kernel(const float *lse_part, int P, int64_t rows, float *lse_out) {
     const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (row >= rows) return;
-    float m = -INFINITY;
-    for (int p = 0; p < P; ++p) m = fmaxf(m, lse_part[p * rows + row]);
-    float den = 0.f;
-    if (m > -INFINITY)
-        for (int p = 0; p < P; ++p) den += __builtin_amdgcn_exp2f(lse_part[p * rows + row] - m);
+    float m = -INFINITY, den = 0.f;
+    for (int p0 = 0; p0 < P; p0 += 8) {                 // online over batches of 8 independent loads
+        float l8[8], m8 = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) l8[i] = p0 + i < P ? lse_part[(p0 + i) * rows + row] : -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m8 = fmaxf(m8, l8[i]);
+        if (m8 == -INFINITY) continue;
+        const float m_new = fmaxf(m, m8);
+        den *= __builtin_amdgcn_exp2f(m - m_new);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) den += __builtin_amdgcn_exp2f(l8[i] - m_new);
+        m = m_new;
+    }
     lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
 }
 

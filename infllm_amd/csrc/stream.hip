@@ -79,8 +79,16 @@ int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
     const int G = d.H / d.Hkv;
     const int wgs = (((n_queries + 31) / 32) * G + 7) / 8 * d.Hkv * d.B;      // 8 wave tasks per workgroup
     int want = (d.num_cus + wgs - 1) / wgs;                                      // one workgroup per CU (LDS bound)
-    int cap = n_tiles / 8;
-    int s = want < d.max_splits ? want : d.max_splits;
+    int cap = n_tiles / 8, limit = d.max_splits;
+    if (n_queries <= 32) {
+        // decode-sized blocks: the stage is a read of K/V, bound by how many workgroups pull on HBM at once, so a
+        // workgroup may get as little as one tile pair; the partials still fit: 2 * limit * n_queries rows of the
+        // 2 * max_splits * exc the caller allocated
+        cap = n_tiles / 2;
+        const int room = d.max_splits * d.exc / n_queries;
+        limit = room < 32 ? room : 32;
+    }
+    int s = want < limit ? want : limit;
     if (s > cap) s = cap;
     return s < 1 ? 1 : s;
 }
