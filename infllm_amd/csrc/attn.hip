@@ -72,7 +72,11 @@ __device__ __forceinline__ s16x4 lds_read_tr(const bf16_t *p) {
 // kernel orders the transfers itself: vmcnt(0) and a barrier before a buffer is read, a barrier before it is refilled.
 __device__ __forceinline__ void load_to_lds16(const bf16_t *g, bf16_t *lds_wave_base) {
     const uint32_t lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)lds_wave_base);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds), "v"(g) : "memory", "m0");
+    uint32_t saved_m0;                    // M0 is the compiler's to manage: put back what it held
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
+                 : "s"(lds), "v"(g)
+                 : "memory");
 }
 
 constexpr int kTileBytes = kTile * kD * 2;        // one K (or V) tile in LDS
