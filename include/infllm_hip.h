@@ -105,7 +105,8 @@ int infllm_rope_rows(const void *d_x, int64_t sb, int64_t sh, int64_t sl, int32_
  * or from a page table of 64-key tiles (memory units, init tokens, overflow
  * remainder: context_manager.py:386-451), all keys of which are visible.
  * Output: per split s, un-merged partial results
- *      o_part [nsplit,B,H,Lq,128] fp32 (normalised by the split's own sum)
+ *      o_part [nsplit,B,H,Lq,128] fp16 bit patterns (normalised by the split's own sum, so bounded by
+ *                                 max |v|; 11 significant bits against the 8 of the bf16 result)
  *      lse_part [nsplit,B,H,Lq]   fp32 (base-2 log-sum-exp of scaled logits)
  */
 typedef struct {
@@ -135,17 +136,17 @@ typedef struct {
     int32_t n_pages;
     int32_t nsplit;
     float softmax_scale;           /* 1/sqrt(128) */
-    float *d_o_part;
+    uint16_t *d_o_part;            /* fp16 */
     float *d_lse_part;
 } infllm_attn_args;
 int infllm_attn_stage(const infllm_attn_args *a, void *stream);
 
 /* Joint softmax across stages/splits (torch_impl.py:15-36):
  * o = sum_p 2^(lse_p - LSE) o_p, LSE = log2 sum_p 2^lse_p.
- * d_o_part [P,B,H,Lq,128], d_lse_part [P,B,H,Lq] -> d_out bf16 [B,H,Lq,128]
- * (strides given), d_lse fp32 [B,H,Lq].  d_lse may be NULL (output only); d_out may be NULL (log-sum-exp
+ * d_o_part fp16 [P,B,H,Lq,128], d_lse_part [P,B,H,Lq] -> d_out bf16 [B,H,Lq,128]
+ * (strides given, multiples of 8 elements), d_lse fp32 [B,H,Lq].  d_lse may be NULL (output only); d_out may be NULL (log-sum-exp
  * only, a much smaller launch: the scores of infllm_local_score need nothing else). */
-int infllm_attn_merge(const float *d_o_part, const float *d_lse_part, int32_t P,
+int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P,
                       int32_t B, int32_t H, int32_t Lq,
                       void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
                       float *d_lse, void *stream);
@@ -276,7 +277,8 @@ typedef struct {
     void *d_q_loc, *d_q_glb;                          /* [2][B*H*exc*128] */
     float *d_qbar;                                    /* [2][B,H*128] */
     float *d_qpart;                                   /* [2][B,ceil(exc/16),H*128] */
-    float *d_o_part, *d_lse_part, *d_lse;             /* [2*max_splits,B,H,exc,(128)], [B,H,exc] */
+    uint16_t *d_o_part;                               /* fp16 [2*max_splits,B,H,exc,128] */
+    float *d_lse_part, *d_lse;                        /* [2*max_splits,B,H,exc], [B,H,exc] */
     int32_t *d_topk_idx, *h_topk_idx;                 /* [B,topk] device / pinned host; h_topk_idx may be NULL when
                                                          d_topk_idx is the device-visible address of pinned memory:
                                                          the top-k kernel then writes the ids where the host reads them */

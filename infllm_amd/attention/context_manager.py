@@ -186,7 +186,7 @@ class ContextManager:
         self.qbar = torch.empty((2, B, H * D), **f32)
         self.qpart = torch.empty((2, B, (exc + 15) // 16, H * D), **f32)
         n_part = 2 * _MAX_SPLITS
-        self.o_part = torch.empty((n_part * B * H * exc * D,), **f32)
+        self.o_part = torch.empty((n_part * B * H * exc * D,), dtype=torch.float16, device=self.device)
         self.lse_part = torch.empty((n_part * B * H * exc,), **f32)
         self.lse = torch.empty((B * H * exc,), **f32)
         self.topk_idx = torch.zeros((B, max(topk, 1)), dtype=torch.int32, device=dev)

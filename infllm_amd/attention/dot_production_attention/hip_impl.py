@@ -40,7 +40,7 @@ class HipMultiStageDotProductionAttention(MultiStageDotProductionAttention):
                 sliding_window = (len_k - Lq, sliding_window)
             offset, window = int(sliding_window[0]), int(sliding_window[1])
             mask = ops.MASK_COMPLEMENT if complement_sliding_window else ops.MASK_WINDOW
-        o_part = torch.empty((1, B, H, Lq, D), dtype=torch.float32, device=q.device)
+        o_part = torch.empty((1, B, H, Lq, D), dtype=torch.float16, device=q.device)
         lse_part = torch.empty((1, B, H, Lq), dtype=torch.float32, device=q.device)
         ops.attn_stage_linear(q, k, v, o_part, lse_part, j_lo=0, j_hi=len_k, mask=mask, offset=offset, window=window)
         self._o_parts.append(o_part)

@@ -44,6 +44,27 @@ __device__ __forceinline__ StageRange visible_range(const infllm_attn_args &a, i
 
 __device__ __forceinline__ int floordiv64(int64_t x) { return (int)(x >> 6); }   // arithmetic shift = floor
 
+// Division by a launch constant without the divide: q = (n * mul) >> shift is exact for every n < 2^31 when
+// mul = floor(2^shift / d) + 1 and shift = 31 + ceil(log2 d) (the excess mul*d - 2^shift is at most d <= 2^ceil(log2 d),
+// so the error term n * excess / (d * 2^shift) stays below 1/d).  The kernel's set-up is a chain of such divisions on
+// the critical path of a workgroup that lives for only a handful of tiles; a hardware-less 64-bit divide costs
+// some two hundred instructions.
+struct FastDiv {
+    uint32_t d, mul, shift;
+};
+inline FastDiv fast_div(uint32_t d) {
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    return FastDiv{d, (uint32_t)((1ull << (31 + l)) / d + 1), 31 + l};
+}
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f) { return (uint32_t)(((uint64_t)n * f.mul) >> f.shift); }
+
+// launch constants the kernel would otherwise derive with divisions
+struct StageGeom {
+    FastDiv gx, gy, hkv, group, nsplit, cap_tiles;
+    int32_t n_tasks;
+};
+
 // LDS layouts.  Tiles go from global memory straight into LDS (global_load_lds_dwordx4: lane l of a
 // wave deposits its 16 bytes at base + 16*l, so one instruction fills 4 rows of 256 bytes), which leaves
 // no staging registers; which 16-byte chunk of which row a lane FETCHES is free, and that is where the
@@ -88,14 +109,14 @@ struct IntC {
 };
 
 template <bool PAGED>
-__global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a) {
+__global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a, StageGeom geo) {
     extern __shared__ __attribute__((aligned(16))) char lds_dyn[];      // kStages K tiles, then kStages V tiles
     char *const Ks = lds_dyn, *const Vs = lds_dyn + kStages * kTileBytes;
     __shared__ int wg_lo[kWaves], wg_hi[kWaves];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
-    const int G = a.H / a.Hkv;
+    const int G = (int)geo.group.d;
     // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  Renumber so that
     // one XCD runs a contiguous run of ids: the workgroups that share a (kv head, split) K/V range then sit
     // behind one L2 and that range leaves HBM once instead of once per XCD.
@@ -105,15 +126,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         if ((total & 7) == 0) {
             const int lin = bx + gx * (by + gy * bz);
             const int id = (lin & 7) * (total >> 3) + (lin >> 3);
-            bx = id % gx;
-            by = (id / gx) % gy;
-            bz = id / (gx * gy);
+            const int rest = (int)fdiv(id, geo.gx);     // id = bx + gx * (by + gy * bz)
+            bx = id - rest * gx;
+            bz = (int)fdiv(rest, geo.gy);
+            by = rest - bz * gy;
         }
     }
-    const int b = by / a.Hkv, g = by % a.Hkv;
+    const int b = (int)fdiv(by, geo.hkv), g = by - b * a.Hkv;
     const int split = bz;
-    const int n_qtiles = (a.Lq + kQTile - 1) / kQTile;
-    const int n_tasks = n_qtiles * G;
+    const int n_tasks = geo.n_tasks;
 #ifdef INFLLM_PHASES
     long long *ph = (long long *)a.d_lse_part + 1024 * 1024;     // debug build only: stamps beyond the lse partials
     int ph_n = 0;
@@ -127,7 +148,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     // ---- this wave's task and the tiles it needs
     const int task = bx * kWaves + wave;
     const bool live = task < n_tasks;
-    const int qt = live ? task / G : 0, hg = live ? task % G : 0;
+    const int qt = live ? (int)fdiv(task, geo.group) : 0, hg = live ? task - qt * G : 0;
     const int h = g * G + hg;
     const int i0 = qt * kQTile, i1 = min(i0 + kQTile, a.Lq) - 1;
 
@@ -158,9 +179,10 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     }
     if (g_t1 <= g_t0) g_t0 = g_t1 = 0;
     {
-        int64_t n = g_t1 - g_t0;
-        int t_begin = g_t0 + (int)(n * split / a.nsplit);
-        int t_end = g_t0 + (int)(n * (split + 1) / a.nsplit);
+        // share [n * split / nsplit, n * (split + 1) / nsplit) of the n tiles, in 32-bit pieces
+        const uint32_t n = (uint32_t)(g_t1 - g_t0), per = fdiv(n, geo.nsplit), rem = n - per * a.nsplit;
+        int t_begin = g_t0 + (int)(per * split + fdiv(rem * split, geo.nsplit));
+        int t_end = g_t0 + (int)(per * (split + 1) + fdiv(rem * (split + 1), geo.nsplit));
         g_t0 = t_begin;
         g_t1 = t_end;
     }
@@ -205,7 +227,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     if (!PAGED) {
         k_head = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh;
         v_head = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh;
-        ring_row = ((int64_t)g_t0 * kTile) % a.cap;
+        ring_row = (int64_t)(g_t0 - (int)(fdiv(g_t0, geo.cap_tiles) * geo.cap_tiles.d)) * kTile;
     }
     // The page table is read through the constant address space: the index is wave-uniform, so these become scalar
     // loads.  As vector loads they would share the vmcnt counter with the tile transfers, and waiting for a page
@@ -455,23 +477,27 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     const int64_t row0 = (((int64_t)split * a.B + b) * a.H + h) * a.Lq + i0;      // row of this wave's first query
     const int64_t row = row0 + col;
     {
-        char *stage = lds_dyn + wave * (kQTile * kD * 4);
+        // fp16 keeps 11 bits of a value that ends up rounded to bf16's 8, and halves what the partials cost in HBM
+        // (with few tiles per workgroup their write is a tenth of the kernel); staged rows are 256 bytes, a lane's
+        // 4-value piece is 8 bytes, and 16-byte chunks are swizzled by the row
+        char *stage = lds_dyn + wave * (kQTile * kD * 2);
 #pragma unroll
         for (int dt = 0; dt < kD / 32; ++dt)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
-                f32x4 o4{oacc[dt][4 * q4] * inv, oacc[dt][4 * q4 + 1] * inv, oacc[dt][4 * q4 + 2] * inv,
-                         oacc[dt][4 * q4 + 3] * inv};
-                const int chunk = dt * 8 + 2 * q4 + grp;                           // 16-byte piece of the row
-                *(f32x4 *)(stage + col * (kD * 4) + ((chunk ^ col) & 31) * 16) = o4;
+                const f16x4 o4{(_Float16)(oacc[dt][4 * q4] * inv), (_Float16)(oacc[dt][4 * q4 + 1] * inv),
+                               (_Float16)(oacc[dt][4 * q4 + 2] * inv), (_Float16)(oacc[dt][4 * q4 + 3] * inv)};
+                const int chunk = dt * 4 + q4;                                     // 16-byte chunk of the row; grp picks its half
+                *(f16x4 *)(stage + col * (kD * 2) + ((chunk ^ col) & 15) * 16 + grp * 8) = o4;
             }
         const int rows_left = a.Lq - i0;                                           // valid queries of this tile
-        const int piece = lane & 31;
+        const int piece = lane & 15;
+        _Float16 *o_part = (_Float16 *)a.d_o_part;
 #pragma unroll
-        for (int k2 = 0; k2 < kQTile / 2; ++k2) {
-            const int qr = 2 * k2 + (lane >> 5);
-            const f32x4 o4 = *(const f32x4 *)(stage + qr * (kD * 4) + ((piece ^ qr) & 31) * 16);
-            if (qr < rows_left) *(f32x4 *)(a.d_o_part + (row0 + qr) * kD + piece * 4) = o4;
+        for (int k4 = 0; k4 < kQTile / 4; ++k4) {
+            const int qr = 4 * k4 + (lane >> 4);
+            const u32x4 o8 = *(const u32x4 *)(stage + qr * (kD * 2) + ((piece ^ qr) & 15) * 16);
+            if (qr < rows_left) *(u32x4 *)(o_part + (row0 + qr) * kD + piece * 8) = o8;
         }
     }
     if (qi >= a.Lq) return;
@@ -479,14 +505,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     PH_STAMP();
 }
 
-// one thread per (row, 4 dims): P partials -> bf16 output row + final lse
-__global__ __launch_bounds__(256) void attn_merge_kernel(const float *o_part, const float *lse_part, int P, int B, int H,
+// one thread per (row, 8 dims): P fp16 partials -> bf16 output row + final lse
+__global__ __launch_bounds__(256) void attn_merge_kernel(const _Float16 *o_part, const float *lse_part, int P, int B, int H,
                                                          int Lq, bf16_t *out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
                                                          float *lse_out) {
     const int64_t rows = (int64_t)B * H * Lq;
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t row = e >> 5;
-    const int c = (int)(e & 31);
+    const int64_t row = e >> 4;
+    const int c = (int)(e & 15);
     if (row >= rows) return;
     // partials in batches of 8 so that the loads of a batch are in flight together (decode-sized blocks merge
     // dozens of partials of very few rows: a chain of dependent loads would be all latency)
@@ -498,30 +524,34 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const float *o_part, co
 #pragma unroll
         for (int i = 0; i < 8; ++i) m = fmaxf(m, l8[i]);
     }
-    f32x4 acc{0.f, 0.f, 0.f, 0.f};
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
     float den = 0.f;
     if (m > -INFINITY) {
         for (int p0 = 0; p0 < P; p0 += 8) {
             float l8[8];
-            f32x4 o8[8];
+            f16x8 o8[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const bool on = p0 + i < P;
                 l8[i] = on ? lse_part[(p0 + i) * rows + row] : -INFINITY;
-                o8[i] = on ? *(const f32x4 *)(o_part + ((p0 + i) * rows + row) * kD + c * 4) : f32x4{0.f, 0.f, 0.f, 0.f};
+                o8[i] = on ? *(const f16x8 *)(o_part + ((p0 + i) * rows + row) * kD + c * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const float w = __builtin_amdgcn_exp2f(l8[i] - m);       // exp2(-inf) = 0: empty partials hold zeros
-                acc += o8[i] * w;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[j] += (float)o8[i][j] * w;
                 den += w;
             }
         }
     }
     const float inv = den > 0.f ? 1.f / den : 0.f;
     const int i = (int)(row % Lq), h = (int)((row / Lq) % H), b = (int)(row / ((int64_t)Lq * H));
-    u32x2 packed{pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv)};
-    *(u32x2 *)(out + (int64_t)b * o_sb + (int64_t)h * o_sh + (int64_t)i * o_sl + c * 4) = packed;
+    u32x4 packed{pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv),
+                 pack_bf16x2(acc[4] * inv, acc[5] * inv), pack_bf16x2(acc[6] * inv, acc[7] * inv)};
+    *(u32x4 *)(out + (int64_t)b * o_sb + (int64_t)h * o_sh + (int64_t)i * o_sl + c * 8) = packed;
     if (c == 0 && lse_out) lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
 }
 
@@ -558,6 +588,9 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
     const int G = a->H / a->Hkv;
     const int n_tasks = ((a->Lq + kQTile - 1) / kQTile) * G;
     dim3 grid((n_tasks + kWaves - 1) / kWaves, a->B * a->Hkv, a->nsplit);
+    INFLLM_REQUIRE((int64_t)grid.x * grid.y * grid.z < (1ll << 31), "attn_stage: grid too large");
+    StageGeom geo{fast_div(grid.x), fast_div(grid.y), fast_div((uint32_t)a->Hkv), fast_div((uint32_t)G),
+                  fast_div((uint32_t)a->nsplit), fast_div(1), n_tasks};
     constexpr size_t lds_bytes = 2 * kStages * kTileBytes;
     static bool lds_set[2] = {false, false};           // dynamic LDS above 64 KiB must be enabled once per kernel
     if (a->d_pages) {
@@ -567,7 +600,7 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
             if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
             lds_set[1] = true;
         }
-        hipLaunchKernelGGL(attn_stage_kernel<true>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL(attn_stage_kernel<true>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, geo);
     } else {
         INFLLM_REQUIRE(a->j_hi <= a->j_lo || (a->d_k && a->d_v), "attn_stage: null k / v pointer");
         INFLLM_REQUIRE(a->cap > 0 && a->cap % kTile == 0, "attn_stage: cap %lld is not a positive multiple of %d",
@@ -575,6 +608,9 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
         INFLLM_REQUIRE(a->j_lo >= 0 && a->j_hi - a->j_lo <= a->cap, "attn_stage: key range [%lld,%lld) exceeds cap %lld",
                        (long long)a->j_lo, (long long)a->j_hi, (long long)a->cap);
         INFLLM_REQUIRE(a->mask >= 0 && a->mask <= 2, "attn_stage: unknown mask %d", a->mask);
+        INFLLM_REQUIRE(a->j_hi < (1ll << 36), "attn_stage: key range beyond 2^36 rows");
+        // tile indices stay below 2^30, so any ring of 2^31 tiles or more never wraps: one divisor stands for all of them
+        geo.cap_tiles = fast_div((uint32_t)std::min<int64_t>(a->cap / kTile, 1ll << 31));
         INFLLM_REQUIRE((a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8 | a->v_sl % 8 | a->v_sh % 8 | a->v_sb % 8) == 0,
                        "attn_stage: k/v strides must be multiples of 8");
         if (!lds_set[0]) {
@@ -582,18 +618,18 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
             if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
             lds_set[0] = true;
         }
-        hipLaunchKernelGGL(attn_stage_kernel<false>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL(attn_stage_kernel<false>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, geo);
     }
     INFLLM_CHECK_LAUNCH("attn_stage");
     return 0;
 }
 
-extern "C" int infllm_attn_merge(const float *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
+extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
                                  int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
                                  void *stream) {
     INFLLM_REQUIRE(d_o_part && d_lse_part, "attn_merge: null pointer");
     INFLLM_REQUIRE(P >= 1 && B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes P=%d B=%d H=%d Lq=%d", P, B, H, Lq);
-    INFLLM_REQUIRE((o_sl % 4 | o_sh % 4 | o_sb % 4) == 0, "attn_merge: output strides must be multiples of 4");
+    INFLLM_REQUIRE((o_sl % 8 | o_sh % 8 | o_sb % 8) == 0, "attn_merge: output strides must be multiples of 8");
     if (!d_out) {                                     // log-sum-exp only
         INFLLM_REQUIRE(d_lse, "attn_merge: neither output nor lse requested");
         const int64_t rows = (int64_t)B * H * Lq;
@@ -602,9 +638,9 @@ extern "C" int infllm_attn_merge(const float *d_o_part, const float *d_lse_part,
         INFLLM_CHECK_LAUNCH("attn_merge (lse)");
         return 0;
     }
-    const int64_t threads = (int64_t)B * H * Lq * 32;
+    const int64_t threads = (int64_t)B * H * Lq * 16;
     hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
+                       (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
     INFLLM_CHECK_LAUNCH("attn_merge");
     return 0;
 }

@@ -108,6 +108,7 @@ def attn_stage_linear(q, k, v, o_part, lse_part, *, cap=None, j_lo=0, j_hi=None,
         cap = NO_WRAP
     if j_hi is None:
         j_hi = k.shape[2]
+    _need(o_part.dtype == torch.float16 and lse_part.dtype == torch.float32, "partials are fp16 rows with fp32 log-sum-exps")
     a = AttnArgs()
     a.d_q, a.q_sb, a.q_sh, a.q_sl = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
     a.B, a.H, a.Hkv, a.Lq = B, H, Hkv, Lq
@@ -125,6 +126,7 @@ def attn_stage_linear(q, k, v, o_part, lse_part, *, cap=None, j_lo=0, j_hi=None,
 def attn_stage_paged(q, pages_dev, n_pages, Hkv, o_part, lse_part, *, nsplit=1, softmax_scale=None):
     """One stage over a device page table [B, n_pages] of infllm_page entries."""
     B, H, Lq, D = q.shape
+    _need(o_part.dtype == torch.float16 and lse_part.dtype == torch.float32, "partials are fp16 rows with fp32 log-sum-exps")
     a = AttnArgs()
     a.d_q, a.q_sb, a.q_sh, a.q_sl = q.data_ptr(), q.stride(0), q.stride(1), q.stride(2)
     a.B, a.H, a.Hkv, a.Lq = B, H, Hkv, Lq
@@ -139,6 +141,7 @@ def attn_merge(o_part, lse_part, P, out, lse):
     """Join P partials: out bf16 [B,H,Lq,D] (any strides with contiguous rows), lse fp32 [B,H,Lq]."""
     B, H, Lq, D = out.shape
     _need(out.stride(-1) == 1 and out.dtype == torch.bfloat16, "bad merge output")
+    _need(o_part.dtype == torch.float16, "partials are fp16 rows")
     check(_lib.load().infllm_attn_merge(o_part.data_ptr(), lse_part.data_ptr(), P, B, H, Lq,
                                         out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
                                         lse.data_ptr() if lse is not None else None, _stream()), "infllm_attn_merge")

@@ -161,7 +161,7 @@ def test_single_stage_matches_oracle(H, Hkv, Lq, Lk, kw, nsplit):
         offset, window = (Lk - Lq, sw) if isinstance(sw, int) else sw
         mask = ops.MASK_COMPLEMENT if kw.get("complement_sliding_window") else ops.MASK_WINDOW
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
-    o_part = torch.empty((nsplit, B, H, Lq, D), dtype=torch.float32, device="cuda")
+    o_part = torch.empty((nsplit, B, H, Lq, D), dtype=torch.float16, device="cuda")
     lse_part = torch.empty((nsplit, B, H, Lq), dtype=torch.float32, device="cuda")
     ops.attn_stage_linear(qd, kd, vd, o_part, lse_part, j_lo=0, j_hi=Lk, mask=mask, offset=offset, window=window, nsplit=nsplit)
     out = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda")
@@ -199,7 +199,7 @@ def test_two_stage_joint_softmax_with_ring_and_pages():
     ring_k[:, :, rows] = k_win.cuda()
     ring_v[:, :, rows] = v_win.cuda()
     qd = q.cuda()
-    o_part = torch.empty((2, B, H, Lq, D), dtype=torch.float32, device="cuda")
+    o_part = torch.empty((2, B, H, Lq, D), dtype=torch.float16, device="cuda")
     lse_part = torch.empty((2, B, H, Lq), dtype=torch.float32, device="cuda")
     ops.attn_stage_linear(qd, ring_k, ring_v, o_part[0:1], lse_part[0:1], cap=cap, j_lo=lo, j_hi=b1,
                           mask=ops.MASK_WINDOW, offset=b0, window=n_local)
@@ -389,7 +389,7 @@ def test_bad_arguments_raise():
     from infllm_amd._lib import InfLLMHipError
     q = torch.zeros((1, 4, 8, D), dtype=torch.bfloat16, device="cuda")
     k = torch.zeros((1, 3, 8, D), dtype=torch.bfloat16, device="cuda")
-    o = torch.zeros((1, 1, 4, 8, D), dtype=torch.float32, device="cuda")
+    o = torch.zeros((1, 1, 4, 8, D), dtype=torch.float16, device="cuda")
     l = torch.zeros((1, 1, 4, 8), dtype=torch.float32, device="cuda")
     with pytest.raises(InfLLMHipError):
         ops.attn_stage_linear(q, k, k, o, l)                      # 4 heads over 3 kv heads
@@ -397,3 +397,5 @@ def test_bad_arguments_raise():
         ops.attn_stage_linear(q, k[:, :1], k[:, :1], o, l, cap=100)   # cap not a multiple of the tile
     with pytest.raises(ValueError):
         ops._bf16_4d(q.float(), "q")
+    with pytest.raises(ValueError):
+        ops.attn_stage_linear(q, k[:, :1], k[:, :1], o.float(), l)   # partials must be fp16
