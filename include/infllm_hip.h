@@ -355,10 +355,12 @@ int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void
 int infllm_layer_flush(void *layer, void *copy_stream);
 
 /* Event timing of the two attention stages (for benchmarks): enable with a record
- * capacity, read back (which: 0 local stage, 1 global stage) after a device sync.
+ * capacity and a stride (every stride-th launch of each stage is bracketed by two events; an event pair
+ * costs the stream several microseconds, so a throughput run samples), read back (which: 0 local stage,
+ * 1 global stage) after a device sync.
  * ms[i] is the launch-to-finish time of one stage launch, n_queries[i] its block size,
  * n_keys[i] the key rows its source held. */
-int infllm_layer_timing(void *layer, int32_t capacity);
+int infllm_layer_timing(void *layer, int32_t capacity, int32_t stride);
 int infllm_layer_read_timing(void *layer, int32_t which, float *ms, int32_t *n_queries, int32_t *n_keys,
                              int32_t capacity);
 

@@ -137,7 +137,7 @@ SYMBOLS = {
     "infllm_block_fetch": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "infllm_block_back": (c_i32, [c_vp, C.POINTER(BackArgs), c_vp, c_vp]),
     "infllm_layer_flush": (c_i32, [c_vp, c_vp]),
-    "infllm_layer_timing": (c_i32, [c_vp, c_i32]),
+    "infllm_layer_timing": (c_i32, [c_vp, c_i32, c_i32]),
     "infllm_layer_read_timing": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32]),
 }
 

@@ -127,7 +127,7 @@ class ContextManager:
         self.trace_blocks, self.trace_units = [], []
         self.stats = dict(blocks=0, hits=0, misses=0, evictions=0)
         self._layer = None
-        self._timing_cap = 0
+        self._timing_cap, self._timing_stride = 0, 1
         self._mass_units = None                # lru-s: selections of the block whose unit masses are still on the device
         global _SIDE_STREAM
         if async_global_stream and _SIDE_STREAM is None and torch.cuda.is_available():
@@ -234,7 +234,7 @@ class ContextManager:
         if not self._layer:
             raise _lib.InfLLMHipError("infllm_layer_create failed: " + (self._lib.infllm_last_error() or b"").decode())
         if self._timing_cap:
-            check(self._lib.infllm_layer_timing(self._layer, self._timing_cap), "infllm_layer_timing")
+            check(self._lib.infllm_layer_timing(self._layer, self._timing_cap, self._timing_stride), "infllm_layer_timing")
         # argument blocks and host arrays reused by every block
         self._fa, self._ba = FrontArgs(), BackArgs()
         self._sel_slots = (ctypes.c_int32 * (B * max(topk, 1)))()
@@ -283,11 +283,11 @@ class ContextManager:
         return self.host_chunks[chunk][idx]
 
     # ----------------------------------------------------------------- timing
-    def enable_timing(self, capacity):
-        """Event-time every local / global stage launch (up to `capacity` of each) for benchmarks."""
-        self._timing_cap = capacity
+    def enable_timing(self, capacity, stride=1):
+        """Event-time every `stride`-th local / global stage launch (up to `capacity` of each) for benchmarks."""
+        self._timing_cap, self._timing_stride = capacity, stride
         if self._layer:
-            check(self._lib.infllm_layer_timing(self._layer, capacity), "infllm_layer_timing")
+            check(self._lib.infllm_layer_timing(self._layer, capacity, stride), "infllm_layer_timing")
 
     def read_timing(self, which):
         """[(ms, n_queries, n_keys)] of the timed launches; which = 0 local stage, 1 global stage."""

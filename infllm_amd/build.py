@@ -29,7 +29,9 @@ def hipcc_path():
 
 
 def build(verbose=True, extra_flags=()):
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH]
+    # ROCr (libhsa-runtime64) is linked for the DMA-engine copy of carved units; in a process it is the copy the HIP
+    # runtime already loaded
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH, "-lhsa-runtime64"]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -4,7 +4,11 @@
 // critical path.  Decisions (which units are cached, what gets carved) stay with the caller.
 #include <atomic>
 #include <chrono>
+#include <cstdlib>
 #include <vector>
+
+#include <hsa/hsa.h>
+#include <hsa/hsa_ext_amd.h>
 
 #include "common.h"
 
@@ -14,6 +18,7 @@ struct StageTimer {
     std::vector<hipEvent_t> ev;       // pairs
     std::vector<int> n_queries, n_keys;
     int used = 0;
+    int seen = 0;                     // launches since timing was enabled
 };
 
 struct Layer {
@@ -35,6 +40,13 @@ struct Layer {
         int slot = 0, first_unit = 0, count = 0;
         std::vector<void *> dst;
     } off;
+    // The same copy through the DMA engine (see issue_offload_dma): agents of this layer's GPU and of the host,
+    // one completion signal per carve staging slot, and which units a slot's copy in flight carries
+    bool dma_ok = false;
+    hsa_agent_t dma_gpu{}, dma_cpu{};
+    std::vector<hsa_signal_t> dma_sig;
+    std::vector<char> dma_busy;
+    std::vector<int> dma_first, dma_count;
     int page_cur = 0, carve_cur = 0;
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
@@ -46,7 +58,7 @@ struct Layer {
     bool prepared = false;                // the next block's prologue already ran
     int64_t prepared_b0 = 0;
     int prepared_n = 0;
-    int timing_cap = 0;
+    int timing_cap = 0, timing_stride = 1;
     StageTimer timer[2];
 };
 
@@ -143,7 +155,120 @@ __global__ __launch_bounds__(64) void build_pages_kernel(PageJob j, infllm_page 
     out[(int64_t)u * j.n_pages + p] = pg;
 }
 
-// copy the pending units from their staging slot to pinned host memory on `cs`
+// ---- the DMA engine for the device-to-host copy of carved units
+// hipMemcpyAsync may run a 2 MiB device-to-host copy as a shader kernel.  Its writes leave through the L2, and
+// every kernel that ends while they drain over PCIe waits for them in its end-of-kernel cache write-back: the kernels
+// of the block chain stretched by the length of the copy.  The ROCr copy below goes through the SDMA engine, which
+// reads HBM and writes host memory without the shader caches.  It is ordered by the host instead of by a stream:
+// it is issued only once the gather kernels that fill the staging slot have finished (event query), and its
+// completion signal is checked before the slot is written again or a fetch reads the units from the host.
+hsa_status_t collect_agent(hsa_agent_t a, void *data) {
+    ((std::vector<hsa_agent_t> *)data)->push_back(a);
+    return HSA_STATUS_SUCCESS;
+}
+
+// Agents for the current HIP device: matched by PCI address; false when ROCr cannot be used (the stream-ordered
+// hipMemcpyAsync path is then the only one).  INFLLM_NO_DMA_ENGINE=1 in the environment turns the engine path off.
+bool dma_find_agents(hsa_agent_t *gpu, hsa_agent_t *cpu) {
+    const char *off = getenv("INFLLM_NO_DMA_ENGINE");
+    if (off && off[0] && off[0] != '0') return false;
+    if (hsa_init() != HSA_STATUS_SUCCESS) return false;            // reference counted: the HIP runtime holds it already
+    std::vector<hsa_agent_t> all;
+    if (hsa_iterate_agents(collect_agent, &all) != HSA_STATUS_SUCCESS) return false;
+    int dev = 0, bus = -1, devid = -1, domain = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    (void)hipDeviceGetAttribute(&bus, hipDeviceAttributePciBusId, dev);
+    (void)hipDeviceGetAttribute(&devid, hipDeviceAttributePciDeviceId, dev);
+    (void)hipDeviceGetAttribute(&domain, hipDeviceAttributePciDomainID, dev);
+    bool have_cpu = false, have_gpu = false;
+    int n_gpu = 0;
+    hsa_agent_t only_gpu{};
+    for (hsa_agent_t a : all) {
+        hsa_device_type_t type;
+        if (hsa_agent_get_info(a, HSA_AGENT_INFO_DEVICE, &type) != HSA_STATUS_SUCCESS) continue;
+        if (type == HSA_DEVICE_TYPE_CPU && !have_cpu) {
+            *cpu = a;
+            have_cpu = true;
+        } else if (type == HSA_DEVICE_TYPE_GPU) {
+            ++n_gpu;
+            only_gpu = a;
+            uint32_t bdf = 0, dom = 0;
+            if (hsa_agent_get_info(a, (hsa_agent_info_t)HSA_AMD_AGENT_INFO_BDFID, &bdf) != HSA_STATUS_SUCCESS) continue;
+            if (hsa_agent_get_info(a, (hsa_agent_info_t)HSA_AMD_AGENT_INFO_DOMAIN, &dom) != HSA_STATUS_SUCCESS) continue;
+            if (!have_gpu && (int)((bdf >> 8) & 0xff) == bus && (int)((bdf >> 3) & 0x1f) == devid && (int)dom == domain) {
+                *gpu = a;
+                have_gpu = true;
+            }
+        }
+    }
+    if (!have_gpu && n_gpu == 1) {
+        *gpu = only_gpu;
+        have_gpu = true;
+    }
+    return have_cpu && have_gpu;
+}
+
+// wait (bounded) until the engine copy out of staging slot `slot` has completed
+int dma_wait_slot(Layer *L, int slot, const char *what) {
+    if (!L->dma_busy[slot]) return 0;
+    const auto t0 = std::chrono::steady_clock::now();
+    while (hsa_signal_load_scacquire(L->dma_sig[slot]) > 0) {
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(10))
+            return infllm_fail(-2, "%s: the DMA engine copy of carved units did not complete within 10 s", what);
+    }
+    L->dma_busy[slot] = 0;
+    return 0;
+}
+
+// Try to hand the pending units to the DMA engine.  Returns 1 when issued, 0 when not possible right now (the gather
+// kernels have not finished, or there is no engine path), < 0 on error.
+int issue_offload_dma(Layer *L) {
+    if (!L->dma_ok || !L->off.pending) return 0;
+    const hipError_t q = hipEventQuery(L->carve_ready);
+    if (q == hipErrorNotReady) {
+        (void)hipGetLastError();               // "not ready" is an answer, not a failure of a later launch
+        return 0;
+    }
+    if (q != hipSuccess) return infllm_fail(-2, "offload: %s", hipGetErrorString(q));
+    const infllm_layer_desc &d = L->d;
+    const int slot = L->off.slot, n = L->off.count;
+    int rc = dma_wait_slot(L, slot, "offload");                                  // an older copy out of the same slot
+    if (rc) return rc;
+    const int64_t unit_all = (int64_t)d.B * 2 * d.Hkv * d.block_size * kD;
+    const bf16_t *stage = (const bf16_t *)d.d_carve_stage + (int64_t)slot * d.max_carve * unit_all;
+    int runs = 0;
+    for (int i = 0; i < n;) {
+        int j = i + 1;
+        while (j < n && (char *)L->off.dst[j] == (char *)L->off.dst[j - 1] + unit_all * sizeof(bf16_t)) ++j;
+        ++runs;
+        i = j;
+    }
+    hsa_signal_store_relaxed(L->dma_sig[slot], runs);                            // every finished copy takes one off
+    int issued = 0;
+    for (int i = 0; i < n;) {                    // one copy per run of units that are contiguous on the host
+        int j = i + 1;
+        while (j < n && (char *)L->off.dst[j] == (char *)L->off.dst[j - 1] + unit_all * sizeof(bf16_t)) ++j;
+        const hsa_status_t hs = hsa_amd_memory_async_copy(L->off.dst[i], L->dma_cpu, stage + (int64_t)i * unit_all, L->dma_gpu,
+                                                          (size_t)(j - i) * unit_all * sizeof(bf16_t), 0, nullptr, L->dma_sig[slot]);
+        if (hs != HSA_STATUS_SUCCESS) {
+            // give the engine path up for this layer: let what was issued finish, the stream path copies the units again
+            hsa_signal_subtract_relaxed(L->dma_sig[slot], runs - issued);
+            L->dma_busy[slot] = issued > 0;
+            rc = dma_wait_slot(L, slot, "offload");
+            L->dma_ok = false;
+            return rc;
+        }
+        ++issued;
+        i = j;
+    }
+    L->dma_busy[slot] = 1;
+    L->dma_first[slot] = L->off.first_unit;
+    L->dma_count[slot] = n;
+    L->off.pending = false;
+    return 1;
+}
+
+// copy the pending units from their staging slot to pinned host memory on `cs` (stream ordered)
 int issue_offload(Layer *L, hipStream_t cs) {
     const infllm_layer_desc &d = L->d;
     const int64_t unit_all = (int64_t)d.B * 2 * d.Hkv * d.block_size * kD;        // one unit, all batch rows
@@ -182,6 +307,15 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
                 if (orc) return orc;
             }
         }
+        for (size_t s = 0; s < L->dma_busy.size(); ++s) {           // units still on their way to the host by the engine
+            if (!L->dma_busy[s]) continue;
+            bool hit = false;
+            for (int i = 0; i < n_miss && !hit; ++i) hit = units[i] >= L->dma_first[s] && units[i] < L->dma_first[s] + L->dma_count[s];
+            if (hit) {
+                int wrc = dma_wait_slot(L, (int)s, "fetch");
+                if (wrc) return wrc;
+            }
+        }
         L->fetch_dst.resize(n_miss);
         for (int i = 0; i < n_miss; ++i) {
             INFLLM_REQUIRE(rows[i] >= 0 && rows[i] < d.B && slots[i] >= 0 && slots[i] < d.max_cached && srcs[i], "fetch: bad miss entry");
@@ -194,13 +328,20 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
             L->fetch_wait = true;
         }
     }
-    if (L->off.pending) return issue_offload(L, cs);
+    if (L->off.pending) {
+        if (L->dma_ok) {                          // the engine takes it as soon as the gathers have finished (see block_back)
+            const int drc = issue_offload_dma(L);
+            return drc < 0 ? drc : 0;
+        }
+        return issue_offload(L, cs);
+    }
     return 0;
 }
 
 int timer_begin(Layer *L, int which, int n_queries, int n_keys, hipStream_t st) {
     StageTimer &t = L->timer[which];
     if (L->timing_cap <= 0 || t.used >= L->timing_cap) return -1;
+    if (t.seen++ % L->timing_stride) return -1;
     const int i = t.used++;
     t.n_queries[i] = n_queries;
     t.n_keys[i] = n_keys;
@@ -249,6 +390,17 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         infllm_layer_destroy(L);
         return bad("hipEventCreate failed");
     }
+    L->dma_busy.assign(d.carve_slots, 0);
+    L->dma_first.assign(d.carve_slots, 0);
+    L->dma_count.assign(d.carve_slots, 0);
+    if (dma_find_agents(&L->dma_gpu, &L->dma_cpu)) {
+        L->dma_ok = true;
+        for (int i = 0; i < d.carve_slots && L->dma_ok; ++i) {
+            hsa_signal_t sig;
+            if (hsa_signal_create(0, 0, nullptr, &sig) == HSA_STATUS_SUCCESS) L->dma_sig.push_back(sig);
+            else L->dma_ok = false;                 // without signals the stream-ordered copy is used
+        }
+    }
     return L;
 }
 
@@ -261,6 +413,10 @@ extern "C" int infllm_layer_destroy(void *layer) {
         if (e) (void)hipEventDestroy(e);
     for (hipEvent_t e : L->carve_evt)
         if (e) (void)hipEventDestroy(e);
+    for (size_t i = 0; i < L->dma_sig.size(); ++i) {
+        if (i < L->dma_busy.size()) (void)dma_wait_slot(L, (int)i, "layer_destroy");
+        (void)hsa_signal_destroy(L->dma_sig[i]);
+    }
     for (auto &t : L->timer)
         for (hipEvent_t e : t.ev)
             if (e) (void)hipEventDestroy(e);
@@ -268,8 +424,8 @@ extern "C" int infllm_layer_destroy(void *layer) {
     return 0;
 }
 
-extern "C" int infllm_layer_timing(void *layer, int32_t capacity) {
-    INFLLM_REQUIRE(layer && capacity >= 0, "layer_timing: bad arguments");
+extern "C" int infllm_layer_timing(void *layer, int32_t capacity, int32_t stride) {
+    INFLLM_REQUIRE(layer && capacity >= 0 && stride >= 1, "layer_timing: bad arguments");
     Layer *L = (Layer *)layer;
     for (auto &t : L->timer) {
         while ((int)t.ev.size() < 2 * capacity) {
@@ -280,8 +436,10 @@ extern "C" int infllm_layer_timing(void *layer, int32_t capacity) {
         t.n_queries.resize(capacity);
         t.n_keys.resize(capacity);
         t.used = 0;
+        t.seen = 0;
     }
     L->timing_cap = capacity;
+    L->timing_stride = stride;
     return 0;
 }
 
@@ -508,12 +666,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         if (frc) return frc;
     }
     L->fetch_issued = false;
-    if (L->fetch_wait) {
-        HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
-        L->fetch_wait = false;
-    }
 
-    // ---- 2. page table of the global stage: units | init | overflow remainder
+    // ---- 2. page table of the global stage: units | init | overflow remainder (slot numbers only: it does not
+    //         wait for the fetch, so it is out of the way when the units arrive)
     const int64_t overflow_end = b1 - d.n_local > a->cursor ? b1 - d.n_local : a->cursor;
     int n_pages = 0;
     if (d.B * a->n_sel <= kPageJobSlots) {
@@ -592,6 +747,10 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     }
 
     // ---- 3. global stage and merge
+    if (L->fetch_wait) {
+        HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
+        L->fetch_wait = false;
+    }
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
     const int sl = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
     int parts = sl;
@@ -690,9 +849,25 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, stream);
     if (rc) return rc;
     if (a->n_carve > 0) {
+        if (L->off.pending) {
+            // the units of an earlier block are still waiting: their gathers were queued a whole block ago, so the
+            // host gets through this wait at once and the engine can take them; else the copy stream does
+            int drc = 0;
+            if (L->dma_ok) {
+                HIP_OK(hipEventSynchronize(L->carve_ready), "block_back: carve event");
+                drc = issue_offload_dma(L);
+                if (drc < 0) return drc;
+            }
+            if (drc == 0) {
+                rc = issue_offload(L, cs);
+                if (rc) return rc;
+            }
+        }
         const int slot = L->carve_cur;
         L->carve_cur = (slot + 1) % d.carve_slots;
         if (L->carve_busy[slot]) HIP_OK(hipEventSynchronize(L->carve_evt[slot]), "block_back: carve slot");
+        rc = dma_wait_slot(L, slot, "block_back");
+        if (rc) return rc;
         const int64_t unit_all = (int64_t)d.B * slot_elems;                       // one unit, all batch rows
         bf16_t *stage = (bf16_t *)d.d_carve_stage + (int64_t)slot * d.max_carve * unit_all;
         rc = infllm_gather_rows(d.d_ring_k_raw, d.ring_cap, d.B, d.Hkv, cursor, a->n_carve * bs, bs, stage, slot_elems, unit_all,
@@ -716,6 +891,17 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
 extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
     INFLLM_REQUIRE(layer, "layer_flush: null layer");
     Layer *L = (Layer *)layer;
-    if (L->off.pending) return issue_offload(L, (hipStream_t)copy_stream);
+    if (L->off.pending) {
+        int drc = issue_offload_dma(L);
+        if (drc < 0) return drc;
+        if (drc == 0) {
+            drc = issue_offload(L, (hipStream_t)copy_stream);
+            if (drc) return drc;
+        }
+    }
+    for (size_t s = 0; s < L->dma_busy.size(); ++s) {       // engine copies are not ordered by any stream: finish them here
+        const int wrc = dma_wait_slot(L, (int)s, "layer_flush");
+        if (wrc) return wrc;
+    }
     return 0;
 }
