@@ -128,13 +128,22 @@ __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
 }
 
 // out[b, c] = scale * sum_p parts[b, p, c], p ascending
-__global__ __launch_bounds__(256) void reduce_partials_kernel(const float *parts, int n_parts, int C, float scale,
-                                                              float *out) {
-    const int c = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+__global__ __launch_bounds__(64) void reduce_partials_kernel(const float *parts, int n_parts, int C, float scale,
+                                                             float *out) {
+    const int c = blockIdx.x * 64 + threadIdx.x, b = blockIdx.y;
     if (c >= C) return;
     const float *src = parts + (int64_t)b * n_parts * C + c;
     float s = 0.f;
-    for (int p = 0; p < n_parts; ++p) s += src[(int64_t)p * C];
+    // the order of the sum stays p ascending; the loads of 16 partials are in flight together, because a chain of
+    // dependent loads is all latency (and that latency multiplies while a unit fetch keeps the memory fabric busy)
+    for (int p0 = 0; p0 < n_parts; p0 += 16) {
+        float v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = p0 + i < n_parts ? src[(int64_t)(p0 + i) * C] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if (p0 + i < n_parts) s += v[i];
+    }
     out[(int64_t)b * C + c] = s * scale;
 }
 
@@ -270,7 +279,7 @@ extern "C" int infllm_reduce_partials(const float *d_parts, int32_t B, int32_t n
                                       void *stream) {
     INFLLM_REQUIRE(d_parts && d_out, "reduce_partials: null pointer");
     INFLLM_REQUIRE(B > 0 && n_parts > 0 && C > 0, "reduce_partials: bad sizes B=%d n_parts=%d C=%d", B, n_parts, C);
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3((C + 255) / 256, B), dim3(256), 0, (hipStream_t)stream, d_parts, n_parts, C,
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((C + 63) / 64, B), dim3(64), 0, (hipStream_t)stream, d_parts, n_parts, C,
                        scale, d_out);
     INFLLM_CHECK_LAUNCH("reduce_partials");
     return 0;
