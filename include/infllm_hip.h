@@ -354,6 +354,43 @@ int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_miss_row, c
 int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream);
 int infllm_layer_flush(void *layer, void *copy_stream);
 
+/* ---- residency policy of the device unit cache, one object per batch row (context_manager.py:246-265 for the
+ * values, 495-515 for the eviction): lru = clock of the last use, fifo = clock of the first load, lru-s = decayed
+ * attention mass; eviction takes the smallest values first (first inserted first on ties) and never a unit of the
+ * current selection.  Host code (no device work): it sits between the arrival of the top-k ids and the fetch. */
+enum { INFLLM_CACHE_LRU = 0, INFLLM_CACHE_FIFO = 1, INFLLM_CACHE_LRU_S = 2 };
+void *infllm_cache_create(int32_t capacity, int32_t strategy, double score_decay);
+int infllm_cache_destroy(void *cache);
+/* One block: selected[n_sel] unit ids -> slots[n_sel] (their slab slots); the misses in selection order with the
+ * slots they get; the evicted ids in eviction order (evicted / n_evicted may be NULL).  Returns the number of misses. */
+int infllm_cache_touch(void *cache, const int32_t *selected, int32_t n_sel, int32_t *slots, int32_t *miss_units,
+                       int32_t *miss_slots, int32_t *evicted, int32_t *n_evicted);
+/* lru-s (context_manager.py:529-543): every resident's value decays, then the given units gain their scores */
+int infllm_cache_add_scores(void *cache, const int32_t *units, const double *scores, int32_t n);
+/* residents in insertion order (any output may be NULL); returns their number */
+int infllm_cache_residents(void *cache, int32_t *units, double *values, int32_t *slots, int32_t capacity);
+
+/* Selection -> policy -> fetch in one native call (replaces a host loop between infllm_layer_wait_topk and
+ * infllm_block_fetch): runs infllm_cache_touch for every batch row, fills the lists infllm_block_back takes and
+ * issues the fetch.  Returns the number of misses (>= 0) or an error (< 0). */
+typedef struct {
+    void *const *caches;                              /* [B] */
+    const int32_t *h_selected;                        /* host [B,n_sel] unit ids (e.g. the pinned top-k ids) */
+    int32_t n_sel;
+    int32_t wait_topk;                                /* != 0: infllm_layer_wait_topk first, then read h_selected */
+    /* host arena of the units: unit u of batch row b is at h_chunk_base[u / units_per_chunk]
+     * + (u % units_per_chunk) * unit_bytes + b * row_bytes (device-visible addresses of pinned memory) */
+    const uint64_t *h_chunk_base;
+    int32_t n_chunks, units_per_chunk;
+    int64_t unit_bytes, row_bytes;
+    int32_t *h_sel_slots;                             /* out [B,n_sel] */
+    int32_t *h_miss_row, *h_miss_slot, *h_miss_unit;  /* out [<= B*n_sel] */
+    const void **h_miss_src;                          /* out [<= B*n_sel] */
+    int32_t *h_evicted;                               /* out, optional: [B,n_sel], row b holds h_n_evicted[b] ids */
+    int32_t *h_n_evicted, *h_n_miss;                  /* out, optional: [B] */
+} infllm_select_args;
+int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, void *copy_stream);
+
 /* Event timing of the two attention stages (for benchmarks): enable with a record
  * capacity and a stride (every stride-th launch of each stage is bracketed by two events; an event pair
  * costs the stream several microseconds, so a throughput run samples), read back (which: 0 local stage,

@@ -106,7 +106,18 @@ class BackArgs(C.Structure):
     ]
 
 
+class SelectArgs(C.Structure):
+    _fields_ = [
+        ("caches", c_vp), ("h_selected", c_vp), ("n_sel", c_i32), ("wait_topk", c_i32),
+        ("h_chunk_base", c_vp), ("n_chunks", c_i32), ("units_per_chunk", c_i32),
+        ("unit_bytes", c_i64), ("row_bytes", c_i64),
+        ("h_sel_slots", c_vp), ("h_miss_row", c_vp), ("h_miss_slot", c_vp), ("h_miss_unit", c_vp), ("h_miss_src", c_vp),
+        ("h_evicted", c_vp), ("h_n_evicted", c_vp), ("h_n_miss", c_vp),
+    ]
+
+
 NO_RETRIEVAL = 1            # INFLLM_NO_RETRIEVAL
+CACHE_STRATEGY = {"lru": 0, "fifo": 1, "lru-s": 2}      # INFLLM_CACHE_*
 
 # name -> (restype, argtypes); every symbol include/infllm_hip.h declares
 SYMBOLS = {
@@ -137,6 +148,12 @@ SYMBOLS = {
     "infllm_block_fetch": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "infllm_block_back": (c_i32, [c_vp, C.POINTER(BackArgs), c_vp, c_vp]),
     "infllm_layer_flush": (c_i32, [c_vp, c_vp]),
+    "infllm_cache_create": (c_vp, [c_i32, c_i32, c_f64]),
+    "infllm_cache_destroy": (c_i32, [c_vp]),
+    "infllm_cache_touch": (c_i32, [c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp]),
+    "infllm_cache_add_scores": (c_i32, [c_vp, c_vp, c_vp, c_i32]),
+    "infllm_cache_residents": (c_i32, [c_vp, c_vp, c_vp, c_vp, c_i32]),
+    "infllm_block_select": (c_i32, [c_vp, C.POINTER(SelectArgs), c_vp, c_vp]),
     "infllm_layer_timing": (c_i32, [c_vp, c_i32, c_i32]),
     "infllm_layer_read_timing": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32]),
 }

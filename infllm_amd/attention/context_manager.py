@@ -43,59 +43,71 @@ _CARVE_SLOTS = 4
 
 
 class CachePolicy:
-    """Residency policy of one batch row (context_manager.py:246-265, 495-515).
+    """Residency policy of one batch row (context_manager.py:246-265, 495-515): a handle on the native
+    object (infllm_cache_*), which ContextManager also drives directly from infllm_block_select.
 
-    ``cached`` is an insertion-ordered dict unit -> value; eviction walks it in
+    ``cached`` is the reference's insertion-ordered dict unit -> value; eviction walks it in
     ascending value (stable), skipping the units selected for this block.
     """
 
     def __init__(self, capacity, strategy, score_decay):
         self.capacity, self.strategy, self.score_decay = capacity, strategy, score_decay
-        self.cached = {}
-        self.clock = 0
-        self.slot_of = {}
-        self.free = list(range(capacity - 1, -1, -1))
+        self._lib = _lib.load()
+        self.handle = self._lib.infllm_cache_create(capacity, _lib.CACHE_STRATEGY[strategy],
+                                                    float(score_decay) if score_decay is not None else 0.0)
+        if not self.handle:
+            raise _lib.InfLLMHipError((self._lib.infllm_last_error() or b"").decode())
         self.evicted_log = None             # set to a list to record the evictions of every block
+        self._units = (ctypes.c_int32 * capacity)()
+        self._slots = (ctypes.c_int32 * capacity)()
+        self._values = (ctypes.c_double * capacity)()
+
+    def __del__(self):
+        if getattr(self, "handle", None):
+            self._lib.infllm_cache_destroy(self.handle)
+            self.handle = None
 
     def touch(self, selected):
         """Returns (misses, evicted) and updates values; slots of evicted units are freed."""
-        cached = self.cached
-        misses = [b for b in selected if b not in cached]
-        surplus = len(cached) - self.capacity + len(misses)
-        evicted = []
-        if surplus > 0:
-            chosen = set(selected)
-            for unit, _ in sorted(cached.items(), key=lambda kv: kv[1]):
-                if unit not in chosen:
-                    evicted.append(unit)
-                if len(evicted) >= surplus:
-                    break
-            for unit in evicted:
-                del cached[unit]
-                self.free.append(self.slot_of.pop(unit))
-        if self.strategy == "lru":
-            self.clock += 1
-            for b in selected:
-                cached[b] = self.clock
-        elif self.strategy == "fifo":
-            self.clock += 1
-            for b in selected:
-                cached.setdefault(b, self.clock)
-        else:                                   # lru-s
-            for b in selected:
-                cached[b] = 0
-        assert len(cached) <= self.capacity, "topk exceeds max_cached_block"
-        for b in misses:
-            self.slot_of[b] = self.free.pop()
+        n = len(selected)
+        assert n <= self.capacity, "topk exceeds max_cached_block"
+        sel = (ctypes.c_int32 * max(n, 1))(*selected)
+        slots, mu, ms = ((ctypes.c_int32 * max(n, 1))() for _ in range(3))
+        ev, n_ev = (ctypes.c_int32 * self.capacity)(), ctypes.c_int32(0)
+        n_miss = self._lib.infllm_cache_touch(self.handle, sel, n, slots, mu, ms, ev, ctypes.byref(n_ev))
+        if n_miss < 0:
+            check(n_miss, "infllm_cache_touch")
+        evicted = list(ev[:n_ev.value])
         if self.evicted_log is not None:
             self.evicted_log.append(evicted)
-        return misses, evicted
+        return list(mu[:n_miss]), evicted
 
     def add_scores(self, units, unit_scores):
-        for u in self.cached:
-            self.cached[u] = self.cached[u] * self.score_decay
-        for u, s in zip(units, unit_scores):
-            self.cached[u] += s
+        n = len(units)
+        check(self._lib.infllm_cache_add_scores(self.handle, (ctypes.c_int32 * max(n, 1))(*units),
+                                                (ctypes.c_double * max(n, 1))(*unit_scores[:n]), n), "infllm_cache_add_scores")
+
+    def _residents(self):
+        n = self._lib.infllm_cache_residents(self.handle, self._units, self._values, self._slots, self.capacity)
+        if n < 0:
+            check(n, "infllm_cache_residents")
+        return n
+
+    @property
+    def cached(self):
+        n = self._residents()
+        as_int = self.strategy != "lru-s"
+        return {self._units[i]: (int(self._values[i]) if as_int else self._values[i]) for i in range(n)}
+
+    @property
+    def slot_of(self):
+        n = self._residents()
+        return {self._units[i]: self._slots[i] for i in range(n)}
+
+    @property
+    def free(self):
+        used = set(self.slot_of.values())
+        return [s for s in range(self.capacity) if s not in used]
 
 
 class ContextManager:
@@ -173,6 +185,7 @@ class ContextManager:
         self.reps = torch.zeros((B, 16, H * D), **bf)
         self.unit_scores = torch.empty((B, 16), **f32)
         self.host_chunks, self._host_base, self._host_dev_base = [], [], []
+        self._chunk_base = (ctypes.c_uint64 * 64)()           # device-visible chunk addresses, as the native side reads them
         self.policy = [CachePolicy(self.max_cached_block, self.cache_strategy, self.score_decay) for _ in range(B)]
         if self.record_trace:
             for pol in self.policy:
@@ -256,6 +269,21 @@ class ContextManager:
             if not ba.d_unit_mass:
                 raise _lib.InfLLMHipError("pinned host memory is not device-mapped: " + (self._lib.infllm_last_error() or b"").decode())
             ba.d_mass_scratch = self.mass_scratch.data_ptr()
+        # selection -> cache policy -> fetch runs natively (infllm_block_select) on these arrays
+        n_ids = B * max(topk, 1)
+        self._sel_ids = (ctypes.c_int32 * n_ids)()
+        self._evicted = (ctypes.c_int32 * n_ids)()
+        self._n_evicted, self._n_miss_row = (ctypes.c_int32 * B)(), (ctypes.c_int32 * B)()
+        self._caches = (ctypes.c_void_p * B)(*[pol.handle for pol in self.policy])
+        sa = self._sa = _lib.SelectArgs()
+        sa.caches = ctypes.addressof(self._caches)
+        sa.h_chunk_base, sa.n_chunks, sa.units_per_chunk = ctypes.addressof(self._chunk_base), 0, _HOST_CHUNK_UNITS
+        sa.unit_bytes, sa.row_bytes = self.unit_bytes, self.slot_bytes
+        sa.h_sel_slots = ba.h_sel_slots
+        sa.h_miss_row, sa.h_miss_slot, sa.h_miss_unit, sa.h_miss_src = ba.h_miss_row, ba.h_miss_slot, ba.h_miss_unit, ba.h_miss_src
+        sa.h_evicted, sa.h_n_evicted, sa.h_n_miss = (ctypes.addressof(self._evicted), ctypes.addressof(self._n_evicted),
+                                                      ctypes.addressof(self._n_miss_row))
+        self._sa_ref = ctypes.byref(sa)
         self._fa_ref, self._ba_ref = ctypes.byref(self._fa), ctypes.byref(self._ba)
         self.initialized = True
 
@@ -275,6 +303,13 @@ class ContextManager:
             if not dev:
                 raise _lib.InfLLMHipError((self._lib.infllm_last_error() or b"").decode())
             self._host_dev_base.append(dev)
+            if len(self._host_dev_base) > len(self._chunk_base):
+                grown = (ctypes.c_uint64 * (2 * len(self._chunk_base)))()
+                grown[:len(self._chunk_base)] = self._chunk_base[:]
+                self._chunk_base = grown
+                self._sa.h_chunk_base = ctypes.addressof(grown)
+            self._chunk_base[len(self._host_dev_base) - 1] = dev
+            self._sa.n_chunks = len(self._host_dev_base)
         return self._host_base[chunk] + idx * self.unit_bytes
 
     def host_unit(self, unit):
@@ -318,19 +353,9 @@ class ContextManager:
         rc = lib.infllm_block_front(layer, self._fa_ref, self._main_raw)
         if rc:
             check(rc, "infllm_block_front")
-        # ---- retrieval result (context_manager.py:366-383)
-        if preselected is not None:                          # chosen for the whole chunk (context_manager.py:381-382)
-            selected = preselected
-        elif N <= topk:
-            selected = [list(range(N))] * B
-        else:
-            rc = lib.infllm_layer_wait_topk(layer)           # the one host wait of a block
-            if rc:
-                check(rc, "infllm_layer_wait_topk")
-            selected = self.topk_idx_host.tolist()
-        # ---- cache policy (context_manager.py:495-515)
-        n_sel = len(selected[0])
-        n_miss = 0
+        # ---- retrieval result (context_manager.py:366-383) -> cache policy (495-515) -> fetch, in one native call:
+        #      this stretch is on the chain from one block's selection to the next, the rest of the host's work is not
+        sa = self._sa
         stats = self.stats
         if self._mass_units is not None:                     # lru-s: the previous block's masses decide this eviction
             check(lib.infllm_layer_wait_mass(layer), "infllm_layer_wait_mass")
@@ -338,27 +363,31 @@ class ContextManager:
             for u in range(B):
                 self.policy[u].add_scores(self._mass_units[u], masses[u][:len(self._mass_units[u])])
             self._mass_units = None
+        if preselected is not None or N <= topk:
+            # chosen for the whole chunk (context_manager.py:381-382), or every unit there is
+            selected = preselected if preselected is not None else [list(range(N))] * B
+            n_sel = len(selected[0])
+            for u in range(B):
+                self._sel_ids[u * n_sel:(u + 1) * n_sel] = selected[u]
+            sa.h_selected, sa.n_sel, sa.wait_topk = ctypes.addressof(self._sel_ids), n_sel, 0
+            n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
+        else:
+            n_sel = topk
+            sa.h_selected, sa.n_sel, sa.wait_topk = self.topk_idx_host.data_ptr(), n_sel, 1     # the one host wait of a block
+            n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
+            selected = None                                   # read back below, off the chain
+        if n_miss < 0:
+            check(n_miss, "infllm_block_select")
+        # the transfer has started; everything from here on overlaps it
+        if selected is None:
+            selected = self.topk_idx_host.tolist()
+        n_ev = sum(self._n_evicted[:B])
+        stats["hits"] += B * n_sel - n_miss
+        stats["misses"] += n_miss
+        stats["evictions"] += n_ev
         for u in range(B):
-            pol = self.policy[u]
-            misses, evicted = pol.touch(selected[u])
-            stats["hits"] += n_sel - len(misses)
-            stats["misses"] += len(misses)
-            stats["evictions"] += len(evicted)
-            slot_of = pol.slot_of
-            base = u * n_sel
-            for i, unit in enumerate(selected[u]):
-                self._sel_slots[base + i] = slot_of[unit]
-            for unit in misses:
-                self._miss_row[n_miss] = u
-                self._miss_slot[n_miss] = slot_of[unit]
-                self._miss_unit[n_miss] = unit
-                chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
-                self._miss_src[n_miss] = self._host_dev_base[chunk] + idx * self.unit_bytes + u * self.slot_bytes
-                n_miss += 1
-        rc = lib.infllm_block_fetch(layer, n_miss, self._miss_row, self._miss_slot, self._miss_unit, self._miss_src,
-                                    self._main_raw, self._copy_raw)     # the transfer starts now; the rest overlaps it
-        if rc:
-            check(rc, "infllm_block_fetch")
+            if self.policy[u].evicted_log is not None:
+                self.policy[u].evicted_log.append(list(self._evicted[u * n_sel:u * n_sel + self._n_evicted[u]]))
         if self.cache_strategy == "lru":
             self.load_count += 1
         # ---- state machine after the block (context_manager.py:614-679)

@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libinfllm_hip.so")
-SOURCES = ["abi.hip", "ingest.hip", "attn.hip", "score.hip", "retrieve.hip", "stream.hip"]
+SOURCES = ["abi.hip", "ingest.hip", "attn.hip", "score.hip", "retrieve.hip", "cache.hip", "stream.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -641,6 +641,45 @@ extern "C" int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_
     return rc;
 }
 
+extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, void *copy_stream) {
+    INFLLM_REQUIRE(layer && a, "block_select: null argument");
+    Layer *L = (Layer *)layer;
+    const infllm_layer_desc &d = L->d;
+    INFLLM_REQUIRE(a->caches && a->n_sel >= 0 && a->n_sel <= d.topk, "block_select: bad selection size %d", a->n_sel);
+    INFLLM_REQUIRE(a->n_sel == 0 || (a->h_selected && a->h_sel_slots && a->h_miss_row && a->h_miss_slot && a->h_miss_unit && a->h_miss_src),
+                   "block_select: null list");
+    INFLLM_REQUIRE(a->n_sel == 0 || (a->h_chunk_base && a->units_per_chunk > 0 && a->n_chunks >= 0 && a->unit_bytes > 0 && a->row_bytes > 0),
+                   "block_select: bad host arena description");
+    if (a->wait_topk) {
+        const int wrc = infllm_layer_wait_topk(layer);
+        if (wrc) return wrc;
+    }
+    int n_miss = 0;
+    int32_t units[64], slots[64];
+    INFLLM_REQUIRE(a->n_sel <= 64, "block_select: more than 64 units per row");
+    for (int u = 0; u < d.B; ++u) {
+        INFLLM_REQUIRE(a->caches[u], "block_select: null cache of row %d", u);
+        int32_t n_ev = 0;
+        const int m = infllm_cache_touch(a->caches[u], a->h_selected + (int64_t)u * a->n_sel, a->n_sel, a->h_sel_slots + (int64_t)u * a->n_sel,
+                                         units, slots, a->h_evicted ? a->h_evicted + (int64_t)u * a->n_sel : nullptr, &n_ev);
+        if (m < 0) return m;
+        if (a->h_n_evicted) a->h_n_evicted[u] = n_ev;
+        if (a->h_n_miss) a->h_n_miss[u] = m;
+        for (int i = 0; i < m; ++i, ++n_miss) {
+            const int chunk = units[i] / a->units_per_chunk, idx = units[i] % a->units_per_chunk;
+            INFLLM_REQUIRE(chunk < a->n_chunks && a->h_chunk_base[chunk], "block_select: unit %d has no host copy", units[i]);
+            a->h_miss_row[n_miss] = u;
+            a->h_miss_slot[n_miss] = slots[i];
+            a->h_miss_unit[n_miss] = units[i];
+            a->h_miss_src[n_miss] = (const void *)(uintptr_t)(a->h_chunk_base[chunk] + (uint64_t)idx * a->unit_bytes + (uint64_t)u * a->row_bytes);
+        }
+    }
+    const int rc = do_fetch(L, n_miss, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src, (hipStream_t)stream, (hipStream_t)copy_stream);
+    if (rc) return rc;
+    L->fetch_issued = true;
+    return n_miss;
+}
+
 extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream) {
     INFLLM_REQUIRE(layer && a, "block_back: null argument");
     Layer *L = (Layer *)layer;
