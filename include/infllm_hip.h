@@ -234,31 +234,39 @@ int infllm_fetch_units(const void *const *h_src, void *const *d_dst, int32_t n, 
 void *infllm_host_device_pointer(void *h_pinned);
 
 /* ---------------------------------------------------------------------------
- * One execution block in two calls.
+ * One execution block in three calls.
  * Replaces the device work of ContextManager._append and append_global
  * (context_manager.py:474-545, 614-679) for one block of at most exc_block_size
- * queries; the host keeps the decisions (cache policy, state machine):
+ * queries; the host keeps the state machine (what is carved when), the cache policy is
+ * infllm_cache_* further down:
  *
  *   infllm_block_front   the block's prologue (RoPE + rings) and retrieval (mean query, unit
  *                        scores, top-k, asynchronous copy of the ids to pinned memory) unless
  *                        the previous block already did them ahead; the local stage; then,
  *                        when the caller passes the NEXT block's rows, that block's prologue
  *                        and the scores of the units that already exist;
- *   infllm_layer_wait_topk   blocks until the ids of this block are readable on the host;
- *   infllm_block_back    fetch of missed units (copy stream), page table, global stage, merge,
+ *   infllm_block_select  waits until the ids of this block are readable on the host, runs the cache
+ *                        policy and issues the fetch of the missed units (copy stream); the same in
+ *                        separate steps: infllm_layer_wait_topk, the caller's own policy,
+ *                        infllm_block_fetch;
+ *   infllm_block_back    (the fetch, if nothing issued it yet,) page table, global stage, merge,
  *                        local score of the tokens about to be carved, init peeling,
  *                        representatives of the new units, and - when the next block was
  *                        prepared - the scores of the new units, the next block's top-k and
- *                        the copy of its ids; only then the rest of the local score and the
- *                        copy of the new units to pinned host memory (copy stream).
+ *                        the copy of its ids; only then the block's output rows, the rest of the
+ *                        local score and the gather of the new units into a staging slot.
  *
  * The chain from one block's ids to the next block's ids is therefore: fetch, global stage,
  * merge, a small score launch, representatives, a small score launch, top-k.
  *
- * The copy of newly carved units to pinned host memory is deferred: it is issued on the copy
- * stream right after the NEXT block's fetch (or before it, when that fetch needs one of those
- * units), so a fetch never queues behind it; infllm_layer_flush issues whatever is still
- * pending and must be called when no further block follows (end of an append() call).
+ * The copy of newly carved units from the staging slot to pinned host memory is deferred and
+ * ordered by the host: once the gather's event has fired (checked at the next block's calls) it
+ * goes to the DMA engine (ROCr asynchronous copy), whose completion signal is checked before the
+ * staging slot is reused and before a fetch reads one of those units.  Where that is not
+ * possible (no ROCr agents, INFLLM_NO_DMA_ENGINE=1, or a fetch needs the units at once) it is a
+ * hipMemcpyAsync on the copy stream.  infllm_layer_flush issues whatever is still pending, waits
+ * for the engine copies, and must be called when no further block follows (end of an append()
+ * call); after it and a synchronisation of the copy stream the host copies are complete.
  *
  * A layer handle owns only events, the rotation of the pinned page-table staging slots and of
  * the carve staging slots; every buffer is the caller's.

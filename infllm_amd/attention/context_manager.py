@@ -15,16 +15,17 @@ stream positions and device-resident rings instead of torch.cat/trim:
   softmax; the local score (probability column sums) is a third kernel that
   needs the merged log-sum-exp;
 * memory units live in pinned host memory (always) and in a slab of
-  ``max_cached_block`` device slots managed by the reference's lru policy
-  (plus fifo); misses are fetched with hipMemcpyAsync on a side stream.
+  ``max_cached_block`` device slots managed by the reference's lru / lru-s
+  policy (plus fifo; native, infllm_cache_*); the misses of a block are read
+  from the pinned pages by one kernel on a side stream.
 
-The host keeps the decisions - the cache policy and the state machine, in
-absolute positions (context_manager.py:614-679 restated): ``cursor`` is the
-first token not yet carved, tokens [0, init_len) are the attention sinks, unit
-u is tokens [n_init + u*bs, n_init + (u+1)*bs).  The device work of one
-execution block is issued by two native calls, infllm_block_front and
-infllm_block_back, with one host wait (for the retrieved unit ids) in between,
-which overlaps the local stage.
+This module keeps the state machine, in absolute positions
+(context_manager.py:614-679 restated): ``cursor`` is the first token not yet
+carved, tokens [0, init_len) are the attention sinks, unit u is tokens
+[n_init + u*bs, n_init + (u+1)*bs).  The device work of one execution block is
+issued by three native calls: infllm_block_front, infllm_block_select (the one
+host wait, for the retrieved unit ids, which overlaps the local stage; then
+cache policy and fetch) and infllm_block_back.
 """
 import ctypes
 
