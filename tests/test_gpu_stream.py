@@ -187,6 +187,24 @@ def test_call_splitting_cache_size_and_side_stream_do_not_change_results():
     assert torch.equal(ref, fifo)
 
 
+def test_carved_units_reach_the_host_by_either_copy_path(monkeypatch):
+    """New units go to their pinned home through the DMA engine, or (INFLLM_NO_DMA_ENGINE=1) by a stream-ordered
+    hipMemcpyAsync: same bytes on the host, same outputs (the tight cache makes later blocks fetch them back)."""
+    T = 1280
+    q, k, v = _stream(T, 8, 2, 14)
+    kw = dict(SMALL, max_cached_block=4, async_global_stream=True)
+    runs = [_run_gpu(q, k, v, [640, 500, 140], 1e4, **kw)]
+    monkeypatch.setenv("INFLLM_NO_DMA_ENGINE", "1")
+    runs.append(_run_gpu(q, k, v, [640, 500, 140], 1e4, **kw))
+    assert torch.equal(runs[0][0], runs[1][0]) and runs[0][1].stats == runs[1][1].stats
+    bs, n_init = SMALL["block_size"], SMALL["n_init"]
+    for _, cm in runs:
+        assert cm.num_global_block == (T - n_init - SMALL["n_local"]) // bs
+        for u in range(cm.num_global_block):
+            lo, hu = n_init + u * bs, cm.host_unit(u)
+            assert torch.equal(hu[0, 0], k[0, :, lo:lo + bs]) and torch.equal(hu[0, 1], v[0, :, lo:lo + bs]), u
+
+
 def test_state_export_and_injection_resume_the_stream_exactly():
     from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
     T0, T1 = 900, 333
