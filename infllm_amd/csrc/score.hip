@@ -7,23 +7,25 @@
 // recomputes Q.K^T.  Orientation: S[query, key] with keys in the MFMA column, so a lane
 // owns one key and the column sum is a running per-lane scalar.  A workgroup owns 256
 // consecutive keys of one query head: each of its 4 waves keeps 64 keys in registers
-// (B operand) for the whole kernel, while tiles of 64 queries stream through LDS
+// (B operand) for the whole kernel, while tiles of 64 or 128 queries stream through LDS
 // (A operand, shared by the 4 waves, double buffered).  Exactly one lane writes each
 // (head, key) cell, so results are deterministic.
 #include "common.h"
 
 namespace {
 
-constexpr int kQStage = 64;                // queries per LDS stage
 constexpr int kQPad = kD + 8;              // LDS row of Q (bf16 elements): 272 bytes rotates the banks
 
 // KS = 32-key halves per wave: 2 for long key ranges; 1 halves the work of a wave per query stage, which is what
-// bounds the short launches that sit on the critical path between two blocks.
-template <int KS>
+// bounds the short launches that sit on the critical path between two blocks.  QS = queries per LDS stage: a short
+// launch is a chain of stages that each wait for one global load (there is next to no arithmetic to hide it behind),
+// so it takes stages of 128 queries and half as many of them.
+template <int KS, int QS>
 __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a) {
-    constexpr int kWaveKeys = 32 * KS, kKeysPerWg = 4 * kWaveKeys;
-    __shared__ __attribute__((aligned(16))) bf16_t Qs[2][kQStage][kQPad];
-    __shared__ __attribute__((aligned(16))) float Ls[2][kQStage];
+    constexpr int kWaveKeys = 32 * KS, kKeysPerWg = 4 * kWaveKeys, kQStage = QS;
+    extern __shared__ __attribute__((aligned(16))) char score_lds[];
+    bf16_t(*Qs)[kQStage][kQPad] = (bf16_t(*)[kQStage][kQPad])score_lds;                               // [2][QS][kQPad]
+    float(*Ls)[kQStage] = (float(*)[kQStage])(score_lds + 2 * kQStage * kQPad * sizeof(bf16_t));      // [2][QS]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
@@ -73,12 +75,12 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     const bf16_t *qbase = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
     const float *lse = a.d_lse + ((int64_t)b * a.H + h) * a.Lq;
     const int ld_chunk = tid & 15, ld_row = tid >> 4;
-    u32x4 qbuf[4];
+    u32x4 qbuf[kQStage / 16];
     float lbuf = 0.f;
     auto load_stage = [&](int s) {
         const int i0 = s * kQStage;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kQStage / 16; ++i) {
             const int qi = i0 + ld_row + 16 * i;
             qbuf[i] = qi < a.Lq ? *(const u32x4 *)(qbase + (int64_t)qi * a.q_sl + ld_chunk * 8) : u32x4{0, 0, 0, 0};
         }
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     };
     auto store_stage = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *(u32x4 *)&Qs[buf][ld_row + 16 * i][ld_chunk * 8] = qbuf[i];
+        for (int i = 0; i < kQStage / 16; ++i) *(u32x4 *)&Qs[buf][ld_row + 16 * i][ld_chunk * 8] = qbuf[i];
         if (tid < kQStage) Ls[buf][tid] = lbuf;
     };
 
@@ -102,7 +104,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
         const int64_t i0 = (int64_t)s * kQStage;
         if (i0 < w_hi && i0 + kQStage > w_lo) {                  // wave-uniform
 #pragma unroll
-            for (int qs = 0; qs < 2; ++qs) {
+            for (int qs = 0; qs < kQStage / 32; ++qs) {
                 const int64_t iq = i0 + qs * 32;
                 if (iq >= w_hi || iq + 32 <= w_lo) continue;
                 bf16x8 qa[kD / 16];                              // A operand: lane = query row
@@ -185,12 +187,22 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
     INFLLM_REQUIRE((a->q_sl % 8 | a->q_sh % 8 | a->q_sb % 8 | a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8) == 0,
                    "local_score: strides must be multiples of 8");
     if (a->j_hi <= a->j_lo) return 0;
+    auto lds_bytes = [](int qs) { return (size_t)(2 * qs * kQPad * sizeof(bf16_t) + 2 * qs * sizeof(float)); };
     if (a->j_hi - a->j_lo > 1024) {
         const int64_t tiles = (a->j_hi - 1) / 64 - a->j_lo / 64 + 1;
-        hipLaunchKernelGGL(local_score_kernel<2>, dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL((local_score_kernel<2, 64>), dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), lds_bytes(64),
+                           (hipStream_t)stream, *a);
     } else {
+        static bool lds_set = false;                   // dynamic LDS above 64 KiB must be enabled once
+        if (!lds_set) {
+            hipError_t e = hipFuncSetAttribute((const void *)local_score_kernel<1, 128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               (int)lds_bytes(128));
+            if (e != hipSuccess) return infllm_fail(-2, "local_score: %s", hipGetErrorString(e));
+            lds_set = true;
+        }
         const int64_t tiles = (a->j_hi - 1) / 32 - a->j_lo / 32 + 1;
-        hipLaunchKernelGGL(local_score_kernel<1>, dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+        hipLaunchKernelGGL((local_score_kernel<1, 128>), dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), lds_bytes(128),
+                           (hipStream_t)stream, *a);
     }
     INFLLM_CHECK_LAUNCH("local_score");
     return 0;
