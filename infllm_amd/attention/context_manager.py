@@ -112,6 +112,8 @@ class CachePolicy:
 
 
 class ContextManager:
+    select_in_steps = False     # True: drive wait / policy / fetch from here (slower), instead of infllm_block_select
+
     def __init__(self, position_embedding, n_init, n_local, block_size, max_cached_block, topk, exc_block_size,
                  score_decay=None, fattn=False, repr_topk=1, cache_strategy="lru", chunk_topk_calc=None,
                  async_global_stream=False, pin_memory=False, faiss=False, perhead=False):
@@ -364,31 +366,33 @@ class ContextManager:
             for u in range(B):
                 self.policy[u].add_scores(self._mass_units[u], masses[u][:len(self._mass_units[u])])
             self._mass_units = None
-        if preselected is not None or N <= topk:
-            # chosen for the whole chunk (context_manager.py:381-382), or every unit there is
-            selected = preselected if preselected is not None else [list(range(N))] * B
-            n_sel = len(selected[0])
-            for u in range(B):
-                self._sel_ids[u * n_sel:(u + 1) * n_sel] = selected[u]
-            sa.h_selected, sa.n_sel, sa.wait_topk = ctypes.addressof(self._sel_ids), n_sel, 0
-            n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
+        if self.select_in_steps:
+            n_sel, n_miss, selected = self._select_stepwise(preselected, N)
         else:
-            n_sel = topk
-            sa.h_selected, sa.n_sel, sa.wait_topk = self.topk_idx_host.data_ptr(), n_sel, 1     # the one host wait of a block
-            n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
-            selected = None                                   # read back below, off the chain
-        if n_miss < 0:
-            check(n_miss, "infllm_block_select")
-        # the transfer has started; everything from here on overlaps it
-        if selected is None:
-            selected = self.topk_idx_host.tolist()
-        n_ev = sum(self._n_evicted[:B])
+            if preselected is not None or N <= topk:
+                # chosen for the whole chunk (context_manager.py:381-382), or every unit there is
+                selected = preselected if preselected is not None else [list(range(N))] * B
+                n_sel = len(selected[0])
+                for u in range(B):
+                    self._sel_ids[u * n_sel:(u + 1) * n_sel] = selected[u]
+                sa.h_selected, sa.n_sel, sa.wait_topk = ctypes.addressof(self._sel_ids), n_sel, 0
+                n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
+            else:
+                n_sel = topk
+                sa.h_selected, sa.n_sel, sa.wait_topk = self.topk_idx_host.data_ptr(), n_sel, 1   # the one host wait of a block
+                n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
+                selected = None                                   # read back below, off the chain
+            if n_miss < 0:
+                check(n_miss, "infllm_block_select")
+            # the transfer has started; everything from here on overlaps it
+            if selected is None:
+                selected = self.topk_idx_host.tolist()
+            stats["evictions"] += sum(self._n_evicted[:B])
+            for u in range(B):
+                if self.policy[u].evicted_log is not None:
+                    self.policy[u].evicted_log.append(list(self._evicted[u * n_sel:u * n_sel + self._n_evicted[u]]))
         stats["hits"] += B * n_sel - n_miss
         stats["misses"] += n_miss
-        stats["evictions"] += n_ev
-        for u in range(B):
-            if self.policy[u].evicted_log is not None:
-                self.policy[u].evicted_log.append(list(self._evicted[u * n_sel:u * n_sel + self._n_evicted[u]]))
         if self.cache_strategy == "lru":
             self.load_count += 1
         # ---- state machine after the block (context_manager.py:614-679)
@@ -426,6 +430,34 @@ class ContextManager:
         self.init_len = init_len + take
         self.cursor = cursor + take + c * bs
         self.num_global_block = N + c
+
+    def _select_stepwise(self, preselected, N):
+        """The same as infllm_block_select in the separate steps the C ABI also offers (a caller with a policy of
+        its own would use them): wait for the ids, one infllm_cache_touch per row, build the lists, issue the fetch."""
+        lib, layer, B = self._lib, self._layer, self.num_units
+        if preselected is not None:
+            selected = preselected
+        elif N <= self.topk:
+            selected = [list(range(N))] * B
+        else:
+            check(lib.infllm_layer_wait_topk(layer), "infllm_layer_wait_topk")
+            selected = self.topk_idx_host.tolist()
+        n_sel, n_miss = len(selected[0]), 0
+        for u in range(B):
+            pol = self.policy[u]
+            misses, evicted = pol.touch(selected[u])
+            self.stats["evictions"] += len(evicted)
+            slot_of = pol.slot_of
+            for i, unit in enumerate(selected[u]):
+                self._sel_slots[u * n_sel + i] = slot_of[unit]
+            for unit in misses:
+                chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
+                self._miss_row[n_miss], self._miss_slot[n_miss], self._miss_unit[n_miss] = u, slot_of[unit], unit
+                self._miss_src[n_miss] = self._host_dev_base[chunk] + idx * self.unit_bytes + u * self.slot_bytes
+                n_miss += 1
+        check(lib.infllm_block_fetch(layer, n_miss, self._miss_row, self._miss_slot, self._miss_unit, self._miss_src,
+                                     self._main_raw, self._copy_raw), "infllm_block_fetch")
+        return n_sel, n_miss, selected
 
     def _chunk_topk(self, q, c0, c1):
         """Selections of every execution block of q[:, :, c0:c1] against the units that exist now

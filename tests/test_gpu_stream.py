@@ -205,6 +205,24 @@ def test_carved_units_reach_the_host_by_either_copy_path(monkeypatch):
             assert torch.equal(hu[0, 0], k[0, :, lo:lo + bs]) and torch.equal(hu[0, 1], v[0, :, lo:lo + bs]), u
 
 
+def test_selection_in_separate_steps_equals_the_fused_call(monkeypatch):
+    """infllm_layer_wait_topk + infllm_cache_touch + infllm_block_fetch, driven from the host, against
+    infllm_block_select: same outputs, same residency events, for every policy."""
+    from infllm_amd.attention import ContextManager
+    T = 1400
+    q, k, v = _stream(T, 8, 2, 15, B=2)
+    for extra in (dict(), dict(cache_strategy="fifo"), dict(cache_strategy="lru-s", score_decay=0.5)):
+        kw = dict(SMALL, max_cached_block=5, async_global_stream=True, **extra)
+        monkeypatch.setattr(ContextManager, "select_in_steps", False)
+        fused, cm0 = _run_gpu(q, k, v, [700, 700], 1e4, **kw)
+        monkeypatch.setattr(ContextManager, "select_in_steps", True)
+        steps, cm1 = _run_gpu(q, k, v, [700, 700], 1e4, **kw)
+        assert torch.equal(fused, steps) and cm0.stats == cm1.stats and cm0.stats["misses"] > 0
+        for u in range(2):
+            assert cm0.policy[u].evicted_log == cm1.policy[u].evicted_log
+            assert cm0.policy[u].cached == cm1.policy[u].cached and cm0.policy[u].slot_of == cm1.policy[u].slot_of
+
+
 def test_state_export_and_injection_resume_the_stream_exactly():
     from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
     T0, T1 = 900, 333
