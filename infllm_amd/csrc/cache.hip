@@ -4,9 +4,10 @@
 // interpreter takes an order of magnitude longer over it.
 //
 // The reference keeps a dict unit -> value and evicts in ascending value, first-inserted first on ties (a stable
-// sort over the dict's insertion order), never a unit of the current selection.  Here every resident carries the
-// sequence number of its insertion, so (value, sequence) is the same order.  Values are doubles: the lru / fifo
-// clocks are small integers, the lru-s scores are the reference's Python floats (same operations, same order).
+// sort over the dict's insertion order), never a unit of the current selection.  Here the residents sit in a vector
+// in insertion order (an evicted unit that comes back goes to the end, as in the dict), and the eviction is a stable
+// sort of that vector by value.  Values are doubles: the lru / fifo clocks are small integers, the lru-s scores are
+// the reference's Python floats (same operations, same order).
 #include <algorithm>
 #include <vector>
 
@@ -17,13 +18,12 @@ namespace {
 struct Resident {
     int32_t unit, slot;
     double value;
-    int64_t seq;
 };
 
 struct UnitCache {
     int capacity, strategy;
     double decay;
-    int64_t clock = 0, next_seq = 0;
+    int64_t clock = 0;
     std::vector<Resident> res;          // in insertion order
     std::vector<int32_t> free_slots;    // used from the back
     std::vector<int32_t> order;         // scratch
@@ -105,7 +105,7 @@ extern "C" int infllm_cache_touch(void *cache, const int32_t *selected, int32_t 
         if (r) {
             if (c.strategy != INFLLM_CACHE_FIFO) r->value = v;          // fifo keeps the clock of the first load
         } else {
-            Resident nr{selected[i], -1, v, c.next_seq++};
+            Resident nr{selected[i], -1, v};
             c.res.push_back(nr);
         }
     }

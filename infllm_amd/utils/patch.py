@@ -14,8 +14,6 @@ patched model ``forward`` puts and collects them; RoPE base and head counts come
 """
 import types
 
-import torch
-
 from ..attention import ATTN_FORWRAD, RotaryEmbeddingESM
 
 

@@ -3,8 +3,6 @@
 Restates inf_llm/attention/inf_llm.py:5-77 with StreamOracle in place of ContextManager, so that a decoder
 patched with it is the fp32 CPU counterpart of the same decoder patched with the product's attention type.
 """
-import torch
-
 from .rope import RopeOracle
 from .stream import StreamOracle
 

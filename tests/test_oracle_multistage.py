@@ -1,7 +1,6 @@
 """Pins for oracle.multistage (restating torch_impl.py): library softmax / SDPA and brute force."""
 import math
 
-import pytest
 import torch
 import torch.nn.functional as F
 
