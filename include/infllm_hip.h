@@ -150,6 +150,13 @@ int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t
                       int32_t B, int32_t H, int32_t Lq,
                       void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
                       float *d_lse, void *stream);
+/* The operator's whole forward in one call (attn.append(local...), attn.append(global..., end=True),
+ * attn.get_result(): context_manager.py:486-489, 526-533): the local stage over a ring or tensor, the global
+ * stage over a page table (either may be NULL), and their merge into d_out / d_lse.  The stages keep their own
+ * nsplit; the global stage's partial buffers must directly follow the local stage's
+ * (global->d_o_part == local->d_o_part + local->nsplit*B*H*Lq*128, likewise d_lse_part). */
+int infllm_attn_fwd(const infllm_attn_args *local, const infllm_attn_args *global,
+                    void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse, void *stream);
 
 /* ---------------------------------------------------------------------------
  * Column sums of the final probabilities of one linear stage
@@ -224,6 +231,8 @@ int infllm_gather_rows(const void *d_ring, int64_t ring_cap, int32_t B, int32_t 
                        int64_t t0, int32_t n, int32_t unit_rows, void *d_out, int64_t out_sb,
                        int64_t out_su, int64_t out_sh, void *stream);
 int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int32_t kind, void *stream);
+/* the same under the name the cache's own transfers go by (MemoryUnit.load / offload, context_manager.py:64-109) */
+int infllm_cache_copy_async(void *dst, const void *src, int64_t nbytes, int32_t kind, void *stream);
 /* infllm_fetch_units: n copies of nbytes each, pinned host -> device, in ONE kernel launch that reads the
  *   device-mapped pinned memory directly (the misses of a block are scattered over the host arena; issuing a
  *   hipMemcpyAsync per 512 KiB unit costs more than moving it).  h_src[i] must be the device-visible address

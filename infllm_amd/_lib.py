@@ -130,6 +130,7 @@ SYMBOLS = {
     "infllm_rope_rows": (c_i32, [c_vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_i32, c_i64, c_i32, c_vp, C.c_double, c_vp, c_vp]),
     "infllm_attn_stage": (c_i32, [C.POINTER(AttnArgs), c_vp]),
     "infllm_attn_merge": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
+    "infllm_attn_fwd": (c_i32, [C.POINTER(AttnArgs), C.POINTER(AttnArgs), c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
     "infllm_local_score": (c_i32, [C.POINTER(ScoreArgs), c_vp]),
     "infllm_unit_scores": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp]),
     "infllm_topk": (c_i32, [c_vp, c_i32, c_i32, c_vp, c_vp]),
@@ -138,6 +139,7 @@ SYMBOLS = {
                                  c_vp, c_i64, c_i64, c_vp, c_vp]),
     "infllm_gather_rows": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i64, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp]),
     "infllm_copy_async": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_vp]),
+    "infllm_cache_copy_async": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_vp]),
     "infllm_fetch_units": (c_i32, [c_vp, c_vp, c_i32, c_i64, c_vp]),
     "infllm_host_device_pointer": (c_vp, [c_vp]),
     "infllm_layer_create": (c_vp, [C.POINTER(LayerDesc)]),

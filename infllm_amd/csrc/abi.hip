@@ -34,6 +34,10 @@ extern "C" int infllm_copy_async(void *dst, const void *src, int64_t nbytes, int
     return 0;
 }
 
+extern "C" int infllm_cache_copy_async(void *dst, const void *src, int64_t nbytes, int32_t kind, void *stream) {
+    return infllm_copy_async(dst, src, nbytes, kind, stream);
+}
+
 // ---------------------------------------------------------------------------
 // Unit fetch: pinned host memory -> device slots in ONE launch.
 // The sources of a block's cache misses are scattered over the host arena, and a

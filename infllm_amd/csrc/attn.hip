@@ -626,6 +626,33 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
 
 extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
                                  int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
+                                 void *stream);
+
+extern "C" int infllm_attn_fwd(const infllm_attn_args *local, const infllm_attn_args *global, void *d_out, int64_t o_sb,
+                               int64_t o_sh, int64_t o_sl, float *d_lse, void *stream) {
+    INFLLM_REQUIRE(local || global, "attn_fwd: no stage given");
+    INFLLM_REQUIRE(d_out || d_lse, "attn_fwd: neither output nor lse requested");
+    const infllm_attn_args *first = local ? local : global;
+    int parts = first->nsplit;
+    if (local && global) {
+        INFLLM_REQUIRE(local->B == global->B && local->H == global->H && local->Lq == global->Lq,
+                       "attn_fwd: the two stages disagree on B / H / Lq");
+        const int64_t rows = (int64_t)local->B * local->H * local->Lq;
+        INFLLM_REQUIRE(global->d_o_part == local->d_o_part + (int64_t)local->nsplit * rows * kD &&
+                           global->d_lse_part == local->d_lse_part + (int64_t)local->nsplit * rows,
+                       "attn_fwd: the global stage's partials must follow the local stage's in one buffer");
+        parts += global->nsplit;
+    }
+    int rc = local ? infllm_attn_stage(local, stream) : 0;
+    if (rc) return rc;
+    rc = global ? infllm_attn_stage(global, stream) : 0;
+    if (rc) return rc;
+    return infllm_attn_merge(first->d_o_part, first->d_lse_part, parts, first->B, first->H, first->Lq, d_out, o_sb, o_sh, o_sl,
+                             d_lse, stream);
+}
+
+extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
+                                 int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
                                  void *stream) {
     INFLLM_REQUIRE(d_o_part && d_lse_part, "attn_merge: null pointer");
     INFLLM_REQUIRE(P >= 1 && B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes P=%d B=%d H=%d Lq=%d", P, B, H, Lq);

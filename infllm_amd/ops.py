@@ -99,9 +99,9 @@ def block_mean(q_glb, B, H, n, exc, qbar):
     check(_lib.load().infllm_block_mean(q_glb.data_ptr(), B, H, n, exc, qbar.data_ptr(), _stream()), "infllm_block_mean")
 
 
-def attn_stage_linear(q, k, v, o_part, lse_part, *, cap=None, j_lo=0, j_hi=None, mask=MASK_NONE, offset=0, window=0,
+def linear_stage_args(q, k, v, o_part, lse_part, *, cap=None, j_lo=0, j_hi=None, mask=MASK_NONE, offset=0, window=0,
                       nsplit=1, softmax_scale=None):
-    """One stage over a linear key source.  q [B,H,Lq,D]; k/v [B,Hkv,rows,D] (rows = ring rows)."""
+    """Argument block of one stage over a linear key source.  q [B,H,Lq,D]; k/v [B,Hkv,rows,D] (rows = ring rows)."""
     B, H, Lq, D = q.shape
     Hkv = k.shape[1]
     if cap is None:
@@ -120,11 +120,11 @@ def attn_stage_linear(q, k, v, o_part, lse_part, *, cap=None, j_lo=0, j_hi=None,
     a.d_pages, a.n_pages, a.nsplit = None, 0, nsplit
     a.softmax_scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
     a.d_o_part, a.d_lse_part = o_part.data_ptr(), lse_part.data_ptr()
-    check(_lib.load().infllm_attn_stage(a, _stream()), "infllm_attn_stage")
+    return a
 
 
-def attn_stage_paged(q, pages_dev, n_pages, Hkv, o_part, lse_part, *, nsplit=1, softmax_scale=None):
-    """One stage over a device page table [B, n_pages] of infllm_page entries."""
+def paged_stage_args(q, pages_dev, n_pages, Hkv, o_part, lse_part, *, nsplit=1, softmax_scale=None):
+    """Argument block of one stage over a device page table [B, n_pages] of infllm_page entries."""
     B, H, Lq, D = q.shape
     _need(o_part.dtype == torch.float16 and lse_part.dtype == torch.float32, "partials are fp16 rows with fp32 log-sum-exps")
     a = AttnArgs()
@@ -134,7 +134,25 @@ def attn_stage_paged(q, pages_dev, n_pages, Hkv, o_part, lse_part, *, nsplit=1, 
     a.cap = KEY_TILE
     a.softmax_scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(D)
     a.d_o_part, a.d_lse_part = o_part.data_ptr(), lse_part.data_ptr()
-    check(_lib.load().infllm_attn_stage(a, _stream()), "infllm_attn_stage")
+    return a
+
+
+def attn_stage_linear(q, k, v, o_part, lse_part, **kw):
+    """One stage over a linear key source (see linear_stage_args)."""
+    check(_lib.load().infllm_attn_stage(linear_stage_args(q, k, v, o_part, lse_part, **kw), _stream()), "infllm_attn_stage")
+
+
+def attn_stage_paged(q, pages_dev, n_pages, Hkv, o_part, lse_part, **kw):
+    """One stage over a device page table (see paged_stage_args)."""
+    check(_lib.load().infllm_attn_stage(paged_stage_args(q, pages_dev, n_pages, Hkv, o_part, lse_part, **kw), _stream()),
+          "infllm_attn_stage")
+
+
+def attn_fwd(local_args, global_args, out, lse):
+    """Both stages (either may be None) and their merge in one call; out bf16 [B,H,Lq,D], lse fp32 [B,H,Lq] or None."""
+    _need(out.stride(-1) == 1 and out.dtype == torch.bfloat16, "bad merge output")
+    check(_lib.load().infllm_attn_fwd(local_args, global_args, out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+                                      lse.data_ptr() if lse is not None else None, _stream()), "infllm_attn_fwd")
 
 
 def attn_merge(o_part, lse_part, P, out, lse):

@@ -224,6 +224,23 @@ def test_two_stage_joint_softmax_with_ring_and_pages():
     lse = torch.empty((B, H, Lq), dtype=torch.float32, device="cuda")
     ops.attn_merge(o_part, lse_part, 2, out, lse)
     _check_out(out, want)
+    # the same through the one-call forward (both stages + merge), with 2 + 1 key splits: same partial layout rules
+    o3 = torch.empty((3, B, H, Lq, D), dtype=torch.float16, device="cuda")
+    l3 = torch.empty((3, B, H, Lq), dtype=torch.float32, device="cuda")
+    la = ops.linear_stage_args(qd, ring_k, ring_v, o3[0:2], l3[0:2], cap=cap, j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW,
+                               offset=b0, window=n_local, nsplit=2)
+    ga = ops.paged_stage_args(qd, pages, len(ent), Hkv, o3[2:3], l3[2:3])
+    out2, lse2 = torch.empty_like(out), torch.empty_like(lse)
+    ops.attn_fwd(la, ga, out2, lse2)
+    _check_out(out2, want)
+    assert torch.allclose(lse2, lse, atol=1e-4)
+    out3 = torch.empty_like(out)
+    ops.attn_fwd(None, ga, out3, None)                       # one stage alone
+    ops.attn_merge(o_part[1:2], lse_part[1:2], 1, out2, None)
+    assert torch.equal(out3, out2)
+    from infllm_amd._lib import InfLLMHipError
+    with pytest.raises(InfLLMHipError):                      # partial buffers that do not follow one another
+        ops.attn_fwd(la, ops.paged_stage_args(qd, pages, len(ent), Hkv, o_part[1:2], lse_part[1:2]), out2, None)
     score = torch.zeros((B, H, cap), dtype=torch.float32, device="cuda")
     ops.local_score(qd, ring_k, lse, score, cap=cap, j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW, offset=b0, window=n_local,
                     accumulate=True, score_cap=cap)

@@ -68,6 +68,43 @@ def test_patch_hf_overrides_base_and_forwards_type_arguments():
         del attention.ATTN_FORWRAD["probe"]
 
 
+def test_yaml_configuration_feeds_patch_hf_like_the_reference_driver(tmp_path):
+    """A run configuration in the reference's layout (config/*.yaml), loaded with the defaults and command-line
+    overrides of benchmark/pred.py:22-40, and its model section handed to patch_hf wholesale (pred.py:56)."""
+    from infllm_amd.utils import load_config, patch_from_config
+    path = tmp_path / "run.yaml"
+    path.write_text("model:\n  type: probe\n  path: some/model\n  block_size: 128\n  n_init: 128\n  n_local: 4096\n"
+                    "  topk: 16\n  repr_topk: 4\n  max_cached_block: 32\n  exc_block_size: 512\n  fattn: false\n"
+                    "  base: 1000000\n  distance_scale: 1.0\n\nmax_len: 2147483647\nchunk_size: 8192\nconv_type: mistral-inst\n")
+    conf = load_config(str(path), ["model.topk=8", "--model.score_decay=0.1", "extra.note=hello", "chunk_size=4096"])
+    assert conf.model.topk == 8 and conf.model.score_decay == 0.1 and conf.extra.note == "hello" and conf.chunk_size == 4096
+    assert conf.model.tokenizer_path == "some/model" and conf.truncation is None and conf.model.fattn is False
+    assert conf.max_len == 2147483647 and conf["model"]["n_local"] == 4096
+    got = {}
+
+    def factory(**kw):
+        got.update(kw)
+        return lambda self, q, kv, rope, use_cache, past, pq, pk, pv, po, d, h, hk: (po(pq(q)), rope)
+    attention.ATTN_FORWRAD["probe"] = factory
+    try:
+        model = patch_from_config(_tiny(), conf)
+        rope = model(input_ids=torch.zeros((1, 2), dtype=torch.long), use_cache=True, return_dict=True).past_key_values[0]
+    finally:
+        del attention.ATTN_FORWRAD["probe"]
+    # base / distance_scale go to the rotary embedding, everything else (type and paths included) to the attention type
+    assert rope.base == 1000000 and rope.distance_scale == 1.0
+    assert got["topk"] == 8 and got["n_local"] == 4096 and got["path"] == "some/model" and "base" not in got
+    # the real attention types swallow the keys that are not theirs (inf_llm.py:5-18 ends in *args, **kwargs)
+    conf.model.type = "inf-llm"
+    assert callable(attention.ATTN_FORWRAD[conf.model.type](**{k: v for k, v in conf.model.items() if k not in ("base", "distance_scale")}))
+    for bad in (["model.topk"], ["=3"]):
+        with pytest.raises(ValueError):
+            load_config(str(path), bad)
+    (tmp_path / "empty.yaml").write_text("max_len: 3\n")
+    with pytest.raises(ValueError):
+        load_config(str(tmp_path / "empty.yaml"))
+
+
 class _Tok:
     eos_token_id = 1
 
