@@ -277,8 +277,13 @@ void *infllm_host_device_pointer(void *h_pinned);
  * for the engine copies, and must be called when no further block follows (end of an append()
  * call); after it and a synchronisation of the copy stream the host copies are complete.
  *
- * A layer handle owns only events, the rotation of the pinned page-table staging slots and of
- * the carve staging slots; every buffer is the caller's.
+ * The next block's selection is prepared in two parts: the top-k of the units that exist when
+ * infllm_block_front prepares the next block is taken there (off the chain), and after the block only
+ * those k candidates and the units carved in between are ranked (same result as one top-k over all).
+ *
+ * A layer handle owns only events, ROCr signals, a [B,topk] device array for those candidates, the
+ * rotation of the pinned page-table staging slots and of the carve staging slots; every other buffer
+ * is the caller's.
  */
 typedef struct {
     int32_t B, H, Hkv;

@@ -298,6 +298,27 @@ __global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *sco
     publish(flag, flag_value);
 }
 
+// The selection over ALL units from two parts: the k best of the units that existed earlier (`cand`, ids ascending,
+// chosen by the kernels above while other work was still in flight) and the n_new units carved since, whose scores
+// arrive last.  A unit of the overall top-k that is not new is among the k best of the old ones, so ranking these
+// n_cand + n_new <= 64 candidates by (key, lower id first) gives the same set, written in ascending id as above.
+__global__ __launch_bounds__(64) void topk_merge_kernel(const float *scores, const int32_t *cand, int n_cand, int first_new,
+                                                        int n_new, int k, int32_t *idx_out, int32_t *flag, int32_t flag_value) {
+    const int lane = threadIdx.x, n = n_cand + n_new;
+    const bool valid = lane < n;
+    const int id = lane < n_cand ? cand[lane] : first_new + (lane - n_cand);       // ascending in the lane
+    const uint32_t key = valid ? order_key(scores[id]) : 0u;
+    int rank = 0;
+    for (int j = 0; j < n; ++j) {
+        const uint32_t kj = __shfl(key, j, 64);
+        rank += (kj > key || (kj == key && j < lane)) ? 1 : 0;
+    }
+    const bool sel = valid && rank < k;
+    const uint64_t mask = __ballot(sel);
+    if (sel) idx_out[__popcll(mask & ((1ull << lane) - 1))] = id;
+    publish(flag, flag_value);
+}
+
 // ---------------------------------------------------------------- representative keys
 constexpr int kMaxUnit = 2048;             // largest supported unit (block_size)
 
@@ -400,6 +421,18 @@ int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_
     default: hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_flag, flag_value);
     }
     INFLLM_CHECK_LAUNCH("topk");
+    return 0;
+}
+
+// internal: see topk_merge_kernel
+int infllm_topk_merge_publish(const float *d_scores, const int32_t *d_cand, int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k,
+                              int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream) {
+    INFLLM_REQUIRE(d_scores && d_cand && d_idx, "topk_merge: null pointer");
+    INFLLM_REQUIRE(n_cand >= 0 && n_new >= 0 && n_cand + n_new <= 64 && k > 0 && k <= n_cand + n_new && first_new >= 0,
+                   "topk_merge: %d + %d candidates for k=%d", n_cand, n_new, k);
+    hipLaunchKernelGGL(topk_merge_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, d_scores, d_cand, n_cand, first_new, n_new, k,
+                       d_idx, d_flag, flag_value);
+    INFLLM_CHECK_LAUNCH("topk_merge");
     return 0;
 }
 

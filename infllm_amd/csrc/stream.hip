@@ -51,6 +51,10 @@ struct Layer {
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
     int32_t topk_seq = 0;
+    // the top-k of the units that existed when the next block was prepared, chosen ahead of the chain: [B,topk]
+    // device ids (this handle's own allocation) and the unit count they were chosen from (-1: none)
+    int32_t *d_cand = nullptr;
+    int cand_units = -1;
     bool has_global = false;
     bool topk_pending = false;
     int slot = 0;                         // workspace slot written last
@@ -85,6 +89,8 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_topk_merge_publish(const float *d_scores, const int32_t *d_cand, int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k,
+                              int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
 namespace {
 
 int splits_for(const infllm_layer_desc &d, int n_queries, int n_tiles) {
@@ -390,6 +396,10 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         infllm_layer_destroy(L);
         return bad("hipEventCreate failed");
     }
+    if (d.topk > 0 && hipMalloc((void **)&L->d_cand, sizeof(int32_t) * d.B * d.topk) != hipSuccess) {
+        L->d_cand = nullptr;                        // not fatal: selections then run over all units every time
+        (void)hipGetLastError();
+    }
     L->dma_busy.assign(d.carve_slots, 0);
     L->dma_first.assign(d.carve_slots, 0);
     L->dma_count.assign(d.carve_slots, 0);
@@ -420,6 +430,7 @@ extern "C" int infllm_layer_destroy(void *layer) {
     for (auto &t : L->timer)
         for (hipEvent_t e : t.ev)
             if (e) (void)hipEventDestroy(e);
+    if (L->d_cand) (void)hipFree(L->d_cand);
     delete L;
     return 0;
 }
@@ -514,6 +525,25 @@ int run_topk(Layer *L, const float *scores, int64_t scores_sb, int n_units, void
     return 0;
 }
 
+// the selection for the next block from the candidates chosen ahead and the n_new units carved since
+int run_topk_merge(Layer *L, const float *scores, int64_t scores_sb, int n_old, int n_new, void *stream) {
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream;
+    const bool poll = d.d_topk_flag && d.h_topk_flag && !d.h_topk_idx;
+    if (poll) ++L->topk_seq;
+    for (int u = 0; u < d.B; ++u) {
+        const bool last = poll && u == d.B - 1;
+        int rc = infllm_topk_merge_publish(scores + (int64_t)u * scores_sb, L->d_cand + (int64_t)u * d.topk, d.topk, n_old, n_new, d.topk,
+                                           d.d_topk_idx + (int64_t)u * d.topk, last ? d.d_topk_flag : nullptr, L->topk_seq, stream);
+        if (rc) return rc;
+    }
+    if (d.h_topk_idx)
+        HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
+    HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    L->topk_pending = true;
+    return 0;
+}
+
 int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t j_hi, void *stream) {
     const infllm_layer_desc &d = L->d;
     if (j_hi <= j_lo) return 0;
@@ -590,6 +620,17 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
             rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->slot, stream);
             if (rc) return rc;
+            // their k best now, while the fetch is in flight: the selection after the block then only has to weigh these
+            // against the few units carved in between, instead of running over every unit on the chain
+            L->cand_units = -1;
+            if (L->d_cand && a->n_units > d.topk) {
+                for (int u = 0; u < d.B; ++u) {
+                    rc = infllm_topk_publish(a->d_unit_scores + (int64_t)u * a->unit_scores_sb, a->n_units, d.topk,
+                                             L->d_cand + (int64_t)u * d.topk, nullptr, 0, stream);
+                    if (rc) return rc;
+                }
+                L->cand_units = a->n_units;
+            }
         }
         L->prepared = true;
         L->prepared_b0 = b1;
@@ -878,9 +919,13 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->slot,
                              stream);
         if (rc) return rc;
-        rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, n_units_next, stream);
+        if (L->cand_units == a->n_units && d.topk + a->n_carve <= 64)
+            rc = run_topk_merge(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, stream);
+        else
+            rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, n_units_next, stream);
         if (rc) return rc;
     }
+    L->cand_units = -1;
     // ---- 5b. the block's output rows
     rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, nullptr, stream);
     if (rc) return rc;
