@@ -127,24 +127,33 @@ __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
     }
 }
 
-// out[b, c] = scale * sum_p parts[b, p, c], p ascending
-__global__ __launch_bounds__(64) void reduce_partials_kernel(const float *parts, int n_parts, int C, float scale,
-                                                             float *out) {
-    const int c = blockIdx.x * 64 + threadIdx.x, b = blockIdx.y;
-    if (c >= C) return;
+// out[b, c] = scale * sum_p parts[b, p, c], p ascending.  A workgroup owns 64 columns; its 4 waves fetch different
+// partials, so that 32 of them are one round trip to memory (a chain of dependent loads is all latency, and that
+// latency multiplies while a unit fetch keeps the memory fabric busy); the sum itself runs in the fixed order.
+__global__ __launch_bounds__(256) void reduce_partials_kernel(const float *parts, int n_parts, int C, float scale,
+                                                              float *out) {
+    __shared__ float stage[32][64];
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + lane, b = blockIdx.y;
     const float *src = parts + (int64_t)b * n_parts * C + c;
     float s = 0.f;
-    // the order of the sum stays p ascending; the loads of 16 partials are in flight together, because a chain of
-    // dependent loads is all latency (and that latency multiplies while a unit fetch keeps the memory fabric busy)
-    for (int p0 = 0; p0 < n_parts; p0 += 16) {
-        float v[16];
+    for (int p0 = 0; p0 < n_parts; p0 += 32) {
+        float v[8];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = p0 + i < n_parts ? src[(int64_t)(p0 + i) * C] : 0.f;
+        for (int i = 0; i < 8; ++i) {
+            const int p = p0 + grp + 4 * i;
+            v[i] = (c < C && p < n_parts) ? src[(int64_t)p * C] : 0.f;
+        }
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
-            if (p0 + i < n_parts) s += v[i];
+        for (int i = 0; i < 8; ++i) stage[grp + 4 * i][lane] = v[i];
+        __syncthreads();
+        if (grp == 0) {
+            const int m = min(32, n_parts - p0);
+            for (int p = 0; p < m; ++p) s += stage[p][lane];
+        }
+        __syncthreads();
     }
-    out[(int64_t)b * C + c] = s * scale;
+    if (grp == 0 && c < C) out[(int64_t)b * C + c] = s * scale;
 }
 
 constexpr int kMeanThreads = 512;
@@ -240,10 +249,15 @@ __global__ __launch_bounds__(256) void rope_rows_kernel(const bf16_t *x, int64_t
     ((uint16_t *)dst)[lane + kD / 2] = (uint16_t)(pack_bf16x2(hi * c + lo * s, 0.f) & 0xffffu);
 }
 
+// grid.z = B, or 2*B to gather from a second ring (ring2 -> out2, same geometry) in the same launch
 __global__ __launch_bounds__(256) void gather_rows_kernel(const bf16_t *ring, int64_t ring_cap, int Hkv, int64_t t0,
                                                           int n, int unit_rows, bf16_t *out, int64_t out_sb,
-                                                          int64_t out_su, int64_t out_sh) {
-    const int b = blockIdx.z, h = blockIdx.y;
+                                                          int64_t out_su, int64_t out_sh, int B, const bf16_t *ring2, bf16_t *out2) {
+    const int b = blockIdx.z % B, h = blockIdx.y;
+    if ((int)blockIdx.z >= B) {
+        ring = ring2;
+        out = out2;
+    }
     const int e = blockIdx.x * 256 + threadIdx.x;      // (row, 16-byte chunk)
     if (e >= n * 16) return;
     int r = e >> 4, c = e & 15;
@@ -279,7 +293,7 @@ extern "C" int infllm_reduce_partials(const float *d_parts, int32_t B, int32_t n
                                       void *stream) {
     INFLLM_REQUIRE(d_parts && d_out, "reduce_partials: null pointer");
     INFLLM_REQUIRE(B > 0 && n_parts > 0 && C > 0, "reduce_partials: bad sizes B=%d n_parts=%d C=%d", B, n_parts, C);
-    hipLaunchKernelGGL(reduce_partials_kernel, dim3((C + 63) / 64, B), dim3(64), 0, (hipStream_t)stream, d_parts, n_parts, C,
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((C + 63) / 64, B), dim3(256), 0, (hipStream_t)stream, d_parts, n_parts, C,
                        scale, d_out);
     INFLLM_CHECK_LAUNCH("reduce_partials");
     return 0;
@@ -330,7 +344,23 @@ extern "C" int infllm_gather_rows(const void *d_ring, int64_t ring_cap, int32_t 
     INFLLM_REQUIRE((out_sb % 8 | out_su % 8 | out_sh % 8) == 0, "gather_rows: output strides must be multiples of 8");
     if (n == 0) return 0;
     hipLaunchKernelGGL(gather_rows_kernel, dim3((n * 16 + 255) / 256, Hkv, B), dim3(256), 0, (hipStream_t)stream,
-                       (const bf16_t *)d_ring, ring_cap, Hkv, t0, n, unit_rows, (bf16_t *)d_out, out_sb, out_su, out_sh);
+                       (const bf16_t *)d_ring, ring_cap, Hkv, t0, n, unit_rows, (bf16_t *)d_out, out_sb, out_su, out_sh, B,
+                       (const bf16_t *)nullptr, (bf16_t *)nullptr);
+    INFLLM_CHECK_LAUNCH("gather_rows");
+    return 0;
+}
+
+// internal: the K and the V rows of the same stream positions in one launch (same arguments as infllm_gather_rows)
+int infllm_gather_rows_pair(const void *d_ring_a, void *d_out_a, const void *d_ring_b, void *d_out_b, int64_t ring_cap, int32_t B,
+                            int32_t Hkv, int64_t t0, int32_t n, int32_t unit_rows, int64_t out_sb, int64_t out_su, int64_t out_sh,
+                            void *stream) {
+    INFLLM_REQUIRE(d_ring_a && d_out_a && d_ring_b && d_out_b, "gather_rows: null pointer");
+    INFLLM_REQUIRE(B > 0 && Hkv > 0 && ring_cap > 0 && n >= 0 && n <= ring_cap && t0 >= 0 && unit_rows > 0, "gather_rows: bad sizes");
+    INFLLM_REQUIRE((out_sb % 8 | out_su % 8 | out_sh % 8) == 0, "gather_rows: output strides must be multiples of 8");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((n * 16 + 255) / 256, Hkv, 2 * B), dim3(256), 0, (hipStream_t)stream,
+                       (const bf16_t *)d_ring_a, ring_cap, Hkv, t0, n, unit_rows, (bf16_t *)d_out_a, out_sb, out_su, out_sh, B,
+                       (const bf16_t *)d_ring_b, (bf16_t *)d_out_b);
     INFLLM_CHECK_LAUNCH("gather_rows");
     return 0;
 }

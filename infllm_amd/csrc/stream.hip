@@ -89,6 +89,9 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_gather_rows_pair(const void *d_ring_a, void *d_out_a, const void *d_ring_b, void *d_out_b, int64_t ring_cap, int32_t B,
+                            int32_t Hkv, int64_t t0, int32_t n, int32_t unit_rows, int64_t out_sb, int64_t out_su, int64_t out_sh,
+                            void *stream);
 int infllm_topk_merge_publish(const float *d_scores, const int32_t *d_cand, int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k,
                               int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
 namespace {
@@ -954,11 +957,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         if (rc) return rc;
         const int64_t unit_all = (int64_t)d.B * slot_elems;                       // one unit, all batch rows
         bf16_t *stage = (bf16_t *)d.d_carve_stage + (int64_t)slot * d.max_carve * unit_all;
-        rc = infllm_gather_rows(d.d_ring_k_raw, d.ring_cap, d.B, d.Hkv, cursor, a->n_carve * bs, bs, stage, slot_elems, unit_all,
-                                (int64_t)bs * kD, stream);
-        if (rc) return rc;
-        rc = infllm_gather_rows(d.d_ring_v, d.ring_cap, d.B, d.Hkv, cursor, a->n_carve * bs, bs, stage + unit_elems, slot_elems,
-                                unit_all, (int64_t)bs * kD, stream);
+        rc = infllm_gather_rows_pair(d.d_ring_k_raw, stage, d.d_ring_v, stage + unit_elems, d.ring_cap, d.B, d.Hkv, cursor,
+                                     a->n_carve * bs, bs, slot_elems, unit_all, (int64_t)bs * kD, stream);
         if (rc) return rc;
         HIP_OK(hipEventRecord(L->carve_ready, st), "block_back: event");
         for (int i = 0; i < a->n_carve; ++i) INFLLM_REQUIRE(a->h_carve_dst[i], "block_back: null carve destination");
