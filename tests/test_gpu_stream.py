@@ -149,6 +149,21 @@ def test_unaligned_geometry_and_batch():
     _compare(700, [333, 367], H=6, Hkv=3, base=1e4, seed=7, B=2, **kw)
 
 
+def test_edge_knobs_and_empty_calls():
+    """No attention sinks, an execution block as long as the local window, a cache exactly as large as the
+    selection, one representative key per unit; calls of 1 and of 0 tokens in between."""
+    kw = dict(n_init=0, n_local=64, block_size=32, max_cached_block=2, topk=2, exc_block_size=64, repr_topk=1)
+    calls = [1, 63, 64, 300, 72]
+    cm, ora, _ = _compare(sum(calls), calls, H=4, Hkv=2, base=1e4, seed=21, **kw)
+    assert cm.init_len == 0 and cm.num_global_block == (sum(calls) - 64) // 32 and cm.stats["misses"] > 0
+    # an empty call changes nothing and returns an empty result
+    q, k, v = _stream(8, 4, 2, 22)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    before = (cm.length, cm.num_global_block, cm.cursor)
+    out = cm.append(qd[:, :, :0], kd[:, :, :0], vd[:, :, :0], qd[:, :, :0], kd[:, :, :0], vd[:, :, :0])
+    assert tuple(out.shape) == (1, 4, 0, D) and (cm.length, cm.num_global_block, cm.cursor) == before
+
+
 def test_many_batch_rows_take_the_host_built_page_table():
     """More than 64 selected (row, unit) pairs per block: the page table no longer fits a kernel argument and
     is staged through pinned memory instead."""
