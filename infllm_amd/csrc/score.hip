@@ -102,6 +102,59 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     for (int s = st_lo; s < st_hi; ++s) {
         const int cur = (s - st_lo) & 1;
         const int64_t i0 = (int64_t)s * kQStage;
+        // Fast path: every (query, key) pair of this stage and this wave's keys is visible.  Then the sub-tiles of 32
+        // queries are software pipelined: the MFMAs of sub-tile qs+1 are issued before the exponentials of sub-tile qs,
+        // in ONE basic block, so that the scheduler can interleave them (an MFMA runs for 32 cycles in the background
+        // of the VALU); with everything behind per-sub-tile branches the two kinds of work only ever alternated.
+        bool fast = i0 >= w_lo && i0 + kQStage <= w_hi && i0 + kQStage <= a.Lq && j0 >= a.j_lo && j0 + kWaveKeys <= a.j_hi;
+        if (a.mask == INFLLM_MASK_WINDOW)
+            fast = fast && (i0 - (j0 + kWaveKeys - 1) + a.offset >= 0) && (i0 + kQStage - 1 - j0 + a.offset < a.window);
+        if (a.mask == INFLLM_MASK_COMPLEMENT) fast = fast && (i0 - (j0 + kWaveKeys - 1) + a.offset >= a.window);
+        if (fast) {
+            constexpr int kSub = kQStage / 32;
+            f32x16 sacc[2][KS];
+            f32x4 l4[2][4];
+            auto issue = [&](int qs, int pb) {
+                bf16x8 qa[kD / 16];                              // A operand: lane = query row
+                const bf16_t *qrow = &Qs[cur][qs * 32 + col][grp * 8];
+#pragma unroll
+                for (int kk = 0; kk < kD / 16; ++kk) qa[kk] = *(const bf16x8 *)(qrow + kk * 16);
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) l4[pb][q4] = *(const f32x4 *)&Ls[cur][qs * 32 + 8 * q4 + 4 * grp];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sacc[pb][ks][r] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < kD / 16; ++kk)
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        sacc[pb][ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[kk], kreg[ks][kk], sacc[pb][ks], 0, 0, 0);
+            };
+            issue(0, 0);
+#pragma unroll
+            for (int qs = 0; qs < kSub; ++qs) {
+                const int pb = qs & 1;
+                if (qs + 1 < kSub) issue(qs + 1, pb ^ 1);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc += __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[pb][ks][r], scale, -l4[pb][r >> 2][r & 3]));
+                    colsum[ks] += acc;
+                }
+                if (qs + 1 < kSub) {
+                    // one MFMA, then its share of the exponentials (16 * KS of each per sub-tile)
+#pragma unroll
+                    for (int i = 0; i < 8 * KS; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);      // VALU
+                        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);      // transcendental
+                    }
+                }
+            }
+        } else
         if (i0 < w_hi && i0 + kQStage > w_lo) {                  // wave-uniform
 #pragma unroll
             for (int qs = 0; qs < kQStage / 32; ++qs) {
@@ -188,18 +241,21 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
                    "local_score: strides must be multiples of 8");
     if (a->j_hi <= a->j_lo) return 0;
     auto lds_bytes = [](int qs) { return (size_t)(2 * qs * kQPad * sizeof(bf16_t) + 2 * qs * sizeof(float)); };
+    static bool lds_set = false;                       // dynamic LDS above 64 KiB must be enabled once per kernel
+    if (!lds_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)local_score_kernel<1, 128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)lds_bytes(128));
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void *)local_score_kernel<2, 128>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds_bytes(128));
+        if (e != hipSuccess) return infllm_fail(-2, "local_score: %s", hipGetErrorString(e));
+        lds_set = true;
+    }
     if (a->j_hi - a->j_lo > 1024) {
         const int64_t tiles = (a->j_hi - 1) / 64 - a->j_lo / 64 + 1;
-        hipLaunchKernelGGL((local_score_kernel<2, 64>), dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), lds_bytes(64),
+        hipLaunchKernelGGL((local_score_kernel<2, 128>), dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), lds_bytes(128),
                            (hipStream_t)stream, *a);
     } else {
-        static bool lds_set = false;                   // dynamic LDS above 64 KiB must be enabled once
-        if (!lds_set) {
-            hipError_t e = hipFuncSetAttribute((const void *)local_score_kernel<1, 128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               (int)lds_bytes(128));
-            if (e != hipSuccess) return infllm_fail(-2, "local_score: %s", hipGetErrorString(e));
-            lds_set = true;
-        }
         const int64_t tiles = (a->j_hi - 1) / 32 - a->j_lo / 32 + 1;
         hipLaunchKernelGGL((local_score_kernel<1, 128>), dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), lds_bytes(128),
                            (hipStream_t)stream, *a);
