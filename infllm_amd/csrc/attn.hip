@@ -576,6 +576,86 @@ __global__ __launch_bounds__(256) void attn_merge_lse_kernel(const float *lse_pa
     lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
 }
 
+// The same two merges for few rows and many partials (decode-sized blocks: a handful of query rows, dozens of key
+// splits).  16 adjacent lanes share a row piece and take every 16th partial each, so all partials are one or two
+// round trips to memory instead of a chain; the lanes' sums are then joined by a fixed butterfly.
+__device__ __forceinline__ float group16_max(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float group16_sum(float v) {
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__global__ __launch_bounds__(256) void attn_merge_wide_kernel(const _Float16 *o_part, const float *lse_part, int P, int B, int H,
+                                                              int Lq, bf16_t *out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
+                                                              float *lse_out) {
+    const int64_t rows = (int64_t)B * H * Lq;
+    const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;       // (row, 8 dims)
+    const int pl = threadIdx.x & 15;
+    const int64_t row = e >> 4;
+    const int c = (int)(e & 15);
+    if (row >= rows) return;                                                 // whole 16-lane groups leave together
+    constexpr int kMine = 8;                                                 // partials per lane: P <= 128
+    float l[kMine];
+    f16x8 o[kMine];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kMine; ++i) {
+        const int p = pl + 16 * i;
+        const bool on = p < P;
+        l[i] = on ? lse_part[p * rows + row] : -INFINITY;
+        o[i] = on ? *(const f16x8 *)(o_part + (p * rows + row) * kD + c * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        m = fmaxf(m, l[i]);
+    }
+    m = group16_max(m);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, den = 0.f;
+    if (m > -INFINITY) {
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) {
+            const float w = __builtin_amdgcn_exp2f(l[i] - m);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] += (float)o[i][j] * w;
+            den += w;
+        }
+    }
+    den = group16_sum(den);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = group16_sum(acc[j]);
+    if (pl != 0) return;
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    const int i = (int)(row % Lq), h = (int)((row / Lq) % H), b = (int)(row / ((int64_t)Lq * H));
+    u32x4 packed{pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv),
+                 pack_bf16x2(acc[4] * inv, acc[5] * inv), pack_bf16x2(acc[6] * inv, acc[7] * inv)};
+    *(u32x4 *)(out + (int64_t)b * o_sb + (int64_t)h * o_sh + (int64_t)i * o_sl + c * 8) = packed;
+    if (c == 0 && lse_out) lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
+}
+
+__global__ __launch_bounds__(256) void attn_merge_lse_wide_kernel(const float *lse_part, int P, int64_t rows, float *lse_out) {
+    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+    const int pl = threadIdx.x & 15;
+    if (row >= rows) return;
+    constexpr int kMine = 8;
+    float l[kMine], m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kMine; ++i) {
+        const int p = pl + 16 * i;
+        l[i] = p < P ? lse_part[p * rows + row] : -INFINITY;
+        m = fmaxf(m, l[i]);
+    }
+    m = group16_max(m);
+    float den = 0.f;
+    if (m > -INFINITY) {
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) den += __builtin_amdgcn_exp2f(l[i] - m);
+    }
+    den = group16_sum(den);
+    if (pl == 0) lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
+}
+
 }  // namespace
 
 extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
@@ -657,17 +737,27 @@ extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_pa
     INFLLM_REQUIRE(d_o_part && d_lse_part, "attn_merge: null pointer");
     INFLLM_REQUIRE(P >= 1 && B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes P=%d B=%d H=%d Lq=%d", P, B, H, Lq);
     INFLLM_REQUIRE((o_sl % 8 | o_sh % 8 | o_sb % 8) == 0, "attn_merge: output strides must be multiples of 8");
+    // few rows, many partials (decode-sized blocks): 16 lanes per row piece, each taking every 16th partial
+    const bool wide = P > 8 && P <= 128 && (int64_t)B * H * Lq <= 2048;
     if (!d_out) {                                     // log-sum-exp only
         INFLLM_REQUIRE(d_lse, "attn_merge: neither output nor lse requested");
         const int64_t rows = (int64_t)B * H * Lq;
-        hipLaunchKernelGGL(attn_merge_lse_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d_lse_part, P,
-                           rows, d_lse);
+        if (wide)
+            hipLaunchKernelGGL(attn_merge_lse_wide_kernel, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                               d_lse_part, P, rows, d_lse);
+        else
+            hipLaunchKernelGGL(attn_merge_lse_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d_lse_part,
+                               P, rows, d_lse);
         INFLLM_CHECK_LAUNCH("attn_merge (lse)");
         return 0;
     }
     const int64_t threads = (int64_t)B * H * Lq * 16;
-    hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
+    if (wide)
+        hipLaunchKernelGGL(attn_merge_wide_kernel, dim3((unsigned)((threads * 16 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                           (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
+    else
+        hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                           (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
     INFLLM_CHECK_LAUNCH("attn_merge");
     return 0;
 }

@@ -249,6 +249,30 @@ def test_two_stage_joint_softmax_with_ring_and_pages():
     assert torch.allclose(score[:, :, rows].cpu(), 2 * want_ls, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("Lq,nsplit", [(1, 24), (3, 64), (5, 9)])
+def test_decode_shape_many_key_splits(Lq, nsplit):
+    """Few query rows and dozens of key splits (what a single-token step launches): the merge of that many
+    partials takes its own kernels; output and log-sum-exp against the oracle, lse-only merge against the full one."""
+    ops = _ops()
+    B, H, Hkv, Lk = 1, 8, 2, 64 * 70
+    q, k, v = _rand((B, H, Lq, D), 40), _rand((B, Hkv, Lk, D), 41), _rand((B, Hkv, Lk, D), 42)
+    want, _ = _oracle_two_stage(q, [(k, v, dict())])
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o_part = torch.empty((nsplit, B, H, Lq, D), dtype=torch.float16, device="cuda")
+    lse_part = torch.empty((nsplit, B, H, Lq), dtype=torch.float32, device="cuda")
+    ops.attn_stage_linear(qd, kd, vd, o_part, lse_part, j_lo=0, j_hi=Lk, nsplit=nsplit)
+    out = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda")
+    lse, lse_only = (torch.empty((B, H, Lq), dtype=torch.float32, device="cuda") for _ in range(2))
+    ops.attn_merge(o_part, lse_part, nsplit, out, lse)
+    _check_out(out, want)
+    logits = torch.einsum("bhqd,bhkd->bhqk", q.float(), k.float().repeat_interleave(H // Hkv, dim=1)) / math.sqrt(D)
+    assert torch.allclose(lse.cpu() * math.log(2.0), torch.logsumexp(logits, dim=-1), atol=2e-2)
+    from infllm_amd import _lib
+    _lib.check(_lib.load().infllm_attn_merge(o_part.data_ptr(), lse_part.data_ptr(), nsplit, B, H, Lq, None, 0, 0, 0,
+                                             lse_only.data_ptr(), torch.cuda.current_stream().cuda_stream), "infllm_attn_merge")
+    assert torch.allclose(lse_only, lse, atol=1e-5)
+
+
 def test_operator_class_protocol():
     from infllm_amd.attention.dot_production_attention import get_multi_stage_dot_production_attention
     Attn, flash = get_multi_stage_dot_production_attention(True)
