@@ -172,6 +172,9 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
+    # One HIP runtime (and one ROCr) per process: PyTorch bundles its own and every device pointer handed to the library
+    # comes from it, so it has to be the copy that is loaded first; the library's dependencies then resolve to it.
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise InfLLMHipError(
             f"{LIB_PATH} is missing: build it with `python -m infllm_amd.build` "
