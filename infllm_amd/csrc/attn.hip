@@ -179,10 +179,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     }
     if (g_t1 <= g_t0) g_t0 = g_t1 = 0;
     {
-        // share [n * split / nsplit, n * (split + 1) / nsplit) of the n tiles, in 32-bit pieces
+        // n / nsplit tiles each; the n % nsplit left over go one each to a run of splits in the middle: the first and
+        // the last split hold the tiles that need the mask (window start, causal diagonal) and take 1-2 us longer over
+        // the same number of tiles, so with the extras at the ends the whole launch waited for them
         const uint32_t n = (uint32_t)(g_t1 - g_t0), per = fdiv(n, geo.nsplit), rem = n - per * a.nsplit;
-        int t_begin = g_t0 + (int)(per * split + fdiv(rem * split, geo.nsplit));
-        int t_end = g_t0 + (int)(per * (split + 1) + fdiv(rem * (split + 1), geo.nsplit));
+        const int first_extra = (int)((a.nsplit - rem) >> 1);
+        const int before = min(max(split - first_extra, 0), (int)rem);            // extras given to lower splits
+        const int mine = (split >= first_extra && split < first_extra + (int)rem) ? 1 : 0;
+        int t_begin = g_t0 + (int)per * split + before;
+        int t_end = t_begin + (int)per + mine;
         g_t0 = t_begin;
         g_t1 = t_end;
     }
