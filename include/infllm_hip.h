@@ -175,9 +175,11 @@ typedef struct {
     int32_t mask;
     int32_t accumulate;            /* 1: add to d_score, 0: overwrite */
     int64_t offset, window;
-    const float *d_lse;            /* [B,H,Lq] from infllm_attn_merge */
+    const float *d_lse;            /* n_parts == 0: [B,H,Lq] from infllm_attn_merge;  n_parts > 0: the
+                                      partial log-sum-exps [n_parts,B,H,Lq] of infllm_attn_stage, joined on the
+                                      fly (saves the merge launch when nothing else needs the joint value yet) */
     float softmax_scale;
-    int32_t reserved;
+    int32_t n_parts;
     float *d_score;                /* fp32 [B,H,score_cap] */
     int64_t score_sb, score_sh, score_cap;
 } infllm_score_args;

@@ -55,7 +55,7 @@ class ScoreArgs(C.Structure):
         ("cap", c_i64), ("j_lo", c_i64), ("j_hi", c_i64),
         ("mask", c_i32), ("accumulate", c_i32),
         ("offset", c_i64), ("window", c_i64),
-        ("d_lse", c_vp), ("softmax_scale", c_f32), ("reserved", c_i32),
+        ("d_lse", c_vp), ("softmax_scale", c_f32), ("n_parts", c_i32),
         ("d_score", c_vp), ("score_sb", c_i64), ("score_sh", c_i64), ("score_cap", c_i64),
     ]
 

@@ -84,7 +84,30 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
             const int qi = i0 + ld_row + 16 * i;
             qbuf[i] = qi < a.Lq ? *(const u32x4 *)(qbase + (int64_t)qi * a.q_sl + ld_chunk * 8) : u32x4{0, 0, 0, 0};
         }
-        if (tid < kQStage) lbuf = i0 + tid < a.Lq ? lse[i0 + tid] : INFINITY;      // +inf => probability 0
+        if (tid < kQStage) {
+            if (i0 + tid >= a.Lq) {
+                lbuf = INFINITY;                                                  // +inf => probability 0
+            } else if (a.n_parts <= 0) {
+                lbuf = lse[i0 + tid];
+            } else {                                                              // join the stages' partial values here
+                const int64_t rows = (int64_t)a.B * a.H * a.Lq;
+                float m = -INFINITY, den = 0.f;
+                for (int p0 = 0; p0 < a.n_parts; p0 += 8) {
+                    float l8[8], m8 = -INFINITY;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) l8[i] = p0 + i < a.n_parts ? lse[(int64_t)(p0 + i) * rows + i0 + tid] : -INFINITY;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) m8 = fmaxf(m8, l8[i]);
+                    if (m8 == -INFINITY) continue;
+                    const float m_new = fmaxf(m, m8);
+                    den *= __builtin_amdgcn_exp2f(m - m_new);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) den += __builtin_amdgcn_exp2f(l8[i] - m_new);
+                    m = m_new;
+                }
+                lbuf = den > 0.f ? m + log2f(den) : INFINITY;
+            }
+        }
     };
     auto store_stage = [&](int buf) {
 #pragma unroll
@@ -237,6 +260,7 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
     INFLLM_REQUIRE(a->j_hi - a->j_lo <= a->cap && a->j_hi - a->j_lo <= a->score_cap,
                    "local_score: key range [%lld,%lld) exceeds the ring", (long long)a->j_lo, (long long)a->j_hi);
     INFLLM_REQUIRE(a->mask >= 0 && a->mask <= 2, "local_score: unknown mask %d", a->mask);
+    INFLLM_REQUIRE(a->n_parts >= 0 && a->n_parts <= 1024, "local_score: %d partial log-sum-exps", a->n_parts);
     INFLLM_REQUIRE((a->q_sl % 8 | a->q_sh % 8 | a->q_sb % 8 | a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8) == 0,
                    "local_score: strides must be multiples of 8");
     if (a->j_hi <= a->j_lo) return 0;

@@ -547,7 +547,8 @@ int run_topk_merge(Layer *L, const float *scores, int64_t scores_sb, int n_old, 
     return 0;
 }
 
-int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t j_hi, void *stream) {
+// n_parts > 0: the stages' partial log-sum-exps are joined inside the launch (d_lse is not ready yet)
+int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t j_hi, int n_parts, void *stream) {
     const infllm_layer_desc &d = L->d;
     if (j_hi <= j_lo) return 0;
     infllm_score_args sc{};
@@ -558,7 +559,7 @@ int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t
     sc.k_sl = kD; sc.k_sh = d.ring_cap * kD; sc.k_sb = (int64_t)d.Hkv * d.ring_cap * kD;
     sc.cap = d.ring_cap; sc.j_lo = j_lo; sc.j_hi = j_hi;
     sc.mask = INFLLM_MASK_WINDOW; sc.accumulate = 1; sc.offset = b0; sc.window = d.n_local;
-    sc.d_lse = d.d_lse; sc.softmax_scale = d.softmax_scale;
+    sc.d_lse = n_parts > 0 ? d.d_lse_part : d.d_lse; sc.n_parts = n_parts; sc.softmax_scale = d.softmax_scale;
     sc.d_score = d.d_ring_score; sc.score_sh = d.ring_cap; sc.score_sb = (int64_t)d.H * d.ring_cap; sc.score_cap = d.ring_cap;
     return infllm_local_score(&sc, stream);
 }
@@ -860,10 +861,14 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         }
         parts += at.nsplit;
     }
-    // only the joint log-sum-exp is needed by what follows on the way to the next selection; the output rows are
-    // merged once that selection is out (step 5b)
-    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, nullptr, 0, 0, 0, d.d_lse, stream);
-    if (rc) return rc;
+    // Only the joint log-sum-exp is needed on the way to the next selection, and only by the small score launch of
+    // step 4, which joins the partial values itself; the merge (output rows and the joint value for the bulk of the
+    // scores) runs once that selection is out (step 5b).  The score-decay policy needs the joint value here.
+    const bool lse_now = a->d_unit_mass && a->n_sel > 0;
+    if (lse_now) {
+        rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, nullptr, 0, 0, 0, d.d_lse, stream);
+        if (rc) return rc;
+    }
 
     // ---- 3b. attention mass each selected unit received (only the score-decay policy asks for it)
     if (a->d_unit_mass && a->n_sel > 0) {
@@ -894,7 +899,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     //         init peeling, representatives of the new units
     const int64_t new_cursor = a->cursor + a->init_take + (int64_t)a->n_carve * bs;
     const int64_t urgent_hi = new_cursor < b1 ? new_cursor : b1;
-    rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, stream);
+    rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, lse_now ? 0 : parts, stream);
     if (rc) return rc;
     int64_t cursor = a->cursor;
     if (a->init_take > 0) {
@@ -930,10 +935,11 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     }
     L->cand_units = -1;
     // ---- 5b. the block's output rows
-    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, nullptr, stream);
+    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl,
+                           lse_now ? nullptr : d.d_lse, stream);
     if (rc) return rc;
     // ---- 6. off the critical path: the rest of the local score, new units to pinned host memory
-    rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, stream);
+    rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, 0, stream);
     if (rc) return rc;
     if (a->n_carve > 0) {
         if (L->off.pending) {
