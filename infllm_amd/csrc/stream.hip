@@ -51,6 +51,7 @@ struct Layer {
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
     int32_t topk_seq = 0;
+    hipStream_t topk_stream = nullptr;    // stream of the last selection (to fall back on when the poll gives up)
     // the top-k of the units that existed when the next block was prepared, chosen ahead of the chain: [B,topk]
     // device ids (this handle's own allocation) and the unit count they were chosen from (-1: none)
     int32_t *d_cand = nullptr;
@@ -523,7 +524,10 @@ int run_topk(Layer *L, const float *scores, int64_t scores_sb, int n_units, void
     }
     if (d.h_topk_idx)      // NULL: d_topk_idx is itself host-visible pinned memory, the kernel wrote there
         HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
-    HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    // an event record costs the stream 2-3 us; with the polled sequence number it would only back up the rare case
+    // in which the poll gives up, and a stream synchronisation does that as well
+    if (!poll) HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    L->topk_stream = st;
     L->topk_pending = true;
     return 0;
 }
@@ -542,7 +546,8 @@ int run_topk_merge(Layer *L, const float *scores, int64_t scores_sb, int n_old, 
     }
     if (d.h_topk_idx)
         HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
-    HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    if (!poll) HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    L->topk_stream = st;
     L->topk_pending = true;
     return 0;
 }
@@ -661,6 +666,9 @@ extern "C" int infllm_layer_wait_topk(void *layer) {
             L->topk_pending = false;
             return 0;
         }
+        HIP_OK(hipStreamSynchronize(L->topk_stream), "layer_wait_topk");        // no event was recorded in this mode
+        L->topk_pending = false;
+        return 0;
     }
     HIP_OK(hipEventSynchronize(L->topk_done), "layer_wait_topk");
     L->topk_pending = false;
