@@ -79,7 +79,7 @@ def run_stream(q, k, v, chunk, timing=False):
 # HBM bytes per launch from hardware counters (FETCH_SIZE, WRITE_SIZE; one profiler run per counter, each scaled by
 # what the counter reads for a 256 MiB elementwise pass: x2.0 and x1.0).  The summaries of those runs sit in
 # profiles/*.hbm_bytes.txt; the figures hold for the default geometry only.
-LOCAL_STAGE_HBM_BYTES = int((20242.0 * 2.0 + 16640.0) * 1024)      # steady-state local stage: 39.5 MiB read + 16.25 MiB written (fp16 partials)
+LOCAL_STAGE_HBM_BYTES = int((20241.0 * 2.0 + 16640.0) * 1024)      # steady-state local stage: 39.5 MiB read + 16.25 MiB written (fp16 partials)
 UNIT_SCORES_HBM_BYTES = int((32860.6 * 2.0 + 64.0) * 1024)         # 8194 x 4096 representatives: 64.2 MiB read
 
 
