@@ -268,7 +268,8 @@ void *infllm_host_device_pointer(void *h_pinned);
  *                        local score and the gather of the new units into a staging slot.
  *
  * The chain from one block's ids to the next block's ids is therefore: fetch, global stage,
- * merge, a small score launch, representatives, a small score launch, top-k.
+ * a small local-score launch (which joins the stages' log-sum-exps itself), representatives, a
+ * small unit-score launch, the final ranking; the merge runs behind it.
  *
  * The copy of newly carved units from the staging slot to pinned host memory is deferred and
  * ordered by the host: once the gather's event has fired (checked at the next block's calls) it
