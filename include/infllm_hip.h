@@ -394,6 +394,12 @@ int infllm_cache_touch(void *cache, const int32_t *selected, int32_t n_sel, int3
 int infllm_cache_add_scores(void *cache, const int32_t *units, const double *scores, int32_t n);
 /* residents in insertion order (any output may be NULL); returns their number */
 int infllm_cache_residents(void *cache, int32_t *units, double *values, int32_t *slots, int32_t capacity);
+/* the slot of a resident unit, -1 when it is not resident */
+int infllm_cache_slot_of(void *cache, int32_t unit);
+/* a second policy object in the same state / bring dst (same capacity and strategy) into the state of src:
+ * what a caller needs to try a selection out before it is final (see infllm_block_prefetch) */
+void *infllm_cache_clone(const void *src);
+int infllm_cache_copy(void *dst, const void *src);
 
 /* Selection -> policy -> fetch in one native call (replaces a host loop between infllm_layer_wait_topk and
  * infllm_block_fetch): runs infllm_cache_touch for every batch row, fills the lists infllm_block_back takes and
@@ -415,6 +421,25 @@ typedef struct {
     int32_t *h_n_evicted, *h_n_miss;                  /* out, optional: [B] */
 } infllm_select_args;
 int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, void *copy_stream);
+
+/* The fetch ahead of the selection.  infllm_block_front ranks the units that exist before its block for the NEXT
+ * block already (the selection proper, late in infllm_block_back, only weighs these candidates against the units
+ * carved in between) and publishes them to the host.  Called after infllm_block_back, this runs the residency
+ * policy for the candidates on a copy of the policy objects and starts the fetch of their misses, a block's length
+ * before the selection is final, so that the transfer is no longer part of the chain selection -> fetch -> global
+ * stage -> next selection.  The next infllm_block_select settles it: when the selection equals the candidates
+ * (all but the blocks in which a freshly carved unit makes the top-k) the copy becomes the policy state, the lists
+ * and the return value are what the call would have produced, and nothing is left to fetch; otherwise the copy is
+ * dropped, the call proceeds from the untouched state, and the residents whose slots the guess overwrote are
+ * fetched again with the misses.  The hit / miss / eviction sequence is therefore the reference's either way.
+ * No guess is made (return 0) when no candidates are pending, or when the policy would evict a unit of the
+ * selection whose global stage may still be running.  Valid only for policies whose state does not change between
+ * this call and the selection (lru, fifo: the lru-s scores arrive with the block's attention mass).
+ * `a` as for infllm_block_select (h_selected, wait_topk and the output lists are not used).  Returns the number of
+ * units whose fetch was started (>= 0) or an error (< 0).  A guess still open at infllm_layer_flush is undone there. */
+int infllm_block_prefetch(void *layer, const infllm_select_args *a, void *stream, void *copy_stream);
+/* how many guesses were made / turned out to be the selection */
+int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed);
 
 /* Event timing of the two attention stages (for benchmarks): enable with a record
  * capacity and a stride (every stride-th launch of each stage is bracketed by two events; an event pair

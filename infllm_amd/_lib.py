@@ -155,7 +155,12 @@ SYMBOLS = {
     "infllm_cache_touch": (c_i32, [c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "infllm_cache_add_scores": (c_i32, [c_vp, c_vp, c_vp, c_i32]),
     "infllm_cache_residents": (c_i32, [c_vp, c_vp, c_vp, c_vp, c_i32]),
+    "infllm_cache_slot_of": (c_i32, [c_vp, c_i32]),
+    "infllm_cache_clone": (c_vp, [c_vp]),
+    "infllm_cache_copy": (c_i32, [c_vp, c_vp]),
     "infllm_block_select": (c_i32, [c_vp, C.POINTER(SelectArgs), c_vp, c_vp]),
+    "infllm_block_prefetch": (c_i32, [c_vp, C.POINTER(SelectArgs), c_vp, c_vp]),
+    "infllm_layer_prefetch_stats": (c_i32, [c_vp, c_vp, c_vp]),
     "infllm_layer_timing": (c_i32, [c_vp, c_i32, c_i32]),
     "infllm_layer_read_timing": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32]),
 }

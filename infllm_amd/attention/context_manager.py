@@ -113,6 +113,7 @@ class CachePolicy:
 
 class ContextManager:
     select_in_steps = False     # True: drive wait / policy / fetch from here (slower), instead of infllm_block_select
+    fetch_ahead = True          # start the next block's fetch from its candidates (infllm_block_prefetch)
 
     def __init__(self, position_embedding, n_init, n_local, block_size, max_cached_block, topk, exc_block_size,
                  score_decay=None, fattn=False, repr_topk=1, cache_strategy="lru", chunk_topk_calc=None,
@@ -420,6 +421,11 @@ class ContextManager:
         rc = lib.infllm_block_back(layer, self._ba_ref, self._main_raw, self._copy_raw)
         if rc:
             check(rc, "infllm_block_back")
+        if n_next and preselected is None and self.fetch_ahead and not self.select_in_steps and self.cache_strategy != "lru-s":
+            sa.n_sel = topk
+            rc = lib.infllm_block_prefetch(layer, self._sa_ref, self._main_raw, self._copy_raw)
+            if rc < 0:
+                check(rc, "infllm_block_prefetch")
         if self.cache_strategy == "lru-s" and n_sel:
             self._mass_units = selected
         if self.record_trace:

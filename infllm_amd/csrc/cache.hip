@@ -143,3 +143,29 @@ extern "C" int infllm_cache_residents(void *cache, int32_t *units, double *value
     }
     return n;
 }
+
+extern "C" void *infllm_cache_clone(const void *src) {
+    if (!src) {
+        infllm_fail(-1, "cache_clone: null cache");
+        return nullptr;
+    }
+    return new UnitCache(*(const UnitCache *)src);
+}
+
+extern "C" int infllm_cache_copy(void *dst, const void *src) {
+    INFLLM_REQUIRE(dst && src, "cache_copy: null cache");
+    UnitCache &d = *(UnitCache *)dst;
+    const UnitCache &s = *(const UnitCache *)src;
+    INFLLM_REQUIRE(d.capacity == s.capacity && d.strategy == s.strategy, "cache_copy: caches of different capacity or strategy");
+    d.decay = s.decay;
+    d.clock = s.clock;
+    d.res = s.res;
+    d.free_slots = s.free_slots;
+    return 0;
+}
+
+extern "C" int infllm_cache_slot_of(void *cache, int32_t unit) {
+    if (!cache) return -1;
+    Resident *r = ((UnitCache *)cache)->find(unit);
+    return r ? r->slot : -1;
+}

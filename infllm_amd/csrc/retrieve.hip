@@ -144,6 +144,12 @@ __device__ int block_exclusive_scan(int v, int *wave_tot, int *total) {
 // Both selection kernels can end by publishing a sequence number next to the ids (flag may be NULL): every
 // thread fences its id stores to system scope, the workgroup meets, then one thread stores the number.  A host
 // that polls the (pinned) flag sees the ids no later than the number.
+// ids go to one place or two (the second, when given, is a host-visible copy of a device-side list)
+__device__ __forceinline__ void put_id(int32_t *a, int32_t *b, int pos, int32_t v) {
+    a[pos] = v;
+    if (b) b[pos] = v;
+}
+
 __device__ __forceinline__ void publish(int32_t *flag, int32_t value) {
     if (!flag) return;
     __threadfence_system();
@@ -151,8 +157,8 @@ __device__ __forceinline__ void publish(int32_t *flag, int32_t value) {
     if (threadIdx.x == 0) __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-__global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *flag,
-                                                           int32_t flag_value) {
+__global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *idx_out2,
+                                                           int32_t *flag, int32_t flag_value) {
     __shared__ int hist[256];
     __shared__ int wave_tot[kSelThreads / 64];
     __shared__ uint32_t sh_prefix;
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
         const int eq_rank = eq_base + block_exclusive_scan(is_eq, wave_tot, &tot_eq);
         const int sel = (n < N && (key > prefix || (is_eq && eq_rank < need))) ? 1 : 0;
         const int pos = out_base + block_exclusive_scan(sel, wave_tot, &tot_sel);
-        if (sel && pos < k) idx_out[pos] = n;
+        if (sel && pos < k) put_id(idx_out, idx_out2, pos, n);
         eq_base += tot_eq;
         out_base += tot_sel;
     }
@@ -208,8 +214,8 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
 // many LDS counters) find the key of the k-th largest; a pass whose bucket is wanted whole ends the search.
 // Output contract as above: indices ascending, lowest indices among keys equal to the k-th.
 template <int R>
-__global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *flag,
-                                                                int32_t flag_value) {
+__global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *idx_out2,
+                                                                int32_t *flag, int32_t flag_value) {
     __shared__ __align__(16) int hist[4096];
     __shared__ int wave_tot[kSelThreads / 64];
     __shared__ uint32_t sh_prefix;
@@ -288,10 +294,10 @@ __global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *sco
         if (j >= n_valid) break;
         const uint32_t mk = key[j] & pmask;
         if (mk > prefix) {
-            idx_out[g_before + min(e_before, need)] = tid * R + j;
+            put_id(idx_out, idx_out2, g_before + min(e_before, need), tid * R + j);
             ++g_before;
         } else if (mk == prefix) {
-            if (e_before < need) idx_out[g_before + e_before] = tid * R + j;
+            if (e_before < need) put_id(idx_out, idx_out2, g_before + e_before, tid * R + j);
             ++e_before;
         }
     }
@@ -395,19 +401,26 @@ extern "C" int infllm_unit_scores(const void *d_reps, int64_t rep_stride, int32_
     return 0;
 }
 
-int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag,
+                             int32_t flag_value, void *stream);
 
 extern "C" int infllm_topk(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, void *stream) {
-    return infllm_topk_publish(d_scores, N, k, d_idx, nullptr, 0, stream);
+    return infllm_topk_publish_pair(d_scores, N, k, d_idx, nullptr, nullptr, 0, stream);
 }
 
 // library-internal: the selection followed by `*d_flag = flag_value` (system scope) once the ids are written
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream) {
+    return infllm_topk_publish_pair(d_scores, N, k, d_idx, nullptr, d_flag, flag_value, stream);
+}
+
+// ... with a second copy of the ids in d_idx2 (may be NULL)
+int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag,
+                             int32_t flag_value, void *stream) {
     INFLLM_REQUIRE(d_scores && d_idx, "topk: null pointer");
     INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && k <= 1024, "topk: k=%d with N=%d", k, N);
     const hipStream_t st = (hipStream_t)stream;
     switch (N <= 16384 ? (N + kSelThreads - 1) / kSelThreads : 0) {       // keys per thread
-#define REGS_CASE(r) hipLaunchKernelGGL(topk_regs_kernel<r>, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_flag, flag_value); break
+#define REGS_CASE(r) hipLaunchKernelGGL(topk_regs_kernel<r>, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_idx2, d_flag, flag_value); break
     case 1: REGS_CASE(1);
     case 2: REGS_CASE(2);
     case 3: REGS_CASE(3);
@@ -418,7 +431,7 @@ int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_
     case 11: case 12: REGS_CASE(12);
     case 13: case 14: case 15: case 16: REGS_CASE(16);
 #undef REGS_CASE
-    default: hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_flag, flag_value);
+    default: hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_idx2, d_flag, flag_value);
     }
     INFLLM_CHECK_LAUNCH("topk");
     return 0;

@@ -5,6 +5,7 @@
 #include <atomic>
 #include <chrono>
 #include <cstdlib>
+#include <cstring>
 #include <vector>
 
 #include <hsa/hsa.h>
@@ -47,6 +48,34 @@ struct Layer {
     std::vector<hsa_signal_t> dma_sig;
     std::vector<char> dma_busy;
     std::vector<int> dma_first, dma_count;
+    // The fetch of missed units through several DMA engines (see fetch_by_engines): engines, the signal the unit
+    // copies count down, a 4-byte flag in signal memory that the main stream waits on and the engines write last,
+    // its pinned source values, and the sequence number of the fetch in flight.
+    bool efetch_ok = false;
+    std::vector<uint32_t> efetch_engines;
+    hsa_signal_t efetch_sig{}, efetch_flag_sig{};
+    uint32_t *d_efetch_flag = nullptr, *h_efetch_val = nullptr;
+    uint32_t efetch_seq = 0;
+    bool efetch_wait = false;
+    // The fetch ahead of the selection (see infllm_block_prefetch): the candidates' host copy with the sequence number
+    // the kernel publishes behind them, the selection whose global stage may still be running, and the guess in flight.
+    int32_t *h_cand = nullptr;                         // pinned [B*topk + 1]
+    int32_t cand_seq = 0;
+    int cand_for_units = -1;                           // unit count the published candidates were chosen from, -1: none
+    std::vector<int32_t> last_sel;                     // [B, last_n_sel]
+    int last_n_sel = 0;
+    struct Ahead {
+        bool active = false;
+        int n_sel = 0, n_miss_all = 0;
+        std::vector<void *> shadow;                    // [B] policy state after the guessed selection
+        std::vector<int32_t> cand, sel_slots;          // [B, n_sel]
+        std::vector<int32_t> miss_row, miss_slot, miss_unit;
+        std::vector<const void *> miss_src;
+        std::vector<int32_t> evicted, n_evicted, n_miss;             // [B, n_sel], [B], [B]
+        std::vector<int32_t> victim_row, victim_unit, victim_slot;   // residents whose slots the guess overwrote
+        std::vector<const void *> victim_src;
+    } ahead;
+    int64_t ahead_issued = 0, ahead_confirmed = 0;
     int page_cur = 0, carve_cur = 0;
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
@@ -90,6 +119,8 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag,
+                             int32_t flag_value, void *stream);
 int infllm_gather_rows_pair(const void *d_ring_a, void *d_out_a, const void *d_ring_b, void *d_out_b, int64_t ring_cap, int32_t B,
                             int32_t Hkv, int64_t t0, int32_t n, int32_t unit_rows, int64_t out_sb, int64_t out_su, int64_t out_sh,
                             void *stream);
@@ -299,22 +330,132 @@ int issue_offload(Layer *L, hipStream_t cs) {
     return 0;
 }
 
+// ---- the fetch of missed units through the DMA engines
+// A kernel that reads pinned memory keeps thousands of PCIe reads outstanding in the L2, and everything else on the
+// chip runs 1.5-2x longer beside it.  The SDMA engines do not go through the shader caches: 8 of them together move
+// a block's misses as fast as the kernel does (a single engine reaches half of that on 512 KiB pieces), and the
+// kernels beside them run at their own speed.  Ordering: the host issues the copies (it has just seen the selection,
+// so the previous global stage, the last reader of the slots, has finished - otherwise it waits for that event
+// here), and the last thing the engines write is a sequence number into a flag in signal memory, on which the main
+// stream waits (hipStreamWaitValue32) before the global stage.
+constexpr int kEfetchEngines = 8;
+constexpr int kEfetchVals = 8;
+
+int efetch_wait_signal(hsa_signal_t sig, const char *what) {
+    const auto t0 = std::chrono::steady_clock::now();
+    while (hsa_signal_load_scacquire(sig) > 0) {
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(10)) return infllm_fail(-2, "%s: DMA engine copies did not complete within 10 s", what);
+    }
+    return 0;
+}
+
+// set the engine fetch up for this layer; on any failure the kernel fetch stays the only path
+void efetch_setup(Layer *L) {
+    const char *off = getenv("INFLLM_NO_DMA_FETCH");
+    if (!L->dma_ok || (off && off[0] && off[0] != '0')) return;
+    int dev = 0, can = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&can, hipDeviceAttributeCanUseStreamWaitValue, dev) != hipSuccess || !can) {
+        (void)hipGetLastError();
+        return;
+    }
+    uint32_t mask = 0;
+    if (hsa_amd_memory_copy_engine_status(L->dma_gpu, L->dma_cpu, &mask) != HSA_STATUS_SUCCESS) return;
+    for (int b = 0; b < 32 && (int)L->efetch_engines.size() < kEfetchEngines; ++b)
+        if (mask & (1u << b)) L->efetch_engines.push_back(1u << b);
+    if (L->efetch_engines.size() < 2) return;
+    if (hipExtMallocWithFlags((void **)&L->d_efetch_flag, 8, hipMallocSignalMemory) != hipSuccess ||
+        hipMemset(L->d_efetch_flag, 0, 8) != hipSuccess || hipHostMalloc((void **)&L->h_efetch_val, kEfetchVals * sizeof(uint32_t)) != hipSuccess ||
+        hsa_signal_create(0, 0, nullptr, &L->efetch_sig) != HSA_STATUS_SUCCESS ||
+        hsa_signal_create(0, 0, nullptr, &L->efetch_flag_sig) != HSA_STATUS_SUCCESS) {
+        (void)hipGetLastError();
+        return;
+    }
+    // the first copy on an engine creates its queue (milliseconds): do that here, once per process and engine
+    for (int i = 0; i < kEfetchVals; ++i) L->h_efetch_val[i] = 0;
+    hsa_signal_store_relaxed(L->efetch_sig, (hsa_signal_value_t)L->efetch_engines.size());
+    int issued = 0;
+    for (uint32_t e : L->efetch_engines) {
+        if (hsa_amd_memory_async_copy_on_engine(L->d_efetch_flag, L->dma_gpu, L->h_efetch_val, L->dma_cpu, 4, 0, nullptr, L->efetch_sig,
+                                                (hsa_amd_sdma_engine_id_t)e, false) != HSA_STATUS_SUCCESS)
+            break;
+        ++issued;
+    }
+    hsa_signal_subtract_relaxed(L->efetch_sig, (hsa_signal_value_t)(L->efetch_engines.size() - issued));
+    if (efetch_wait_signal(L->efetch_sig, "layer_create") != 0 || issued != (int)L->efetch_engines.size()) return;
+    L->efetch_ok = true;
+}
+
+// Returns 1 when the engines took the fetch, 0 when the caller should use the kernel, < 0 on error.
+int fetch_by_engines(Layer *L, int n_miss, const void *const *srcs, int64_t nbytes, bool ahead) {
+    if (!L->efetch_ok || !L->dma_ok) return 0;          // stream-ordered offloads are not ordered before the engines
+    for (size_t s = 0; s < L->carve_busy.size(); ++s) {  // ... and the few that were issued (layer_flush) have to land first
+        if (!L->carve_busy[s]) continue;
+        HIP_OK(hipEventSynchronize(L->carve_evt[s]), "fetch: wait offload");
+        L->carve_busy[s] = 0;
+    }
+    // slots may still be read by the previous global stage unless the host has seen a later result of the stream
+    // (a fetch ahead writes no slot of the selection in use, and the stage before that has finished)
+    if (!ahead && L->has_global && hipEventQuery(L->global_done) != hipSuccess) {
+        (void)hipGetLastError();
+        HIP_OK(hipEventSynchronize(L->global_done), "fetch: wait global");
+    }
+    int rc = efetch_wait_signal(L->efetch_flag_sig, "fetch");             // the previous fetch's flag copy (long done)
+    if (rc) return rc;
+    const uint32_t seq = ++L->efetch_seq;
+    uint32_t *val = L->h_efetch_val + (seq % kEfetchVals);
+    *val = seq;
+    hsa_signal_store_relaxed(L->efetch_sig, n_miss);
+    hsa_signal_store_relaxed(L->efetch_flag_sig, 1);
+    int issued = 0;
+    bool ok = true;
+    for (int i = 0; i < n_miss && ok; ++i) {
+        ok = hsa_amd_memory_async_copy_on_engine(L->fetch_dst[i], L->dma_gpu, srcs[i], L->dma_cpu, (size_t)nbytes, 0, nullptr, L->efetch_sig,
+                                                 (hsa_amd_sdma_engine_id_t)L->efetch_engines[i % L->efetch_engines.size()], false) ==
+             HSA_STATUS_SUCCESS;
+        issued += ok ? 1 : 0;
+    }
+    if (ok)
+        ok = hsa_amd_memory_async_copy_on_engine(L->d_efetch_flag, L->dma_gpu, val, L->dma_cpu, 4, 1, &L->efetch_sig, L->efetch_flag_sig,
+                                                 (hsa_amd_sdma_engine_id_t)L->efetch_engines[0], false) == HSA_STATUS_SUCCESS;
+    if (!ok) {
+        // give the engine path up: let what was issued land, then the kernel copies everything again
+        hsa_signal_subtract_relaxed(L->efetch_sig, n_miss - issued);
+        hsa_signal_store_relaxed(L->efetch_flag_sig, 0);
+        rc = efetch_wait_signal(L->efetch_sig, "fetch");
+        L->efetch_ok = false;
+        --L->efetch_seq;
+        return rc;
+    }
+    L->efetch_wait = true;
+    return 1;
+}
+
 // missed units -> their slab slots on the copy stream; then the pending offload (never ahead of a fetch
 // unless the fetch needs one of the units that are still on their way to the host)
 int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, const int32_t *units, const void *const *srcs,
-             hipStream_t st, hipStream_t cs) {
+             hipStream_t st, hipStream_t cs, bool ahead = false) {
     const infllm_layer_desc &d = L->d;
     const bool side = cs != st;
     const int64_t slot_elems = 2 * (int64_t)d.Hkv * d.block_size * kD;
     if (n_miss > 0) {
         INFLLM_REQUIRE(rows && slots && units && srcs, "fetch: null miss list");
-        if (side && L->has_global) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "fetch: wait global");
         if (L->off.pending) {
             bool hit = false;
             for (int i = 0; i < n_miss && !hit; ++i) hit = units[i] >= L->off.first_unit && units[i] < L->off.first_unit + L->off.count;
             if (hit) {
-                int orc = issue_offload(L, cs);
-                if (orc) return orc;
+                // the DMA engines that fetch are not ordered behind `cs`: there, the units go out by the engine too
+                // (waited for just below), or the host waits for the stream copy
+                int orc = 0;
+                if (L->efetch_ok && L->dma_ok) {
+                    HIP_OK(hipEventSynchronize(L->carve_ready), "fetch: wait gathers");
+                    orc = issue_offload_dma(L);
+                    if (orc < 0) return orc;
+                }
+                if (L->off.pending) {
+                    orc = issue_offload(L, cs);
+                    if (orc) return orc;
+                    if (L->efetch_ok) HIP_OK(hipStreamSynchronize(cs), "fetch: wait offload");
+                }
             }
         }
         for (size_t s = 0; s < L->dma_busy.size(); ++s) {           // units still on their way to the host by the engine
@@ -331,11 +472,16 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
             INFLLM_REQUIRE(rows[i] >= 0 && rows[i] < d.B && slots[i] >= 0 && slots[i] < d.max_cached && srcs[i], "fetch: bad miss entry");
             L->fetch_dst[i] = (bf16_t *)d.d_slab + ((int64_t)rows[i] * d.max_cached + slots[i]) * slot_elems;
         }
-        int frc = infllm_fetch_units(srcs, L->fetch_dst.data(), n_miss, slot_elems * (int64_t)sizeof(bf16_t), cs);
-        if (frc) return frc;
-        if (side) {
-            HIP_OK(hipEventRecord(L->fetch_done, cs), "fetch: event");
-            L->fetch_wait = true;
+        const int erc = fetch_by_engines(L, n_miss, srcs, slot_elems * (int64_t)sizeof(bf16_t), ahead);
+        if (erc < 0) return erc;
+        if (erc == 0) {
+            if (side && L->has_global && !ahead) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "fetch: wait global");
+            int frc = infllm_fetch_units(srcs, L->fetch_dst.data(), n_miss, slot_elems * (int64_t)sizeof(bf16_t), cs);
+            if (frc) return frc;
+            if (side) {
+                HIP_OK(hipEventRecord(L->fetch_done, cs), "fetch: event");
+                L->fetch_wait = true;
+            }
         }
     }
     if (L->off.pending) {
@@ -415,6 +561,12 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
             else L->dma_ok = false;                 // without signals the stream-ordered copy is used
         }
     }
+    efetch_setup(L);
+    if (hipHostMalloc((void **)&L->h_cand, ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
+        (void)hipGetLastError();
+        L->h_cand = nullptr;                        // no fetch ahead of the selection then
+    } else
+        std::memset(L->h_cand, 0, ((size_t)d.B * d.topk + 1) * sizeof(int32_t));
     return L;
 }
 
@@ -435,6 +587,19 @@ extern "C" int infllm_layer_destroy(void *layer) {
         for (hipEvent_t e : t.ev)
             if (e) (void)hipEventDestroy(e);
     if (L->d_cand) (void)hipFree(L->d_cand);
+    if (L->h_cand) (void)hipHostFree(L->h_cand);
+    for (void *c : L->ahead.shadow)
+        if (c) (void)infllm_cache_destroy(c);
+    if (L->efetch_sig.handle) {
+        (void)efetch_wait_signal(L->efetch_sig, "layer_destroy");
+        (void)hsa_signal_destroy(L->efetch_sig);
+    }
+    if (L->efetch_flag_sig.handle) {
+        (void)efetch_wait_signal(L->efetch_flag_sig, "layer_destroy");
+        (void)hsa_signal_destroy(L->efetch_flag_sig);
+    }
+    if (L->d_efetch_flag) (void)hipFree(L->d_efetch_flag);
+    if (L->h_efetch_val) (void)hipHostFree(L->h_efetch_val);
     delete L;
     return 0;
 }
@@ -598,6 +763,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     }
     L->prepared = false;
     L->cur_slot = L->slot;
+    L->cand_for_units = -1;
 
     // ---- local stage: causal sliding window over the ring
     const int64_t b1 = a->b0 + a->n;
@@ -633,12 +799,16 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
             // against the few units carved in between, instead of running over every unit on the chain
             L->cand_units = -1;
             if (L->d_cand && a->n_units > d.topk) {
+                // the host gets a copy, with a sequence number behind the last row's: it may fetch them ahead
+                if (L->h_cand) ++L->cand_seq;
                 for (int u = 0; u < d.B; ++u) {
-                    rc = infllm_topk_publish(a->d_unit_scores + (int64_t)u * a->unit_scores_sb, a->n_units, d.topk,
-                                             L->d_cand + (int64_t)u * d.topk, nullptr, 0, stream);
+                    rc = infllm_topk_publish_pair(a->d_unit_scores + (int64_t)u * a->unit_scores_sb, a->n_units, d.topk,
+                                                  L->d_cand + (int64_t)u * d.topk, L->h_cand ? L->h_cand + (int64_t)u * d.topk : nullptr,
+                                                  L->h_cand && u == d.B - 1 ? L->h_cand + (int64_t)d.B * d.topk : nullptr, L->cand_seq, stream);
                     if (rc) return rc;
                 }
                 L->cand_units = a->n_units;
+                L->cand_for_units = L->h_cand ? a->n_units : -1;
             }
         }
         L->prepared = true;
@@ -694,6 +864,116 @@ extern "C" int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_
     return rc;
 }
 
+namespace {
+
+const void *host_unit(const infllm_select_args *a, int unit, int row) {
+    const int chunk = unit / a->units_per_chunk, idx = unit % a->units_per_chunk;
+    if (chunk >= a->n_chunks || !a->h_chunk_base[chunk]) return nullptr;
+    return (const void *)(uintptr_t)(a->h_chunk_base[chunk] + (uint64_t)idx * a->unit_bytes + (uint64_t)row * a->row_bytes);
+}
+
+// A guess that is not confirmed leaves residents behind whose slots it overwrote: they are fetched again (those
+// that are still resident, in the slot they had; all of them when no policy objects are given, i.e. when the policy
+// has not moved since the guess).  `extra` lists misses to fetch in the same go.
+int ahead_repair(Layer *L, void *const *caches, int n_extra, const int32_t *rows, const int32_t *slots, const int32_t *units,
+                 const void *const *srcs, hipStream_t st, hipStream_t cs) {
+    Layer::Ahead &g = L->ahead;
+    std::vector<int32_t> r(rows, rows + n_extra), sl(slots, slots + n_extra), un(units, units + n_extra);
+    std::vector<const void *> sr(srcs, srcs + n_extra);
+    for (size_t i = 0; i < g.victim_unit.size(); ++i) {
+        if (caches && infllm_cache_slot_of(caches[g.victim_row[i]], g.victim_unit[i]) != g.victim_slot[i]) continue;     // gone by now
+        r.push_back(g.victim_row[i]);
+        sl.push_back(g.victim_slot[i]);
+        un.push_back(g.victim_unit[i]);
+        sr.push_back(g.victim_src[i]);
+    }
+    g.victim_unit.clear();
+    return do_fetch(L, (int)r.size(), r.data(), sl.data(), un.data(), sr.data(), st, cs);
+}
+
+}  // namespace
+
+extern "C" int infllm_block_prefetch(void *layer, const infllm_select_args *a, void *stream, void *copy_stream) {
+    INFLLM_REQUIRE(layer && a, "block_prefetch: null argument");
+    Layer *L = (Layer *)layer;
+    const infllm_layer_desc &d = L->d;
+    Layer::Ahead &g = L->ahead;
+    INFLLM_REQUIRE(!g.active, "block_prefetch: the previous guess has not been settled by infllm_block_select");
+    const int k = d.topk, B = d.B;
+    if (L->cand_for_units < 0 || !L->h_cand || k > 64) return 0;
+    L->cand_for_units = -1;
+    INFLLM_REQUIRE(a->caches && a->h_chunk_base && a->units_per_chunk > 0 && a->n_chunks >= 0 && a->unit_bytes > 0 && a->row_bytes > 0,
+                   "block_prefetch: bad cache list / host arena description");
+    // the candidates were chosen right after the local stage of the block in flight
+    const volatile int32_t *flag = L->h_cand + (int64_t)B * k;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t spins = 0; *flag != L->cand_seq; ++spins) {
+        if ((spins & 1023u) == 1023u && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) return 0;
+        __builtin_ia32_pause();
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
+    g.n_sel = k;
+    g.cand.assign(L->h_cand, L->h_cand + (int64_t)B * k);
+    g.sel_slots.resize((size_t)B * k);
+    g.evicted.resize((size_t)B * k);
+    g.n_evicted.assign(B, 0);
+    g.n_miss.assign(B, 0);
+    g.miss_row.clear(); g.miss_slot.clear(); g.miss_unit.clear(); g.miss_src.clear();
+    g.victim_row.clear(); g.victim_unit.clear(); g.victim_slot.clear(); g.victim_src.clear();
+    g.shadow.resize(B, nullptr);
+    for (int u = 0; u < B; ++u) {
+        INFLLM_REQUIRE(a->caches[u], "block_prefetch: null cache of row %d", u);
+        if (!g.shadow[u]) {
+            g.shadow[u] = infllm_cache_clone(a->caches[u]);
+            INFLLM_REQUIRE(g.shadow[u], "block_prefetch: no shadow cache");
+        } else {
+            const int crc = infllm_cache_copy(g.shadow[u], a->caches[u]);
+            if (crc) return crc;
+        }
+        int32_t units[64], slots[64], n_ev = 0;
+        const int32_t *cand = g.cand.data() + (int64_t)u * k;
+        for (int i = 0; i < k; ++i)
+            if (cand[i] < 0 || !host_unit(a, cand[i], u)) return 0;                 // not a list of units: no guess
+        const int m = infllm_cache_touch(g.shadow[u], cand, k, g.sel_slots.data() + (int64_t)u * k, units, slots,
+                                         g.evicted.data() + (int64_t)u * k, &n_ev);
+        if (m < 0) return m;
+        g.n_evicted[u] = n_ev;
+        g.n_miss[u] = m;
+        for (int e = 0; e < n_ev; ++e) {
+            const int32_t unit = g.evicted[(int64_t)u * k + e];
+            // a victim that the block in flight still reads: no fetch ahead this time
+            if ((int64_t)(u + 1) * L->last_n_sel <= (int64_t)L->last_sel.size())
+                for (int j = 0; j < L->last_n_sel; ++j)
+                    if (L->last_sel[(int64_t)u * L->last_n_sel + j] == unit) return 0;
+            g.victim_row.push_back(u);
+            g.victim_unit.push_back(unit);
+            g.victim_slot.push_back(infllm_cache_slot_of(a->caches[u], unit));
+            g.victim_src.push_back(host_unit(a, unit, u));
+        }
+        for (int i = 0; i < m; ++i) {
+            g.miss_row.push_back(u);
+            g.miss_slot.push_back(slots[i]);
+            g.miss_unit.push_back(units[i]);
+            g.miss_src.push_back(host_unit(a, units[i], u));
+        }
+    }
+    g.n_miss_all = (int)g.miss_unit.size();
+    const int rc = do_fetch(L, g.n_miss_all, g.miss_row.data(), g.miss_slot.data(), g.miss_unit.data(), g.miss_src.data(),
+                            (hipStream_t)stream, (hipStream_t)copy_stream, true);
+    if (rc) return rc;
+    g.active = true;
+    ++L->ahead_issued;
+    return g.n_miss_all;
+}
+
+extern "C" int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed) {
+    INFLLM_REQUIRE(layer, "layer_prefetch_stats: null layer");
+    Layer *L = (Layer *)layer;
+    if (issued) *issued = L->ahead_issued;
+    if (confirmed) *confirmed = L->ahead_confirmed;
+    return 0;
+}
+
 extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, void *copy_stream) {
     INFLLM_REQUIRE(layer && a, "block_select: null argument");
     Layer *L = (Layer *)layer;
@@ -706,6 +986,37 @@ extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, voi
     if (a->wait_topk) {
         const int wrc = infllm_layer_wait_topk(layer);
         if (wrc) return wrc;
+    }
+    L->last_n_sel = a->n_sel;
+    if (a->n_sel > 0) L->last_sel.assign(a->h_selected, a->h_selected + (int64_t)d.B * a->n_sel);
+    else L->last_sel.clear();
+    bool repair = false;
+    if (L->ahead.active) {
+        Layer::Ahead &g = L->ahead;
+        g.active = false;
+        if (a->n_sel == g.n_sel && std::memcmp(a->h_selected, g.cand.data(), sizeof(int32_t) * d.B * a->n_sel) == 0) {
+            // the guess was the selection: its policy state becomes the state, its fetch is the block's fetch
+            for (int u = 0; u < d.B; ++u) {
+                INFLLM_REQUIRE(a->caches[u], "block_select: null cache of row %d", u);
+                const int crc = infllm_cache_copy(a->caches[u], g.shadow[u]);
+                if (crc) return crc;
+                if (a->h_n_evicted) a->h_n_evicted[u] = g.n_evicted[u];
+                if (a->h_n_miss) a->h_n_miss[u] = g.n_miss[u];
+            }
+            std::memcpy(a->h_sel_slots, g.sel_slots.data(), sizeof(int32_t) * d.B * a->n_sel);
+            if (a->h_evicted) std::memcpy(a->h_evicted, g.evicted.data(), sizeof(int32_t) * d.B * a->n_sel);
+            for (int i = 0; i < g.n_miss_all; ++i) {
+                a->h_miss_row[i] = g.miss_row[i];
+                a->h_miss_slot[i] = g.miss_slot[i];
+                a->h_miss_unit[i] = g.miss_unit[i];
+                a->h_miss_src[i] = g.miss_src[i];
+            }
+            g.victim_unit.clear();
+            ++L->ahead_confirmed;
+            L->fetch_issued = true;
+            return g.n_miss_all;
+        }
+        repair = !g.victim_unit.empty();
     }
     int n_miss = 0;
     int32_t units[64], slots[64];
@@ -727,7 +1038,10 @@ extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, voi
             a->h_miss_src[n_miss] = (const void *)(uintptr_t)(a->h_chunk_base[chunk] + (uint64_t)idx * a->unit_bytes + (uint64_t)u * a->row_bytes);
         }
     }
-    const int rc = do_fetch(L, n_miss, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src, (hipStream_t)stream, (hipStream_t)copy_stream);
+    const int rc = repair ? ahead_repair(L, a->caches, n_miss, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src,
+                                         (hipStream_t)stream, (hipStream_t)copy_stream)
+                          : do_fetch(L, n_miss, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src, (hipStream_t)stream,
+                                     (hipStream_t)copy_stream);
     if (rc) return rc;
     L->fetch_issued = true;
     return n_miss;
@@ -843,6 +1157,10 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
         L->fetch_wait = false;
     }
+    if (L->efetch_wait) {           // the engines write the fetch's sequence number behind the units (a later fetch a larger one)
+        HIP_OK(hipStreamWaitValue32(st, L->d_efetch_flag, L->efetch_seq, hipStreamWaitValueGte, 0xffffffffu), "block_back: wait fetch flag");
+        L->efetch_wait = false;
+    }
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
     const int sl = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
     int parts = sl;
@@ -863,7 +1181,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         rc = infllm_attn_stage(&at, stream);
         timer_end(L, 1, ti, st);
         if (rc) return rc;
-        if (side) {
+        if (side || L->efetch_ok) {          // the next fetch (copy stream or DMA engines) must not overtake these reads
             HIP_OK(hipEventRecord(L->global_done, st), "block_back: event");
             L->has_global = true;
         }
@@ -989,6 +1307,12 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
 extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
     INFLLM_REQUIRE(layer, "layer_flush: null layer");
     Layer *L = (Layer *)layer;
+    if (L->ahead.active) {                      // a guess nobody settled: put back what it overwrote
+        L->ahead.active = false;
+        hipStream_t cs = (hipStream_t)copy_stream;
+        const int rrc = ahead_repair(L, nullptr, 0, nullptr, nullptr, nullptr, nullptr, cs, cs);
+        if (rrc) return rrc;
+    }
     if (L->off.pending) {
         int drc = issue_offload_dma(L);
         if (drc < 0) return drc;
