@@ -328,6 +328,14 @@ class ContextManager:
         if self._layer:
             check(self._lib.infllm_layer_timing(self._layer, capacity, stride), "infllm_layer_timing")
 
+    def prefetch_stats(self):
+        """(guesses made, guesses that turned out to be the selection) of the fetch ahead of the selection."""
+        issued, confirmed = ctypes.c_int64(0), ctypes.c_int64(0)
+        if self._layer:
+            check(self._lib.infllm_layer_prefetch_stats(self._layer, ctypes.byref(issued), ctypes.byref(confirmed)),
+                  "infllm_layer_prefetch_stats")
+        return issued.value, confirmed.value
+
     def read_timing(self, which):
         """[(ms, n_queries, n_keys)] of the timed launches; which = 0 local stage, 1 global stage."""
         cap = self._timing_cap

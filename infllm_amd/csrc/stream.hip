@@ -57,6 +57,7 @@ struct Layer {
     uint32_t *d_efetch_flag = nullptr, *h_efetch_val = nullptr;
     uint32_t efetch_seq = 0;
     bool efetch_wait = false;
+    int cur_n = 0;                                     // queries of the block in flight
     // The fetch ahead of the selection (see infllm_block_prefetch): the candidates' host copy with the sequence number
     // the kernel publishes behind them, the selection whose global stage may still be running, and the guess in flight.
     int32_t *h_cand = nullptr;                         // pinned [B*topk + 1]
@@ -76,6 +77,7 @@ struct Layer {
         std::vector<const void *> victim_src;
     } ahead;
     int64_t ahead_issued = 0, ahead_confirmed = 0;
+    bool ahead_any_path = false;                       // guess also when the fetch kernel has to move the units
     int page_cur = 0, carve_cur = 0;
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
@@ -339,6 +341,7 @@ int issue_offload(Layer *L, hipStream_t cs) {
 // here), and the last thing the engines write is a sequence number into a flag in signal memory, on which the main
 // stream waits (hipStreamWaitValue32) before the global stage.
 constexpr int kEfetchEngines = 8;
+constexpr int kEngineMinQueries = 64;
 constexpr int kEfetchVals = 8;
 
 int efetch_wait_signal(hsa_signal_t sig, const char *what) {
@@ -472,9 +475,15 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
             INFLLM_REQUIRE(rows[i] >= 0 && rows[i] < d.B && slots[i] >= 0 && slots[i] < d.max_cached && srcs[i], "fetch: bad miss entry");
             L->fetch_dst[i] = (bf16_t *)d.d_slab + ((int64_t)rows[i] * d.max_cached + slots[i]) * slot_elems;
         }
-        const int erc = fetch_by_engines(L, n_miss, srcs, slot_elems * (int64_t)sizeof(bf16_t), ahead);
+        // The engines pay where other kernels run beside the fetch; a short block (a decode step) has nothing to
+        // run beside it, and there the fetch kernel gets the units into place a little sooner (measured).
+        const int erc = ahead || L->cur_n >= kEngineMinQueries ? fetch_by_engines(L, n_miss, srcs, slot_elems * (int64_t)sizeof(bf16_t), ahead) : 0;
         if (erc < 0) return erc;
         if (erc == 0) {
+            if (L->efetch_ok) {                   // engine copies of an earlier fetch may aim at the same slots
+                const int wrc = efetch_wait_signal(L->efetch_flag_sig, "fetch");
+                if (wrc) return wrc;
+            }
             if (side && L->has_global && !ahead) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "fetch: wait global");
             int frc = infllm_fetch_units(srcs, L->fetch_dst.data(), n_miss, slot_elems * (int64_t)sizeof(bf16_t), cs);
             if (frc) return frc;
@@ -562,6 +571,10 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         }
     }
     efetch_setup(L);
+    {
+        const char *any = getenv("INFLLM_FETCH_AHEAD_ALWAYS");
+        L->ahead_any_path = any && any[0] && any[0] != '0';
+    }
     if (hipHostMalloc((void **)&L->h_cand, ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
         (void)hipGetLastError();
         L->h_cand = nullptr;                        // no fetch ahead of the selection then
@@ -763,6 +776,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     }
     L->prepared = false;
     L->cur_slot = L->slot;
+    L->cur_n = a->n;
     L->cand_for_units = -1;
 
     // ---- local stage: causal sliding window over the ring
@@ -902,6 +916,9 @@ extern "C" int infllm_block_prefetch(void *layer, const infllm_select_args *a, v
     const int k = d.topk, B = d.B;
     if (L->cand_for_units < 0 || !L->h_cand || k > 64) return 0;
     L->cand_for_units = -1;
+    // Beside the block's own kernels the fetch kernel slows them down by more than the shorter chain gains (measured):
+    // without the DMA engines the fetch stays behind the selection, unless INFLLM_FETCH_AHEAD_ALWAYS=1 asks for it.
+    if (!L->efetch_ok && !L->ahead_any_path) return 0;
     INFLLM_REQUIRE(a->caches && a->h_chunk_base && a->units_per_chunk > 0 && a->n_chunks >= 0 && a->unit_bytes > 0 && a->row_bytes > 0,
                    "block_prefetch: bad cache list / host arena description");
     // the candidates were chosen right after the local stage of the block in flight

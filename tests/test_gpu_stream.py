@@ -220,6 +220,38 @@ def test_carved_units_reach_the_host_by_either_copy_path(monkeypatch):
             assert torch.equal(hu[0, 0], k[0, :, lo:lo + bs]) and torch.equal(hu[0, 1], v[0, :, lo:lo + bs]), u
 
 
+def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
+    """The next block's misses are fetched from the candidates chosen before the block's own units are carved
+    (infllm_block_prefetch).  Whether the guess is confirmed or not, outputs, hit / miss / eviction counts, the
+    eviction sequence and the final residency are those of the run without it - with the units moved by the DMA
+    engines and by the fetch kernel (INFLLM_NO_DMA_FETCH=1), for lru and fifo, with a tight and a roomy cache."""
+    from infllm_amd.attention import ContextManager
+    T = 2600
+    q, k, v = _stream(T, 8, 2, 21, B=2)
+    seen_confirmed = seen_refuted = 0
+    for extra in (dict(max_cached_block=5), dict(max_cached_block=12), dict(max_cached_block=6, cache_strategy="fifo")):
+        kw = dict(SMALL, async_global_stream=True, **extra)
+        monkeypatch.setattr(ContextManager, "fetch_ahead", False)
+        plain, cm0 = _run_gpu(q, k, v, [1300, 1300], 1e4, **kw)
+        assert cm0.prefetch_stats() == (0, 0) and cm0.stats["misses"] > 0
+        monkeypatch.setattr(ContextManager, "fetch_ahead", True)
+        monkeypatch.setenv("INFLLM_FETCH_AHEAD_ALWAYS", "1")       # by default only the engines fetch ahead
+        for no_dma in ("0", "1"):
+            monkeypatch.setenv("INFLLM_NO_DMA_FETCH", no_dma)
+            ahead, cm1 = _run_gpu(q, k, v, [1300, 1300], 1e4, **kw)
+            issued, confirmed = cm1.prefetch_stats()
+            assert issued > 0 and 0 <= confirmed <= issued
+            seen_confirmed += confirmed
+            seen_refuted += issued - confirmed
+            assert torch.equal(plain, ahead) and cm0.stats == cm1.stats
+            for u in range(2):
+                assert cm0.policy[u].evicted_log == cm1.policy[u].evicted_log
+                assert cm0.policy[u].cached == cm1.policy[u].cached and cm0.policy[u].slot_of == cm1.policy[u].slot_of
+        monkeypatch.delenv("INFLLM_NO_DMA_FETCH")
+        monkeypatch.delenv("INFLLM_FETCH_AHEAD_ALWAYS")
+    assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
+
+
 def test_selection_in_separate_steps_equals_the_fused_call(monkeypatch):
     """infllm_layer_wait_topk + infllm_cache_touch + infllm_block_fetch, driven from the host, against
     infllm_block_select: same outputs, same residency events, for every policy."""
