@@ -390,6 +390,12 @@ int infllm_cache_destroy(void *cache);
  * slots they get; the evicted ids in eviction order (evicted / n_evicted may be NULL).  Returns the number of misses. */
 int infllm_cache_touch(void *cache, const int32_t *selected, int32_t n_sel, int32_t *slots, int32_t *miss_units,
                        int32_t *miss_slots, int32_t *evicted, int32_t *n_evicted);
+/* The same with slot wishes: a missed unit listed in hint_units takes its hint_slots entry when that slot is free
+ * once the evictions are done (a caller that has moved the unit there already, see infllm_block_prefetch); which slot
+ * a unit occupies changes nothing else. */
+int infllm_cache_touch_hinted(void *cache, const int32_t *selected, int32_t n_sel, int32_t *slots, int32_t *miss_units,
+                              int32_t *miss_slots, int32_t *evicted, int32_t *n_evicted, const int32_t *hint_units,
+                              const int32_t *hint_slots, int32_t n_hints);
 /* lru-s (context_manager.py:529-543): every resident's value decays, then the given units gain their scores */
 int infllm_cache_add_scores(void *cache, const int32_t *units, const double *scores, int32_t n);
 /* residents in insertion order (any output may be NULL); returns their number */
@@ -430,8 +436,10 @@ int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, 
  * stage -> next selection.  The next infllm_block_select settles it: when the selection equals the candidates
  * (all but the blocks in which a freshly carved unit makes the top-k) the copy becomes the policy state, the lists
  * and the return value are what the call would have produced, and nothing is left to fetch; otherwise the copy is
- * dropped, the call proceeds from the untouched state, and the residents whose slots the guess overwrote are
- * fetched again with the misses.  The hit / miss / eviction sequence is therefore the reference's either way.
+ * dropped and the call proceeds from the untouched state, except that a missed unit which the guess has moved
+ * already takes the slot it was moved to where that slot is free (infllm_cache_touch_hinted), so that only the other
+ * misses are fetched, together with the residents whose slots the guess overwrote.  The hit / miss / eviction
+ * sequence is therefore the reference's either way; which slot a unit occupies may differ from a run without guesses.
  * No guess is made (return 0) when no candidates are pending, or when the policy would evict a unit of the
  * selection whose global stage may still be running.  Valid only for policies whose state does not change between
  * this call and the selection (lru, fifo: the lru-s scores arrive with the block's attention mass).

@@ -153,6 +153,7 @@ SYMBOLS = {
     "infllm_cache_create": (c_vp, [c_i32, c_i32, c_f64]),
     "infllm_cache_destroy": (c_i32, [c_vp]),
     "infllm_cache_touch": (c_i32, [c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp]),
+    "infllm_cache_touch_hinted": (c_i32, [c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i32]),
     "infllm_cache_add_scores": (c_i32, [c_vp, c_vp, c_vp, c_i32]),
     "infllm_cache_residents": (c_i32, [c_vp, c_vp, c_vp, c_vp, c_i32]),
     "infllm_cache_slot_of": (c_i32, [c_vp, c_i32]),

@@ -56,7 +56,14 @@ extern "C" int infllm_cache_destroy(void *cache) {
 
 extern "C" int infllm_cache_touch(void *cache, const int32_t *selected, int32_t n_sel, int32_t *slots, int32_t *miss_units,
                                   int32_t *miss_slots, int32_t *evicted, int32_t *n_evicted) {
+    return infllm_cache_touch_hinted(cache, selected, n_sel, slots, miss_units, miss_slots, evicted, n_evicted, nullptr, nullptr, 0);
+}
+
+extern "C" int infllm_cache_touch_hinted(void *cache, const int32_t *selected, int32_t n_sel, int32_t *slots, int32_t *miss_units,
+                                         int32_t *miss_slots, int32_t *evicted, int32_t *n_evicted, const int32_t *hint_units,
+                                         const int32_t *hint_slots, int32_t n_hints) {
     INFLLM_REQUIRE(cache && n_sel >= 0 && (n_sel == 0 || (selected && slots && miss_units && miss_slots)), "cache_touch: bad arguments");
+    INFLLM_REQUIRE(n_hints >= 0 && (n_hints == 0 || (hint_units && hint_slots)), "cache_touch: bad hint list");
     UnitCache &c = *(UnitCache *)cache;
     INFLLM_REQUIRE(n_sel <= c.capacity, "cache_touch: %d selected units exceed max_cached_block %d", n_sel, c.capacity);
     int n_miss = 0;
@@ -109,11 +116,24 @@ extern "C" int infllm_cache_touch(void *cache, const int32_t *selected, int32_t 
             c.res.push_back(nr);
         }
     }
-    // slots are taken in the order of the miss list (= selection order), after the evictions freed theirs
+    // a missed unit with a hint takes the hinted slot when that is free now ...
+    for (int i = 0; i < n_miss && n_hints > 0; ++i)
+        for (int h = 0; h < n_hints; ++h) {
+            if (hint_units[h] != miss_units[i]) continue;
+            auto it = std::find(c.free_slots.begin(), c.free_slots.end(), hint_slots[h]);
+            if (it != c.free_slots.end()) {
+                c.find(miss_units[i])->slot = *it;
+                c.free_slots.erase(it);
+            }
+            break;
+        }
+    // ... the others take slots in the order of the miss list (= selection order), after the evictions freed theirs
     for (int i = 0; i < n_miss; ++i) {
         Resident *r = c.find(miss_units[i]);
-        r->slot = c.free_slots.back();
-        c.free_slots.pop_back();
+        if (r->slot < 0) {
+            r->slot = c.free_slots.back();
+            c.free_slots.pop_back();
+        }
         miss_slots[m++] = r->slot;
     }
     for (int i = 0; i < n_sel; ++i) slots[i] = c.find(selected[i])->slot;

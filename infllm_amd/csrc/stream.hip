@@ -58,6 +58,7 @@ struct Layer {
     uint32_t efetch_seq = 0;
     bool efetch_wait = false;
     int cur_n = 0;                                     // queries of the block in flight
+    bool guessing = false;                             // the last selection settled a fetch made ahead of it
     // The fetch ahead of the selection (see infllm_block_prefetch): the candidates' host copy with the sequence number
     // the kernel publishes behind them, the selection whose global stage may still be running, and the guess in flight.
     int32_t *h_cand = nullptr;                         // pinned [B*topk + 1]
@@ -95,7 +96,7 @@ struct Layer {
     int64_t prepared_b0 = 0;
     int prepared_n = 0;
     int timing_cap = 0, timing_stride = 1;
-    StageTimer timer[2];
+    StageTimer timer[3];               // local stage, global stage, the main stream's wait for the fetch
 };
 
 #define HIP_OK(call, what)                                                              \
@@ -638,7 +639,7 @@ extern "C" int infllm_layer_timing(void *layer, int32_t capacity, int32_t stride
 
 extern "C" int infllm_layer_read_timing(void *layer, int32_t which, float *ms, int32_t *n_queries, int32_t *n_keys,
                                         int32_t capacity) {
-    INFLLM_REQUIRE(layer && (which == 0 || which == 1) && ms && capacity >= 0, "layer_read_timing: bad arguments");
+    INFLLM_REQUIRE(layer && which >= 0 && which <= 2 && ms && capacity >= 0, "layer_read_timing: bad arguments");
     Layer *L = (Layer *)layer;
     StageTimer &t = L->timer[which];
     int n = t.used < capacity ? t.used : capacity;
@@ -1008,6 +1009,7 @@ extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, voi
     if (a->n_sel > 0) L->last_sel.assign(a->h_selected, a->h_selected + (int64_t)d.B * a->n_sel);
     else L->last_sel.clear();
     bool repair = false;
+    L->guessing = L->ahead.active;
     if (L->ahead.active) {
         Layer::Ahead &g = L->ahead;
         g.active = false;
@@ -1033,31 +1035,43 @@ extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, voi
             L->fetch_issued = true;
             return g.n_miss_all;
         }
-        repair = !g.victim_unit.empty();
+        repair = true;
     }
-    int n_miss = 0;
-    int32_t units[64], slots[64];
+    // From here on the policy state is the one before any guess.  After a guess that was not the selection, most of
+    // what it moved is still wanted: a missed unit takes the slot the guess put it in where that slot is free (the
+    // policy does not care which slot a unit has), and only the others are left to fetch.
+    Layer::Ahead &g = L->ahead;
+    int n_miss = 0, n_todo = 0;
+    int32_t units[64], slots[64], hint_units[64], hint_slots[64];
     INFLLM_REQUIRE(a->n_sel <= 64, "block_select: more than 64 units per row");
     for (int u = 0; u < d.B; ++u) {
         INFLLM_REQUIRE(a->caches[u], "block_select: null cache of row %d", u);
-        int32_t n_ev = 0;
-        const int m = infllm_cache_touch(a->caches[u], a->h_selected + (int64_t)u * a->n_sel, a->n_sel, a->h_sel_slots + (int64_t)u * a->n_sel,
-                                         units, slots, a->h_evicted ? a->h_evicted + (int64_t)u * a->n_sel : nullptr, &n_ev);
+        int32_t n_ev = 0, n_hints = 0;
+        if (repair)
+            for (int i = 0; i < g.n_miss_all && n_hints < 64; ++i)
+                if (g.miss_row[i] == u) hint_units[n_hints] = g.miss_unit[i], hint_slots[n_hints++] = g.miss_slot[i];
+        const int m = infllm_cache_touch_hinted(a->caches[u], a->h_selected + (int64_t)u * a->n_sel, a->n_sel,
+                                                a->h_sel_slots + (int64_t)u * a->n_sel, units, slots,
+                                                a->h_evicted ? a->h_evicted + (int64_t)u * a->n_sel : nullptr, &n_ev, hint_units, hint_slots, n_hints);
         if (m < 0) return m;
         if (a->h_n_evicted) a->h_n_evicted[u] = n_ev;
         if (a->h_n_miss) a->h_n_miss[u] = m;
         for (int i = 0; i < m; ++i, ++n_miss) {
-            const int chunk = units[i] / a->units_per_chunk, idx = units[i] % a->units_per_chunk;
-            INFLLM_REQUIRE(chunk < a->n_chunks && a->h_chunk_base[chunk], "block_select: unit %d has no host copy", units[i]);
-            a->h_miss_row[n_miss] = u;
-            a->h_miss_slot[n_miss] = slots[i];
-            a->h_miss_unit[n_miss] = units[i];
-            a->h_miss_src[n_miss] = (const void *)(uintptr_t)(a->h_chunk_base[chunk] + (uint64_t)idx * a->unit_bytes + (uint64_t)u * a->row_bytes);
+            bool in_place = false;                                  // the guess has put (or is putting) it there
+            for (int h = 0; h < n_hints && !in_place; ++h) in_place = hint_units[h] == units[i] && hint_slots[h] == slots[i];
+            if (in_place) continue;
+            const void *src = host_unit(a, units[i], u);
+            INFLLM_REQUIRE(src, "block_select: unit %d has no host copy", units[i]);
+            a->h_miss_row[n_todo] = u;
+            a->h_miss_slot[n_todo] = slots[i];
+            a->h_miss_unit[n_todo] = units[i];
+            a->h_miss_src[n_todo] = src;
+            ++n_todo;
         }
     }
-    const int rc = repair ? ahead_repair(L, a->caches, n_miss, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src,
+    const int rc = repair ? ahead_repair(L, a->caches, n_todo, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src,
                                          (hipStream_t)stream, (hipStream_t)copy_stream)
-                          : do_fetch(L, n_miss, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src, (hipStream_t)stream,
+                          : do_fetch(L, n_todo, a->h_miss_row, a->h_miss_slot, a->h_miss_unit, a->h_miss_src, (hipStream_t)stream,
                                      (hipStream_t)copy_stream);
     if (rc) return rc;
     L->fetch_issued = true;
@@ -1170,6 +1184,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     }
 
     // ---- 3. global stage and merge
+    const int tw = L->fetch_wait || L->efetch_wait ? timer_begin(L, 2, a->n, a->n_miss, st) : -1;
     if (L->fetch_wait) {
         HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
         L->fetch_wait = false;
@@ -1178,6 +1193,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         HIP_OK(hipStreamWaitValue32(st, L->d_efetch_flag, L->efetch_seq, hipStreamWaitValueGte, 0xffffffffu), "block_back: wait fetch flag");
         L->efetch_wait = false;
     }
+    timer_end(L, 2, tw, st);
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
     const int sl = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
     int parts = sl;
@@ -1242,7 +1258,15 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     //         init peeling, representatives of the new units
     const int64_t new_cursor = a->cursor + a->init_take + (int64_t)a->n_carve * bs;
     const int64_t urgent_hi = new_cursor < b1 ? new_cursor : b1;
-    rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, lse_now ? 0 : parts, stream);
+    // While the fetches run ahead of the selection nothing waits for this block's selection at once, and the split
+    // into an urgent and a bulk score launch only costs stream time: the merge and one score launch come first then.
+    const bool one_pass = L->guessing && !lse_now;
+    if (one_pass) {
+        rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, d.d_lse, stream);
+        if (rc) return rc;
+        rc = run_local_score(L, a->n, a->b0, cur, lo, b1, 0, stream);
+    } else
+        rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, lse_now ? 0 : parts, stream);
     if (rc) return rc;
     int64_t cursor = a->cursor;
     if (a->init_take > 0) {
@@ -1278,12 +1302,14 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     }
     L->cand_units = -1;
     // ---- 5b. the block's output rows
-    rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl,
-                           lse_now ? nullptr : d.d_lse, stream);
-    if (rc) return rc;
-    // ---- 6. off the critical path: the rest of the local score, new units to pinned host memory
-    rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, 0, stream);
-    if (rc) return rc;
+    if (!one_pass) {
+        rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl,
+                               lse_now ? nullptr : d.d_lse, stream);
+        if (rc) return rc;
+        // ---- 6. off the critical path: the rest of the local score, new units to pinned host memory
+        rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, 0, stream);
+        if (rc) return rc;
+    }
     if (a->n_carve > 0) {
         if (L->off.pending) {
             // the units of an earlier block are still waiting: their gathers were queued a whole block ago, so the

@@ -246,7 +246,8 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
             assert torch.equal(plain, ahead) and cm0.stats == cm1.stats
             for u in range(2):
                 assert cm0.policy[u].evicted_log == cm1.policy[u].evicted_log
-                assert cm0.policy[u].cached == cm1.policy[u].cached and cm0.policy[u].slot_of == cm1.policy[u].slot_of
+                assert cm0.policy[u].cached == cm1.policy[u].cached            # which slot a unit sits in may differ
+                assert sorted(cm1.policy[u].slot_of.values()) == sorted(set(cm1.policy[u].slot_of.values()))
         monkeypatch.delenv("INFLLM_NO_DMA_FETCH")
         monkeypatch.delenv("INFLLM_FETCH_AHEAD_ALWAYS")
     assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
@@ -267,7 +268,10 @@ def test_selection_in_separate_steps_equals_the_fused_call(monkeypatch):
         assert torch.equal(fused, steps) and cm0.stats == cm1.stats and cm0.stats["misses"] > 0
         for u in range(2):
             assert cm0.policy[u].evicted_log == cm1.policy[u].evicted_log
-            assert cm0.policy[u].cached == cm1.policy[u].cached and cm0.policy[u].slot_of == cm1.policy[u].slot_of
+            assert cm0.policy[u].cached == cm1.policy[u].cached
+            # the slots themselves may differ: the fused call fetches ahead of the selection and keeps what it moved
+            assert set(cm0.policy[u].slot_of) == set(cm1.policy[u].slot_of)
+            assert len(set(cm0.policy[u].slot_of.values())) == len(cm0.policy[u].slot_of)
 
 
 def test_state_export_and_injection_resume_the_stream_exactly():
