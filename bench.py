@@ -293,6 +293,8 @@ def main():
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12 if steady else 0.0
     glob_keys = KNOBS["topk"] * KNOBS["block_size"] + KNOBS["n_init"] + exc
     glob = [ms for c in runs for ms, nq, nk in c.read_timing(1) if nq == exc and nk == glob_keys]
+    waits = [ms for c in runs for ms, nq, nk in c.read_timing(2) if nq == exc]
+    guesses = [sum(x) for x in zip(*(c.prefetch_stats() for c in runs))]
     res = {
         "metric": "InfLLM attn tokens/s @128K ctx (1 layer, Mistral-7B geom); % HBM/MFMA roofline",
         "value": T * args.steps / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -308,6 +310,9 @@ def main():
                      "avg_launch_ms": avg_ms, "launches_timed": len(steady),
                      "global_stage_avg_ms": sum(glob) / max(len(glob), 1)},
         "cache": cm.stats,
+        # the next block's misses are fetched from its candidates, ahead of the selection: how often the candidates
+        # were the selection, and how long the main stream still waited for units (the wait itself costs ~6 us)
+        "fetch_ahead": {"guesses": guesses[0], "confirmed": guesses[1], "stream_wait_avg_ms": sum(waits) / max(len(waits), 1)},
     }
     if args.cpu_tokens > 0:
         res["cpu_baseline"] = cpu_baseline(args.cpu_tokens, min(os.cpu_count() or 1, 16))

@@ -245,7 +245,7 @@ int infllm_fetch_units(const void *const *h_src, void *const *d_dst, int32_t n, 
 void *infllm_host_device_pointer(void *h_pinned);
 
 /* ---------------------------------------------------------------------------
- * One execution block in three calls.
+ * One execution block in three calls (four with the fetch ahead of the selection).
  * Replaces the device work of ContextManager._append and append_global
  * (context_manager.py:474-545, 614-679) for one block of at most exc_block_size
  * queries; the host keeps the state machine (what is carved when), the cache policy is
@@ -265,7 +265,16 @@ void *infllm_host_device_pointer(void *h_pinned);
  *                        representatives of the new units, and - when the next block was
  *                        prepared - the scores of the new units, the next block's top-k and
  *                        the copy of its ids; only then the block's output rows, the rest of the
- *                        local score and the gather of the new units into a staging slot.
+ *                        local score and the gather of the new units into a staging slot
+ *                        (while fetches run ahead of the selection: merge and ONE local-score launch
+ *                        before the representatives, since nothing waits for the selection at once);
+ *   infllm_block_prefetch  (optional, further down) starts the NEXT block's fetch from its candidates.
+ *
+ * The fetch of missed units goes through 8 DMA engines (ROCr copies) for blocks of 64 queries or more, and the
+ * main stream waits with hipStreamWaitValue32 for a sequence number the engines write behind the units; shorter
+ * blocks, and processes without usable engines (or with INFLLM_NO_DMA_FETCH=1), use the zero-copy kernel
+ * of infllm_fetch_units on the copy stream.  Either way the fetch is ordered behind the last reader of the slots
+ * and behind the offload of units that are still on their way to the host.
  *
  * The chain from one block's ids to the next block's ids is therefore: fetch, global stage,
  * a small local-score launch (which joins the stages' log-sum-exps itself), representatives, a
@@ -284,9 +293,9 @@ void *infllm_host_device_pointer(void *h_pinned);
  * infllm_block_front prepares the next block is taken there (off the chain), and after the block only
  * those k candidates and the units carved in between are ranked (same result as one top-k over all).
  *
- * A layer handle owns only events, ROCr signals, a [B,topk] device array for those candidates, the
- * rotation of the pinned page-table staging slots and of the carve staging slots; every other buffer
- * is the caller's.
+ * A layer handle owns only events, ROCr signals, a [B,topk] device array and a pinned copy for those
+ * candidates, 8 bytes of signal memory, shadow policy objects for the guess in flight, the rotation of the
+ * pinned page-table staging slots and of the carve staging slots; every other buffer is the caller's.
  */
 typedef struct {
     int32_t B, H, Hkv;
@@ -452,7 +461,7 @@ int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed
 /* Event timing of the two attention stages (for benchmarks): enable with a record
  * capacity and a stride (every stride-th launch of each stage is bracketed by two events; an event pair
  * costs the stream several microseconds, so a throughput run samples), read back (which: 0 local stage,
- * 1 global stage) after a device sync.
+ * 1 global stage, 2 the main stream's wait for the fetch in infllm_block_back) after a device sync.
  * ms[i] is the launch-to-finish time of one stage launch, n_queries[i] its block size,
  * n_keys[i] the key rows its source held. */
 int infllm_layer_timing(void *layer, int32_t capacity, int32_t stride);
