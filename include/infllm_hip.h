@@ -197,6 +197,15 @@ int infllm_local_score(const infllm_score_args *a, void *stream);
 int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C,
                       const float *d_qbar, int32_t k,
                       float *d_scores, int32_t *d_idx, void *stream);
+/* The selection over ALL units from two parts (what the stream does between blocks): d_cand[n_cand] are the k best,
+ * ids ascending, of units [0, first_new) (infllm_topk over their scores, taken while other work was in flight);
+ * this scores the n_new units [first_new, first_new + n_new) (d_scores[first_new ...] = reps . qbar, the same
+ * arithmetic as infllm_unit_scores) and ranks them against the candidates in the same launch: d_idx[k] as
+ * infllm_topk over all first_new + n_new scores would give (a unit of the overall top-k that is not new is among
+ * the k best of the old ones).  n_cand + n_new <= 64; rows of 512, 1024, 2048 or 4096 elements. */
+int infllm_score_new_topk(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores,
+                          const int32_t *d_cand, int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx,
+                          void *stream);
 /* The two halves of infllm_score_topk: scores of rows [first, first+count) into d_scores[first..], and the
  * selection over d_scores[0..N).  Scoring the units that exist early and only the newly carved ones late keeps
  * the retrieval of the next block short. */

@@ -325,6 +325,60 @@ __global__ __launch_bounds__(64) void topk_merge_kernel(const float *scores, con
     publish(flag, flag_value);
 }
 
+// The two steps above in one launch for the few units carved since the candidates were chosen: wave w of the
+// one workgroup scores new units w, w + 4, ... (the arithmetic of unit_scores_rows_kernel, term by term, so a
+// unit's score does not depend on which kernel computed it), then the first wave ranks candidates and new units.
+template <int CPL>
+__global__ __launch_bounds__(256) void score_new_rank_kernel(const bf16_t *reps, int64_t rep_stride, const float *qbar, float *scores,
+                                                             const int32_t *cand, int n_cand, int first_new, int n_new, int k,
+                                                             int32_t *idx_out, int32_t *flag, int32_t flag_value) {
+    __shared__ float fresh[64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float q[CPL][8];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) {
+        const f32x4 lo = *(const f32x4 *)(qbar + j * 512 + lane * 8), hi = *(const f32x4 *)(qbar + j * 512 + lane * 8 + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) q[j][i] = lo[i], q[j][4 + i] = hi[i];
+    }
+    for (int r = wave; r < n_new; r += 4) {
+        const bf16_t *row = reps + (int64_t)(first_new + r) * rep_stride + lane * 8;
+        u32x4 w[CPL];
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) w[j] = *(const u32x4 *)(row + j * 512);
+        float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc0 += bf16_bits_to_f32(w[j][i] & 0xffffu) * q[j][2 * i];
+                acc1 += bf16_bits_to_f32(w[j][i] >> 16) * q[j][2 * i + 1];
+            }
+        }
+        const float acc = wave_sum(acc0 + acc1);
+        if (lane == 0) {
+            scores[first_new + r] = acc;
+            fresh[r] = acc;
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const int n = n_cand + n_new;
+        const bool valid = lane < n;
+        const int id = lane < n_cand ? cand[lane] : first_new + (lane - n_cand);       // ascending in the lane
+        const uint32_t key = !valid ? 0u : order_key(lane < n_cand ? scores[id] : fresh[lane - n_cand]);
+        int rank = 0;
+        for (int j = 0; j < n; ++j) {
+            const uint32_t kj = __shfl(key, j, 64);
+            rank += (kj > key || (kj == key && j < lane)) ? 1 : 0;
+        }
+        const bool sel = valid && rank < k;
+        const uint64_t mask = __ballot(sel);
+        if (sel) idx_out[__popcll(mask & ((1ull << lane) - 1))] = id;
+    }
+    publish(flag, flag_value);
+}
+
 // ---------------------------------------------------------------- representative keys
 constexpr int kMaxUnit = 2048;             // largest supported unit (block_size)
 
@@ -447,6 +501,34 @@ int infllm_topk_merge_publish(const float *d_scores, const int32_t *d_cand, int3
                        d_idx, d_flag, flag_value);
     INFLLM_CHECK_LAUNCH("topk_merge");
     return 0;
+}
+
+// unit scores of the n_new units from first_new on, then the ranking of infllm_topk_merge_publish, in one launch.
+// Returns 1 when the row length has no such kernel (the caller then launches the two steps).
+int infllm_score_new_rank(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores, const int32_t *d_cand,
+                          int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx, int32_t *d_flag,
+                          int32_t flag_value, void *stream) {
+    INFLLM_REQUIRE(d_reps && d_qbar && d_scores && d_cand && d_idx, "score_new_rank: null pointer");
+    INFLLM_REQUIRE(n_cand >= 0 && n_new >= 0 && n_cand + n_new <= 64 && k > 0 && k <= n_cand + n_new && first_new >= 0,
+                   "score_new_rank: %d + %d candidates for k=%d", n_cand, n_new, k);
+    INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "score_new_rank: row stride %lld", (long long)rep_stride);
+    const bf16_t *reps = (const bf16_t *)d_reps;
+    switch (C % 512 == 0 ? C / 512 : 0) {
+#define RANK_CASE(n) case n: hipLaunchKernelGGL(score_new_rank_kernel<n>, dim3(1), dim3(256), 0, (hipStream_t)stream, reps, rep_stride, d_qbar, \
+                                                 d_scores, d_cand, n_cand, first_new, n_new, k, d_idx, d_flag, flag_value); break
+        RANK_CASE(1); RANK_CASE(2); RANK_CASE(4); RANK_CASE(8);
+#undef RANK_CASE
+    default: return 1;
+    }
+    INFLLM_CHECK_LAUNCH("score_new_rank");
+    return 0;
+}
+
+extern "C" int infllm_score_new_topk(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores,
+                                     const int32_t *d_cand, int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx,
+                                     void *stream) {
+    const int rc = infllm_score_new_rank(d_reps, rep_stride, C, d_qbar, d_scores, d_cand, n_cand, first_new, n_new, k, d_idx, nullptr, 0, stream);
+    return rc == 1 ? infllm_fail(-1, "score_new_topk: rows of %d elements (supported: 512, 1024, 2048, 4096)", C) : rc;
 }
 
 extern "C" int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbar,

@@ -122,6 +122,9 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_score_new_rank(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores, const int32_t *d_cand,
+                          int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx, int32_t *d_flag,
+                          int32_t flag_value, void *stream);
 int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag,
                              int32_t flag_value, void *stream);
 int infllm_gather_rows_pair(const void *d_ring_a, void *d_out_a, const void *d_ring_b, void *d_out_b, int64_t ring_cap, int32_t B,
@@ -731,6 +734,31 @@ int run_topk_merge(Layer *L, const float *scores, int64_t scores_sb, int n_old, 
     return 0;
 }
 
+// the scores of the n_new units carved since the candidates were chosen and the ranking, one launch per batch row;
+// returns 1 (nothing launched) when there is no such kernel for this geometry
+int run_score_new_rank(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_su, float *scores, int64_t scores_sb, int n_old, int n_new,
+                       void *stream) {
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream;
+    const int C = d.H * kD;
+    if (C % 512 != 0 || (C / 512 != 1 && C / 512 != 2 && C / 512 != 4 && C / 512 != 8) || n_new < 1) return 1;
+    const bool poll = d.d_topk_flag && d.h_topk_flag && !d.h_topk_idx;
+    if (poll) ++L->topk_seq;
+    for (int u = 0; u < d.B; ++u) {
+        const bool last = poll && u == d.B - 1;
+        int rc = infllm_score_new_rank((const bf16_t *)reps + (int64_t)u * rep_sb, rep_su, C, d.d_qbar + ((int64_t)L->slot * d.B + u) * C,
+                                       scores + (int64_t)u * scores_sb, L->d_cand + (int64_t)u * d.topk, d.topk, n_old, n_new, d.topk,
+                                       d.d_topk_idx + (int64_t)u * d.topk, last ? d.d_topk_flag : nullptr, L->topk_seq, stream);
+        if (rc) return rc < 0 ? rc : infllm_fail(-2, "score_new_rank: no kernel after the geometry check");
+    }
+    if (d.h_topk_idx)
+        HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
+    if (!poll) HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    L->topk_stream = st;
+    L->topk_pending = true;
+    return 0;
+}
+
 // n_parts > 0: the stages' partial log-sum-exps are joined inside the launch (d_lse is not ready yet)
 int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t j_hi, int n_parts, void *stream) {
     const infllm_layer_desc &d = L->d;
@@ -1291,14 +1319,20 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     const int n_units_next = a->n_units + a->n_carve;
     if (L->prepared && n_units_next > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL)) {
         INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_back: null representative / score buffer");
-        rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->slot,
-                             stream);
-        if (rc) return rc;
-        if (L->cand_units == a->n_units && d.topk + a->n_carve <= 64)
-            rc = run_topk_merge(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, stream);
-        else
-            rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, n_units_next, stream);
-        if (rc) return rc;
+        const bool merge = L->cand_units == a->n_units && d.topk + a->n_carve <= 64;
+        rc = merge ? run_score_new_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, stream)
+                   : 1;
+        if (rc < 0) return rc;
+        if (rc == 1) {                  // the two steps on their own
+            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->slot,
+                                 stream);
+            if (rc) return rc;
+            if (merge)
+                rc = run_topk_merge(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, stream);
+            else
+                rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, n_units_next, stream);
+            if (rc) return rc;
+        }
     }
     L->cand_units = -1;
     // ---- 5b. the block's output rows

@@ -190,6 +190,14 @@ def score_topk(reps, n, qbar, k, scores, idx):
           "infllm_score_topk")
 
 
+def score_new_topk(reps, qbar, scores, cand, first_new, n_new, k, idx):
+    """scores[first_new:first_new+n_new] = reps[those rows] @ qbar, then idx[:k] = the top-k over all first_new + n_new
+    scores, given cand = the top-k (ascending ids) of the first first_new."""
+    check(_lib.load().infllm_score_new_topk(reps.data_ptr(), reps.stride(0), reps.shape[1], qbar.data_ptr(), scores.data_ptr(),
+                                            cand.data_ptr(), cand.numel(), first_new, n_new, k, idx.data_ptr(), _stream()),
+          "infllm_score_new_topk")
+
+
 def topk(scores, n, k, idx):
     """idx[:k] = ascending indices of the k largest of scores[:n] (lowest indices among equal scores)."""
     check(_lib.load().infllm_topk(scores.data_ptr(), n, k, idx.data_ptr(), _stream()), "infllm_topk")

@@ -325,6 +325,29 @@ def test_score_topk_matches_bruteforce(N, k):
         assert abs(want[i] - kth) <= 1e-3 * abs(kth)
 
 
+@pytest.mark.parametrize("n_old,n_new,k,heads", [(991, 4, 16, 32), (40, 1, 16, 32), (16, 16, 16, 8), (300, 7, 4, 16), (5000, 48, 16, 4),
+                                                 (64, 3, 1, 32)])
+def test_new_units_scored_and_ranked_in_one_launch_equal_the_two_steps(n_old, n_new, k, heads):
+    """infllm_score_new_topk against infllm_score_topk over all rows: the new rows' scores bit for bit, the same ids
+    (also with exact ties between an old and a new unit, which go to the lower index)."""
+    ops = _ops()
+    C, N = heads * D, n_old + n_new
+    reps = _rand((N, C), 300 + N)
+    reps[n_old:n_old + min(2, n_new)] = reps[:min(2, n_new)]              # exact ties old / new
+    qbar = torch.randn(C, generator=torch.Generator().manual_seed(43)).cuda()
+    repd = reps.cuda()
+    want_scores = torch.empty((N,), dtype=torch.float32, device="cuda")
+    want_idx = torch.empty((k,), dtype=torch.int32, device="cuda")
+    ops.score_topk(repd, N, qbar, k, want_scores, want_idx)
+    scores = torch.full((N,), float("nan"), dtype=torch.float32, device="cuda")
+    cand = torch.empty((k,), dtype=torch.int32, device="cuda")
+    ops.score_topk(repd, n_old, qbar, k, scores, cand)
+    idx = torch.empty((k,), dtype=torch.int32, device="cuda")
+    ops.score_new_topk(repd, qbar, scores, cand, n_old, n_new, k, idx)
+    assert torch.equal(scores, want_scores)
+    assert idx.cpu().tolist() == want_idx.cpu().tolist()
+
+
 def test_topk_with_exact_ties_takes_lowest_indices():
     ops = _ops()
     N, C = 300, 128
