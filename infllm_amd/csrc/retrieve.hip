@@ -382,11 +382,38 @@ __global__ __launch_bounds__(256) void score_new_rank_kernel(const bf16_t *reps,
 // ---------------------------------------------------------------- representative keys
 constexpr int kMaxUnit = 2048;             // largest supported unit (block_size)
 
-// one wave per (query head, unit, batch row)
+// The copy of the same units' K and V rows out of the rings into contiguous staging (what infllm_gather_rows does)
+// can ride in the launch that picks their representatives: independent work, one launch less in the stream.
+struct CarveCopy {
+    const bf16_t *ring_a, *ring_b;
+    bf16_t *out_a, *out_b;
+    int64_t ring_cap, t0, out_sb, out_su, out_sh;
+    int32_t Hkv, B, n, unit_rows, x_extra;         // n rows from t0 on; x_extra = extra workgroups along x (0: no copy)
+};
+
+// one wave per (query head, unit, batch row); workgroups with blockIdx.x >= H copy
 __global__ __launch_bounds__(64) void repr_keys_kernel(const float *ring_score, const bf16_t *ring_k, int64_t ring_cap,
                                                        int H, int Hkv, int64_t t0, int bs, int repr_topk, bf16_t *rep_out,
-                                                       int64_t rep_sb, int64_t rep_su, int32_t *idx_out) {
+                                                       int64_t rep_sb, int64_t rep_su, int32_t *idx_out, CarveCopy cc) {
     __shared__ float sc[kMaxUnit];
+    if ((int)blockIdx.x >= H) {
+        const int64_t g = ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * cc.x_extra + ((int)blockIdx.x - H);
+        const int64_t e = g * 64 + threadIdx.x;                        // (ring, batch row, kv head, row, 16-byte chunk)
+        if (e >= (int64_t)2 * cc.B * cc.Hkv * cc.n * 16) return;
+        const int c = (int)(e & 15);
+        int64_t rest = e >> 4;
+        const int r = (int)(rest % cc.n);
+        rest /= cc.n;
+        const int hk = (int)(rest % cc.Hkv);
+        rest /= cc.Hkv;
+        const int bb = (int)(rest % cc.B);
+        const bool second = rest / cc.B != 0;
+        const bf16_t *src = (second ? cc.ring_b : cc.ring_a) + (((int64_t)bb * cc.Hkv + hk) * cc.ring_cap + (cc.t0 + r) % cc.ring_cap) * kD + c * 8;
+        bf16_t *dst = (second ? cc.out_b : cc.out_a) + (int64_t)bb * cc.out_sb + (int64_t)(r / cc.unit_rows) * cc.out_su +
+                      (int64_t)hk * cc.out_sh + (int64_t)(r % cc.unit_rows) * kD + c * 8;
+        *(u32x4 *)dst = *(const u32x4 *)src;
+        return;
+    }
     const int h = blockIdx.x, u = blockIdx.y, b = blockIdx.z, lane = threadIdx.x;
     const int n_units = gridDim.y;
     const int g = h / (H / Hkv);
@@ -539,9 +566,12 @@ extern "C" int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t
     return rc;
 }
 
-extern "C" int infllm_repr_keys(const float *d_ring_score, const void *d_ring_k_raw, int64_t ring_cap, int32_t B, int32_t H,
-                                int32_t Hkv, int64_t t0, int32_t bs, int32_t n_units, int32_t repr_topk, void *d_rep_out,
-                                int64_t rep_sb, int64_t rep_su, int32_t *d_idx_out, void *stream) {
+// internal: infllm_repr_keys, and in the same launch the K (ring_v: V) rows of those units out of the rings into
+// d_out_k / d_out_v as infllm_gather_rows lays them out (unit_rows = bs); d_ring_v == NULL: no copy
+int infllm_repr_keys_carve(const float *d_ring_score, const void *d_ring_k_raw, int64_t ring_cap, int32_t B, int32_t H, int32_t Hkv,
+                           int64_t t0, int32_t bs, int32_t n_units, int32_t repr_topk, void *d_rep_out, int64_t rep_sb, int64_t rep_su,
+                           int32_t *d_idx_out, const void *d_ring_v, void *d_out_k, void *d_out_v, int64_t out_sb, int64_t out_su,
+                           int64_t out_sh, void *stream) {
     INFLLM_REQUIRE(d_ring_score && d_ring_k_raw && d_rep_out, "repr_keys: null pointer");
     INFLLM_REQUIRE(B > 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "repr_keys: bad geometry B=%d H=%d Hkv=%d", B, H, Hkv);
     INFLLM_REQUIRE(bs > 0 && bs <= kMaxUnit, "repr_keys: unit size %d not in 1..%d", bs, kMaxUnit);
@@ -550,9 +580,26 @@ extern "C" int infllm_repr_keys(const float *d_ring_score, const void *d_ring_k_
                    n_units);
     INFLLM_REQUIRE(rep_sb % 2 == 0 && rep_su % 2 == 0, "repr_keys: output strides must be even");
     if (n_units == 0) return 0;
-    hipLaunchKernelGGL(repr_keys_kernel, dim3(H, n_units, B), dim3(64), 0, (hipStream_t)stream, d_ring_score,
+    CarveCopy cc{};
+    if (d_ring_v) {
+        INFLLM_REQUIRE(d_out_k && d_out_v && (out_sb % 8 | out_su % 8 | out_sh % 8) == 0, "repr_keys: bad copy destination");
+        cc.ring_a = (const bf16_t *)d_ring_k_raw; cc.ring_b = (const bf16_t *)d_ring_v;
+        cc.out_a = (bf16_t *)d_out_k; cc.out_b = (bf16_t *)d_out_v;
+        cc.ring_cap = ring_cap; cc.t0 = t0; cc.out_sb = out_sb; cc.out_su = out_su; cc.out_sh = out_sh;
+        cc.Hkv = Hkv; cc.B = B; cc.n = n_units * bs; cc.unit_rows = bs;
+        const int64_t waves = ((int64_t)2 * B * Hkv * cc.n * 16 + 63) / 64, per_x = (int64_t)n_units * B;
+        cc.x_extra = (int32_t)((waves + per_x - 1) / per_x);
+    }
+    hipLaunchKernelGGL(repr_keys_kernel, dim3(H + cc.x_extra, n_units, B), dim3(64), 0, (hipStream_t)stream, d_ring_score,
                        (const bf16_t *)d_ring_k_raw, ring_cap, H, Hkv, t0, bs, repr_topk, (bf16_t *)d_rep_out, rep_sb,
-                       rep_su, d_idx_out);
+                       rep_su, d_idx_out, cc);
     INFLLM_CHECK_LAUNCH("repr_keys");
     return 0;
+}
+
+extern "C" int infllm_repr_keys(const float *d_ring_score, const void *d_ring_k_raw, int64_t ring_cap, int32_t B, int32_t H,
+                                int32_t Hkv, int64_t t0, int32_t bs, int32_t n_units, int32_t repr_topk, void *d_rep_out,
+                                int64_t rep_sb, int64_t rep_su, int32_t *d_idx_out, void *stream) {
+    return infllm_repr_keys_carve(d_ring_score, d_ring_k_raw, ring_cap, B, H, Hkv, t0, bs, n_units, repr_topk, d_rep_out, rep_sb, rep_su,
+                                  d_idx_out, nullptr, nullptr, nullptr, 0, 0, 0, stream);
 }

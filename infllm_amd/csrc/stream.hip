@@ -125,6 +125,10 @@ int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_
 int infllm_score_new_rank(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores, const int32_t *d_cand,
                           int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx, int32_t *d_flag,
                           int32_t flag_value, void *stream);
+int infllm_repr_keys_carve(const float *d_ring_score, const void *d_ring_k_raw, int64_t ring_cap, int32_t B, int32_t H, int32_t Hkv,
+                           int64_t t0, int32_t bs, int32_t n_units, int32_t repr_topk, void *d_rep_out, int64_t rep_sb, int64_t rep_su,
+                           int32_t *d_idx_out, const void *d_ring_v, void *d_out_k, void *d_out_v, int64_t out_sb, int64_t out_su,
+                           int64_t out_sh, void *stream);
 int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag,
                              int32_t flag_value, void *stream);
 int infllm_gather_rows_pair(const void *d_ring_a, void *d_out_a, const void *d_ring_b, void *d_out_b, int64_t ring_cap, int32_t B,
@@ -1309,10 +1313,42 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         cursor += a->init_take;
     }
     if (a->n_carve > 0) {
+        // representatives of the new units, and in the same launch their rows out of the rings into a staging slot
+        // (from there they go to pinned host memory, off the critical path)
         INFLLM_REQUIRE(a->d_rep_out && a->h_carve_dst, "block_back: null carve outputs");
-        rc = infllm_repr_keys(d.d_ring_score, d.d_ring_k_raw, d.ring_cap, d.B, d.H, d.Hkv, cursor, bs, a->n_carve, d.repr_topk,
-                              a->d_rep_out, a->rep_sb, a->rep_su, a->d_repr_idx, stream);
+        for (int i = 0; i < a->n_carve; ++i) INFLLM_REQUIRE(a->h_carve_dst[i], "block_back: null carve destination");
+        if (L->off.pending) {
+            // the units of an earlier block are still waiting: their copy into staging was queued a whole block ago, so
+            // the host gets through this wait at once and the engine can take them; else the copy stream does
+            int drc = 0;
+            if (L->dma_ok) {
+                HIP_OK(hipEventSynchronize(L->carve_ready), "block_back: carve event");
+                drc = issue_offload_dma(L);
+                if (drc < 0) return drc;
+            }
+            if (drc == 0) {
+                rc = issue_offload(L, cs);
+                if (rc) return rc;
+            }
+        }
+        const int slot = L->carve_cur;
+        L->carve_cur = (slot + 1) % d.carve_slots;
+        if (L->carve_busy[slot]) HIP_OK(hipEventSynchronize(L->carve_evt[slot]), "block_back: carve slot");
+        rc = dma_wait_slot(L, slot, "block_back");
         if (rc) return rc;
+        const int64_t unit_all = (int64_t)d.B * slot_elems;                       // one unit, all batch rows
+        bf16_t *stage = (bf16_t *)d.d_carve_stage + (int64_t)slot * d.max_carve * unit_all;
+        rc = infllm_repr_keys_carve(d.d_ring_score, d.d_ring_k_raw, d.ring_cap, d.B, d.H, d.Hkv, cursor, bs, a->n_carve, d.repr_topk,
+                                    a->d_rep_out, a->rep_sb, a->rep_su, a->d_repr_idx, d.d_ring_v, stage, stage + unit_elems, slot_elems,
+                                    unit_all, (int64_t)bs * kD, stream);
+        if (rc) return rc;
+        HIP_OK(hipEventRecord(L->carve_ready, st), "block_back: event");
+        L->off.pending = true;
+        L->off.slot = slot;
+        L->off.first_unit = a->n_units;
+        L->off.count = a->n_carve;
+        L->off.dst.assign(a->h_carve_dst, a->h_carve_dst + a->n_carve);
+        L->copy_stream = cs;
     }
     // ---- 5. the next block's retrieval (its prologue ran in block_front)
     L->topk_pending = false;
@@ -1343,40 +1379,6 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         // ---- 6. off the critical path: the rest of the local score, new units to pinned host memory
         rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, 0, stream);
         if (rc) return rc;
-    }
-    if (a->n_carve > 0) {
-        if (L->off.pending) {
-            // the units of an earlier block are still waiting: their gathers were queued a whole block ago, so the
-            // host gets through this wait at once and the engine can take them; else the copy stream does
-            int drc = 0;
-            if (L->dma_ok) {
-                HIP_OK(hipEventSynchronize(L->carve_ready), "block_back: carve event");
-                drc = issue_offload_dma(L);
-                if (drc < 0) return drc;
-            }
-            if (drc == 0) {
-                rc = issue_offload(L, cs);
-                if (rc) return rc;
-            }
-        }
-        const int slot = L->carve_cur;
-        L->carve_cur = (slot + 1) % d.carve_slots;
-        if (L->carve_busy[slot]) HIP_OK(hipEventSynchronize(L->carve_evt[slot]), "block_back: carve slot");
-        rc = dma_wait_slot(L, slot, "block_back");
-        if (rc) return rc;
-        const int64_t unit_all = (int64_t)d.B * slot_elems;                       // one unit, all batch rows
-        bf16_t *stage = (bf16_t *)d.d_carve_stage + (int64_t)slot * d.max_carve * unit_all;
-        rc = infllm_gather_rows_pair(d.d_ring_k_raw, stage, d.d_ring_v, stage + unit_elems, d.ring_cap, d.B, d.Hkv, cursor,
-                                     a->n_carve * bs, bs, slot_elems, unit_all, (int64_t)bs * kD, stream);
-        if (rc) return rc;
-        HIP_OK(hipEventRecord(L->carve_ready, st), "block_back: event");
-        for (int i = 0; i < a->n_carve; ++i) INFLLM_REQUIRE(a->h_carve_dst[i], "block_back: null carve destination");
-        L->off.pending = true;
-        L->off.slot = slot;
-        L->off.first_unit = a->n_units;
-        L->off.count = a->n_carve;
-        L->off.dst.assign(a->h_carve_dst, a->h_carve_dst + a->n_carve);
-        L->copy_stream = cs;
     }
     return 0;
 }
