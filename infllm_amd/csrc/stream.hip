@@ -40,7 +40,13 @@ struct Layer {
         bool pending = false;
         int slot = 0, first_unit = 0, count = 0;
         std::vector<void *> dst;
+        // how the host learns that the copy into staging has finished: the selection kernel launched behind it has
+        // published its sequence number (after_seq != 0), or the event carve_ready (has_event)
+        int32_t after_seq = 0;
+        bool has_event = false;
     } off;
+    int32_t seen_seq = 0;                 // last selection sequence number the host has read
+    hipStream_t main_stream = nullptr;    // of the last infllm_block_back
     // The same copy through the DMA engine (see issue_offload_dma): agents of this layer's GPU and of the host,
     // one completion signal per carve staging slot, and which units a slot's copy in flight carries
     bool dma_ok = false;
@@ -271,16 +277,54 @@ int dma_wait_slot(Layer *L, int slot, const char *what) {
     return 0;
 }
 
+// Has the copy of the pending units into their staging slot finished?  1 yes, 0 not yet, < 0 error.
+int carve_copied(Layer *L) {
+    if (L->off.has_event) {
+        const hipError_t q = hipEventQuery(L->carve_ready);
+        if (q == hipErrorNotReady) {
+            (void)hipGetLastError();               // "not ready" is an answer, not a failure of a later launch
+            return 0;
+        }
+        if (q != hipSuccess) return infllm_fail(-2, "offload: %s", hipGetErrorString(q));
+        return 1;
+    }
+    if (L->off.after_seq == 0) return 1;           // nothing was launched
+    if (L->seen_seq - L->off.after_seq >= 0) return 1;
+    const volatile int32_t *flag = L->d.h_topk_flag;
+    return flag && *flag - L->off.after_seq >= 0 ? 1 : 0;
+}
+
+// an event for it after all (recorded late it covers more than the copy, which is harmless)
+int carve_event(Layer *L) {
+    if (!L->off.has_event) {
+        HIP_OK(hipEventRecord(L->carve_ready, L->main_stream), "offload: event");
+        L->off.has_event = true;
+    }
+    return 0;
+}
+
+// host wait for the same
+int carve_wait(Layer *L) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t spins = 0; !L->off.has_event; ++spins) {
+        const int c = carve_copied(L);
+        if (c) return c < 0 ? c : 0;
+        if ((spins & 1023u) == 1023u && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) {
+            const int erc = carve_event(L);
+            if (erc) return erc;
+        }
+        __builtin_ia32_pause();
+    }
+    HIP_OK(hipEventSynchronize(L->carve_ready), "offload: wait for the copy into staging");
+    return 0;
+}
+
 // Try to hand the pending units to the DMA engine.  Returns 1 when issued, 0 when not possible right now (the gather
 // kernels have not finished, or there is no engine path), < 0 on error.
 int issue_offload_dma(Layer *L) {
     if (!L->dma_ok || !L->off.pending) return 0;
-    const hipError_t q = hipEventQuery(L->carve_ready);
-    if (q == hipErrorNotReady) {
-        (void)hipGetLastError();               // "not ready" is an answer, not a failure of a later launch
-        return 0;
-    }
-    if (q != hipSuccess) return infllm_fail(-2, "offload: %s", hipGetErrorString(q));
+    const int ready = carve_copied(L);
+    if (ready <= 0) return ready;
     const infllm_layer_desc &d = L->d;
     const int slot = L->off.slot, n = L->off.count;
     int rc = dma_wait_slot(L, slot, "offload");                                  // an older copy out of the same slot
@@ -324,6 +368,8 @@ int issue_offload(Layer *L, hipStream_t cs) {
     const infllm_layer_desc &d = L->d;
     const int64_t unit_all = (int64_t)d.B * 2 * d.Hkv * d.block_size * kD;        // one unit, all batch rows
     const bf16_t *stage = (const bf16_t *)d.d_carve_stage + (int64_t)L->off.slot * d.max_carve * unit_all;
+    const int erc = carve_event(L);
+    if (erc) return erc;
     HIP_OK(hipStreamWaitEvent(cs, L->carve_ready, 0), "offload: wait carve");
     const int n = L->off.count;
     for (int i = 0; i < n;) {                   // one copy per run of units that are contiguous on the host
@@ -458,7 +504,8 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
                 // (waited for just below), or the host waits for the stream copy
                 int orc = 0;
                 if (L->efetch_ok && L->dma_ok) {
-                    HIP_OK(hipEventSynchronize(L->carve_ready), "fetch: wait gathers");
+                    orc = carve_wait(L);
+                    if (orc) return orc;
                     orc = issue_offload_dma(L);
                     if (orc < 0) return orc;
                 }
@@ -881,10 +928,12 @@ extern "C" int infllm_layer_wait_topk(void *layer) {
         if (*flag == L->topk_seq) {
             std::atomic_thread_fence(std::memory_order_acquire);
             L->topk_pending = false;
+            L->seen_seq = L->topk_seq;
             return 0;
         }
         HIP_OK(hipStreamSynchronize(L->topk_stream), "layer_wait_topk");        // no event was recorded in this mode
         L->topk_pending = false;
+        L->seen_seq = L->topk_seq;
         return 0;
     }
     HIP_OK(hipEventSynchronize(L->topk_done), "layer_wait_topk");
@@ -1246,7 +1295,10 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         rc = infllm_attn_stage(&at, stream);
         timer_end(L, 1, ti, st);
         if (rc) return rc;
-        if (side || L->efetch_ok) {          // the next fetch (copy stream or DMA engines) must not overtake these reads
+        // The next fetch (copy stream or DMA engines) must not overtake these reads.  While guesses are being settled
+        // no event is needed for that: a fetch ahead never writes a slot of the selection in use, and a fetch behind
+        // a selection is issued by a host that has read that selection, which the stream produced after this stage.
+        if ((side || L->efetch_ok) && !L->guessing) {
             HIP_OK(hipEventRecord(L->global_done, st), "block_back: event");
             L->has_global = true;
         }
@@ -1288,6 +1340,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
 
     // ---- 4. what the next block's retrieval waits for: scores of the tokens that leave the ring now,
     //         init peeling, representatives of the new units
+    bool carved = false;
+    L->main_stream = st;
     const int64_t new_cursor = a->cursor + a->init_take + (int64_t)a->n_carve * bs;
     const int64_t urgent_hi = new_cursor < b1 ? new_cursor : b1;
     // While the fetches run ahead of the selection nothing waits for this block's selection at once, and the split
@@ -1322,7 +1376,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
             // the host gets through this wait at once and the engine can take them; else the copy stream does
             int drc = 0;
             if (L->dma_ok) {
-                HIP_OK(hipEventSynchronize(L->carve_ready), "block_back: carve event");
+                drc = carve_wait(L);
+                if (drc) return drc;
                 drc = issue_offload_dma(L);
                 if (drc < 0) return drc;
             }
@@ -1342,7 +1397,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
                                     a->d_rep_out, a->rep_sb, a->rep_su, a->d_repr_idx, d.d_ring_v, stage, stage + unit_elems, slot_elems,
                                     unit_all, (int64_t)bs * kD, stream);
         if (rc) return rc;
-        HIP_OK(hipEventRecord(L->carve_ready, st), "block_back: event");
+        carved = true;
+        L->off.after_seq = 0;
+        L->off.has_event = false;
         L->off.pending = true;
         L->off.slot = slot;
         L->off.first_unit = a->n_units;
@@ -1351,6 +1408,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         L->copy_stream = cs;
     }
     // ---- 5. the next block's retrieval (its prologue ran in block_front)
+    const int32_t seq_before = L->topk_seq;
     L->topk_pending = false;
     const int n_units_next = a->n_units + a->n_carve;
     if (L->prepared && n_units_next > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL)) {
@@ -1371,6 +1429,15 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         }
     }
     L->cand_units = -1;
+    if (carved) {
+        // An event record costs the stream 2-3 us.  When a selection kernel that publishes a sequence number follows
+        // the copy into staging, that number tells the host as much; otherwise the event does.
+        if (L->dma_ok && L->topk_seq != seq_before) L->off.after_seq = L->topk_seq;
+        else {
+            rc = carve_event(L);
+            if (rc) return rc;
+        }
+    }
     // ---- 5b. the block's output rows
     if (!one_pass) {
         rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl,
