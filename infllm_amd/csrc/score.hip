@@ -30,8 +30,15 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
     const int G = a.H / a.Hkv;
-    const int b = blockIdx.y / a.H, h = blockIdx.y % a.H, g = h / G;
-    const int64_t jg = (a.j_lo / kWaveKeys + (int64_t)blockIdx.x * 4) * kWaveKeys;   // first key of the workgroup
+    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H, g = h / G;
+    // Workgroups are dispatched x fastest: all heads of one key tile, then the next tile.  The two tiles at either end
+    // of a masked key range see only part of the queries and finish early, so they go last: when the grid is a little
+    // more than what the chip holds at once, the workgroups that start late are then the short ones.
+    const int n_tiles = gridDim.y, slot = blockIdx.y;
+    int tile = slot;
+    if (n_tiles >= 6 && a.mask != INFLLM_MASK_NONE)
+        tile = slot < n_tiles - 4 ? slot + 2 : slot == n_tiles - 4 ? 1 : slot == n_tiles - 3 ? n_tiles - 2 : slot == n_tiles - 2 ? 0 : n_tiles - 1;
+    const int64_t jg = (a.j_lo / kWaveKeys + (int64_t)tile * 4) * kWaveKeys;         // first key of the workgroup
     const int64_t j0 = jg + (int64_t)wave * kWaveKeys;                               // first key of this wave
     const float scale = a.softmax_scale * 1.4426950408889634f;
 
@@ -264,6 +271,8 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
     INFLLM_REQUIRE((a->q_sl % 8 | a->q_sh % 8 | a->q_sb % 8 | a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8) == 0,
                    "local_score: strides must be multiples of 8");
     if (a->j_hi <= a->j_lo) return 0;
+    INFLLM_REQUIRE(a->j_hi - a->j_lo <= (int64_t)65000 * 256, "local_score: key range of %lld rows exceeds one launch",
+                   (long long)(a->j_hi - a->j_lo));
     auto lds_bytes = [](int qs) { return (size_t)(2 * qs * kQPad * sizeof(bf16_t) + 2 * qs * sizeof(float)); };
     static bool lds_set = false;                       // dynamic LDS above 64 KiB must be enabled once per kernel
     if (!lds_set) {
@@ -277,11 +286,11 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
     }
     if (a->j_hi - a->j_lo > 1024) {
         const int64_t tiles = (a->j_hi - 1) / 64 - a->j_lo / 64 + 1;
-        hipLaunchKernelGGL((local_score_kernel<2, 128>), dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), lds_bytes(128),
+        hipLaunchKernelGGL((local_score_kernel<2, 128>), dim3(a->B * a->H, (unsigned)((tiles + 3) / 4)), dim3(256), lds_bytes(128),
                            (hipStream_t)stream, *a);
     } else {
         const int64_t tiles = (a->j_hi - 1) / 32 - a->j_lo / 32 + 1;
-        hipLaunchKernelGGL((local_score_kernel<1, 128>), dim3((unsigned)((tiles + 3) / 4), a->B * a->H), dim3(256), lds_bytes(128),
+        hipLaunchKernelGGL((local_score_kernel<1, 128>), dim3(a->B * a->H, (unsigned)((tiles + 3) / 4)), dim3(256), lds_bytes(128),
                            (hipStream_t)stream, *a);
     }
     INFLLM_CHECK_LAUNCH("local_score");
