@@ -64,6 +64,67 @@ def test_cache_policy_equals_oracle_model(strategy):
         assert sorted(list(pol.slot_of.values()) + pol.free) == list(range(6))
 
 
+@pytest.mark.parametrize("strategy", ["lru", "fifo"])
+def test_trying_a_selection_out_on_a_copy_leaves_the_policy_as_the_oracle_model_has_it(strategy):
+    """The protocol of the fetch ahead of the selection, on the host alone: a guessed selection is applied to a clone
+    (infllm_cache_clone / _copy); when the real selection equals the guess the clone becomes the state, otherwise the
+    real selection is applied to the untouched state with the guess's slots as wishes (infllm_cache_touch_hinted).
+    Either way misses, evictions and residency follow the oracle's model, every unit sits in a slot of its own, a
+    wish is granted exactly when the slot is free after the evictions, and a unit whose wish was granted keeps the
+    slot the guess gave it."""
+    import ctypes
+    lib = _lib.load()
+    rng = random.Random(11)
+    cap, k = 7, 3
+    pol, model = CachePolicy(cap, strategy, None), UnitCacheModel(cap, strategy, None)
+    shadow = lib.infllm_cache_clone(pol.handle)
+    assert shadow
+    I = ctypes.c_int32
+    n_units, confirmed, refuted, granted_total = 4, 0, 0, 0
+    try:
+        for step in range(400):
+            n_units += rng.randint(0, 2)
+            guess = sorted(rng.sample(range(n_units), k))
+            real = guess
+            if rng.random() < 0.4:                       # as in the stream: a fresh unit displaces one of the guess
+                others = [u for u in range(n_units) if u not in guess]
+                real = sorted(rng.sample(guess, k - 1) + [rng.choice(others)])
+            before = dict(pol.slot_of)
+            assert lib.infllm_cache_copy(shadow, pol.handle) == 0
+            g_slots, g_mu, g_ms, g_ev, g_nev = (I * k)(), (I * k)(), (I * k)(), (I * cap)(), I(0)
+            g_miss = lib.infllm_cache_touch(shadow, (I * k)(*guess), k, g_slots, g_mu, g_ms, g_ev, ctypes.byref(g_nev))
+            assert g_miss >= 0 and pol.slot_of == before                  # the guess has not touched the real state
+            for u in before:
+                assert lib.infllm_cache_slot_of(pol.handle, u) == before[u]
+            assert lib.infllm_cache_slot_of(pol.handle, n_units + 5) == -1
+            model.touch(real)
+            want = model.events[-1]
+            if real == guess:
+                confirmed += 1
+                assert lib.infllm_cache_copy(pol.handle, shadow) == 0
+                assert sorted(g_mu[:g_miss]) == want["misses"] and list(g_ev[:g_nev.value]) == want["evicted"]
+            else:
+                refuted += 1
+                slots, mu, ms, ev, nev = (I * k)(), (I * k)(), (I * k)(), (I * cap)(), I(0)
+                n_miss = lib.infllm_cache_touch_hinted(pol.handle, (I * k)(*real), k, slots, mu, ms, ev, ctypes.byref(nev),
+                                                       g_mu, g_ms, g_miss)
+                assert sorted(mu[:n_miss]) == want["misses"] and list(ev[:nev.value]) == want["evicted"]
+                hint = dict(zip(g_mu[:g_miss], g_ms[:g_miss]))
+                freed = {before[u] for u in want["evicted"]}
+                free_then = (set(range(cap)) - set(before.values())) | freed
+                for u, sl in zip(mu[:n_miss], ms[:n_miss]):
+                    if u in hint and hint[u] in free_then:
+                        assert sl == hint[u]
+                        granted_total += 1
+            assert pol.cached == model.cached
+            assert len(set(pol.slot_of.values())) == len(pol.slot_of) and set(pol.slot_of) == set(pol.cached)
+    finally:
+        lib.infllm_cache_destroy(shadow)
+    assert confirmed > 50 and refuted > 50 and granted_total > 20
+    other = CachePolicy(cap + 1, strategy, None)
+    assert lib.infllm_cache_copy(other.handle, pol.handle) != 0          # different capacity: refused
+
+
 def test_cache_policy_lru_s_equals_oracle_model():
     rng = random.Random(6)
     pol, model = CachePolicy(5, "lru-s", 0.9), UnitCacheModel(5, "lru-s", 0.9)
