@@ -6,6 +6,8 @@
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <utility>
 #include <vector>
 
 #include <hsa/hsa.h>
@@ -61,6 +63,7 @@ struct Layer {
     std::vector<uint32_t> efetch_engines;
     hsa_signal_t efetch_sig{}, efetch_flag_sig{};
     uint32_t *d_efetch_flag = nullptr, *h_efetch_val = nullptr;
+    int efetch_dev = 0;
     uint32_t efetch_seq = 0;
     bool efetch_wait = false;
     int cur_n = 0;                                     // queries of the block in flight
@@ -406,6 +409,40 @@ int efetch_wait_signal(hsa_signal_t sig, const char *what) {
     return 0;
 }
 
+// Flag words in signal memory are never given back to the runtime: memory of that kind that a kernel has read (the
+// stream's wait is a kernel) is best not freed while the process lives, so a layer that goes away leaves its word
+// to the next one on the same device.
+struct FlagPool {
+    std::mutex mu;
+    std::vector<std::pair<int, uint32_t *>> spare;          // (device, word)
+};
+FlagPool &flag_pool() {
+    static FlagPool *p = new FlagPool();                     // outlives static destruction order
+    return *p;
+}
+uint32_t *flag_take(int dev) {
+    {
+        std::lock_guard<std::mutex> g(flag_pool().mu);
+        auto &v = flag_pool().spare;
+        for (size_t i = 0; i < v.size(); ++i)
+            if (v[i].first == dev) {
+                uint32_t *w = v[i].second;
+                v.erase(v.begin() + i);
+                return w;
+            }
+    }
+    uint32_t *w = nullptr;
+    if (hipExtMallocWithFlags((void **)&w, 8, hipMallocSignalMemory) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return w;
+}
+void flag_give(int dev, uint32_t *w) {
+    std::lock_guard<std::mutex> g(flag_pool().mu);
+    flag_pool().spare.emplace_back(dev, w);
+}
+
 // set the engine fetch up for this layer; on any failure the kernel fetch stays the only path
 void efetch_setup(Layer *L) {
     const char *off = getenv("INFLLM_NO_DMA_FETCH");
@@ -420,8 +457,8 @@ void efetch_setup(Layer *L) {
     for (int b = 0; b < 32 && (int)L->efetch_engines.size() < kEfetchEngines; ++b)
         if (mask & (1u << b)) L->efetch_engines.push_back(1u << b);
     if (L->efetch_engines.size() < 2) return;
-    if (hipExtMallocWithFlags((void **)&L->d_efetch_flag, 8, hipMallocSignalMemory) != hipSuccess ||
-        hipMemset(L->d_efetch_flag, 0, 8) != hipSuccess || hipHostMalloc((void **)&L->h_efetch_val, kEfetchVals * sizeof(uint32_t)) != hipSuccess ||
+    L->efetch_dev = dev;
+    if (!(L->d_efetch_flag = flag_take(dev)) || hipHostMalloc((void **)&L->h_efetch_val, kEfetchVals * sizeof(uint32_t)) != hipSuccess ||
         hsa_signal_create(0, 0, nullptr, &L->efetch_sig) != HSA_STATUS_SUCCESS ||
         hsa_signal_create(0, 0, nullptr, &L->efetch_flag_sig) != HSA_STATUS_SUCCESS) {
         (void)hipGetLastError();
@@ -666,7 +703,7 @@ extern "C" int infllm_layer_destroy(void *layer) {
         (void)efetch_wait_signal(L->efetch_flag_sig, "layer_destroy");
         (void)hsa_signal_destroy(L->efetch_flag_sig);
     }
-    if (L->d_efetch_flag) (void)hipFree(L->d_efetch_flag);
+    if (L->d_efetch_flag) flag_give(L->efetch_dev, L->d_efetch_flag);
     if (L->h_efetch_val) (void)hipHostFree(L->h_efetch_val);
     delete L;
     return 0;
