@@ -16,8 +16,10 @@ stream positions and device-resident rings instead of torch.cat/trim:
   needs the merged log-sum-exp;
 * memory units live in pinned host memory (always) and in a slab of
   ``max_cached_block`` device slots managed by the reference's lru / lru-s
-  policy (plus fifo; native, infllm_cache_*); the misses of a block are read
-  from the pinned pages by one kernel on a side stream.
+  policy (plus fifo; native, infllm_cache_*); the misses of a block are moved
+  by the DMA engines (short blocks: read from the pinned pages by one kernel
+  on a side stream), for lru / fifo starting from the selection's candidates a
+  block ahead of the selection itself (``fetch_ahead``).
 
 This module keeps the state machine, in absolute positions
 (context_manager.py:614-679 restated): ``cursor`` is the first token not yet
@@ -25,7 +27,8 @@ carved, tokens [0, init_len) are the attention sinks, unit u is tokens
 [n_init + u*bs, n_init + (u+1)*bs).  The device work of one execution block is
 issued by three native calls: infllm_block_front, infllm_block_select (the one
 host wait, for the retrieved unit ids, which overlaps the local stage; then
-cache policy and fetch) and infllm_block_back.
+cache policy and fetch) and infllm_block_back, plus infllm_block_prefetch for
+the next block.
 """
 import ctypes
 

@@ -1,7 +1,10 @@
-// One execution block of the streaming path in two calls
-// (inf_llm/attention/context_manager.py:474-545, 614-679): the launches of a block are
-// issued natively, back to back, so that the host interpreter is not on the GPU's
-// critical path.  Decisions (which units are cached, what gets carved) stay with the caller.
+// One execution block of the streaming path in a few native calls
+// (inf_llm/attention/context_manager.py:474-545, 614-679): front (local stage, the next block's prologue and
+// candidates), select (selection -> residency policy -> fetch), back (global stage, merge, scores, new units) and,
+// optionally, prefetch (the next block's fetch from its candidates, settled by the next select).  The launches of a
+// block are issued back to back so that the host interpreter is not on the GPU's critical path; missed units and
+// carved units travel through the DMA engines (ROCr), ordered by the host and by a flag the stream waits on.
+// What is carved when stays with the caller; the residency policy is infllm_cache_* (cache.hip).
 #include <atomic>
 #include <chrono>
 #include <cstdlib>
