@@ -30,7 +30,10 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
     const int G = a.H / a.Hkv;
-    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H, g = h / G;
+    // blockIdx.x walks the kv heads first, then the query heads of a group: workgroups go to the 8 XCDs round-robin by
+    // linear id, so with 8 (16, ...) kv heads the query heads that share a K tile sit behind the same L2 and that tile
+    // leaves HBM once instead of once per query head
+    const int b = blockIdx.x / a.H, hx = blockIdx.x % a.H, g = hx % a.Hkv, h = g * G + hx / a.Hkv;
     // Workgroups are dispatched x fastest: all heads of one key tile, then the next tile.  The two tiles at either end
     // of a masked key range see only part of the queries and finish early, so they go last: when the grid is a little
     // more than what the chip holds at once, the workgroups that start late are then the short ones.
