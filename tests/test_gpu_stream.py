@@ -253,6 +253,36 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
     assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
 
 
+def test_stage_timers_sample_the_launches_they_are_asked_for():
+    """infllm_layer_timing / infllm_layer_read_timing (what bench.py's roofline figure is made of): every stride-th
+    launch of the local stage, of the global stage and of the stream's wait for the fetch is bracketed by events; the
+    records carry the launch's sizes and a positive duration, and timing changes no result."""
+    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
+    T = 1600
+    q, k, v = _stream(T, 8, 2, 23)
+    kw = dict(SMALL, max_cached_block=5, async_global_stream=True)
+    plain, _ = _run_gpu(q, k, v, [T], 1e4, **kw)
+    rope = RotaryEmbeddingESM(D, base=1e4, device="cuda")
+    cm = ContextManager(rope, kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"], kw["topk"],
+                        kw["exc_block_size"], None, False, kw["repr_topk"], "lru", None, True, False, False, False)
+    cm.enable_timing(64, 2)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    out = cm.append(qd, kd, vd, qd, kd, vd)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), plain)
+    n_blocks = T // kw["exc_block_size"]
+    local, glob, wait = cm.read_timing(0), cm.read_timing(1), cm.read_timing(2)
+    assert len(local) == (n_blocks + 1) // 2                       # every second launch of n_blocks
+    assert 0 < len(glob) <= len(local) and 0 < len(wait) <= len(glob)
+    for ms, nq, nk in local + glob + wait:
+        assert 0.0 < ms < 50.0 and nq == kw["exc_block_size"]
+    assert max(nk for _, _, nk in local) == kw["n_local"] + kw["exc_block_size"]
+    import ctypes
+    from infllm_amd._lib import InfLLMHipError, check
+    with pytest.raises(InfLLMHipError):                            # there is no fourth timer
+        check(cm._lib.infllm_layer_read_timing(cm._layer, 3, (ctypes.c_float * 4)(), None, None, 4), "infllm_layer_read_timing")
+
+
 def test_selection_in_separate_steps_equals_the_fused_call(monkeypatch):
     """infllm_layer_wait_topk + infllm_cache_touch + infllm_block_fetch, driven from the host, against
     infllm_block_select: same outputs, same residency events, for every policy."""
