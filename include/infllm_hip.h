@@ -458,8 +458,9 @@ int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, 
  * already takes the slot it was moved to where that slot is free (infllm_cache_touch_hinted), so that only the other
  * misses are fetched, together with the residents whose slots the guess overwrote.  The hit / miss / eviction
  * sequence is therefore the reference's either way; which slot a unit occupies may differ from a run without guesses.
- * No guess is made (return 0) when no candidates are pending, or when the policy would evict a unit of the
- * selection whose global stage may still be running.  Valid only for policies whose state does not change between
+ * No guess is made (return 0) when no candidates are pending, when the policy would evict a unit of the
+ * selection whose global stage may still be running, or when the DMA engines are not in use (beside the block's
+ * own kernels the fetch kernel costs more than the shorter chain gains; INFLLM_FETCH_AHEAD_ALWAYS=1 guesses anyway).  Valid only for policies whose state does not change between
  * this call and the selection (lru, fifo: the lru-s scores arrive with the block's attention mass).
  * `a` as for infllm_block_select (h_selected, wait_topk and the output lists are not used).  Returns the number of
  * units whose fetch was started (>= 0) or an error (< 0).  A guess still open at infllm_layer_flush is undone there. */
