@@ -328,6 +328,42 @@ def test_state_export_and_injection_resume_the_stream_exactly():
     assert cm_b.length == T0 + T1 == cm1.length and cm_b.num_global_block == cm1.num_global_block
 
 
+def test_full_size_stream_is_the_same_with_and_without_the_fetch_ahead(monkeypatch):
+    """BASELINE config 2 at full size (131,072 tokens, Mistral geometry, mixture keys, 32 slots for 16 selected units of
+    512 KiB each): the stream with the fetch ahead of the selection (DMA engines, about four of five guesses confirmed,
+    the others repaired) against the stream without it - outputs bit for bit, hit / miss / eviction counts, the eviction
+    sequence, the final residency, and the units' pinned host copies against the input."""
+    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
+    H, Hkv, T, exc, n_local, n_init, bs, topk = 32, 8, 131072, 512, 4096, 128, 128, 16
+    q, k, v = _stream(T, H, Hkv, seed=101)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+
+    def run(ahead):
+        monkeypatch.setattr(ContextManager, "fetch_ahead", ahead)
+        rope = RotaryEmbeddingESM(D, base=1e6, device="cuda")
+        cm = ContextManager(rope, n_init, n_local, bs, 32, topk, exc, None, False, 4, "lru", None, True)
+        outs = []
+        for i, st in enumerate(range(0, T, 8192)):
+            sl = slice(st, st + 8192)
+            if i == 1:
+                cm.policy[0].evicted_log = []
+            outs.append(cm.append(qd[:, :, sl], kd[:, :, sl], vd[:, :, sl], qd[:, :, sl], kd[:, :, sl], vd[:, :, sl]).cpu())
+        torch.cuda.synchronize()
+        return torch.cat(outs, dim=2), cm
+
+    plain, cm0 = run(False)
+    ahead, cm1 = run(True)
+    issued, confirmed = cm1.prefetch_stats()
+    assert cm0.prefetch_stats() == (0, 0) and issued > 200 and issued // 2 < confirmed < issued
+    assert torch.equal(plain, ahead)
+    assert cm0.stats == cm1.stats and cm0.stats["misses"] > 3000
+    assert cm0.policy[0].evicted_log == cm1.policy[0].evicted_log and cm0.policy[0].cached == cm1.policy[0].cached
+    assert cm1.num_global_block == (T - n_init - n_local) // bs
+    for u in range(0, cm1.num_global_block, 41):
+        lo, hu = n_init + u * bs, cm1.host_unit(u)
+        assert torch.equal(hu[0, 0], k[0, :, lo:lo + bs]) and torch.equal(hu[0, 1], v[0, :, lo:lo + bs]), u
+
+
 def test_full_size_stream_one_block_against_the_oracle_from_exported_state():
     """BASELINE config 2 at full size (131,072 tokens, Mistral geometry, mixture keys).  The whole stream is too long
     for the CPU oracle, so: closed forms for the state, and ONE execution block (the last) recomputed on the CPU
