@@ -170,3 +170,12 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "absent.so"))
     with pytest.raises(_lib.InfLLMHipError):
         _lib.load()
+
+
+def test_bench_refuses_more_than_one_gpu_with_a_message():
+    """bench.py --gpus N with N above 1 exits with a message that says why (no GPU is touched on that path)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    p = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "ONE GPU" in p.stderr and p.stdout.strip() == ""
