@@ -1496,8 +1496,15 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
     if (L->ahead.active) {                      // a guess nobody settled: put back what it overwrote
         L->ahead.active = false;
         hipStream_t cs = (hipStream_t)copy_stream;
-        const int rrc = ahead_repair(L, nullptr, 0, nullptr, nullptr, nullptr, nullptr, cs, cs);
+        int rrc = ahead_repair(L, nullptr, 0, nullptr, nullptr, nullptr, nullptr, cs, cs);
         if (rrc) return rrc;
+        // nothing later is ordered behind this repair by itself: finish it here (it is not a path a stream takes)
+        if (L->efetch_ok) {
+            rrc = efetch_wait_signal(L->efetch_flag_sig, "layer_flush");
+            if (rrc) return rrc;
+        }
+        HIP_OK(hipStreamSynchronize(cs), "layer_flush: repair");
+        L->fetch_wait = L->efetch_wait = false;
     }
     if (L->off.pending) {
         int drc = issue_offload_dma(L);
