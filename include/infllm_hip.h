@@ -471,7 +471,8 @@ int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed
 /* Event timing of the two attention stages (for benchmarks): enable with a record
  * capacity and a stride (every stride-th launch of each stage is bracketed by two events; an event pair
  * costs the stream several microseconds, so a throughput run samples), read back (which: 0 local stage,
- * 1 global stage, 2 the main stream's wait for the fetch in infllm_block_back) after a device sync.
+ * 1 global stage, 2 the main stream's wait for the fetch in infllm_block_back); the read waits for launches
+ * that are still running.
  * ms[i] is the launch-to-finish time of one stage launch, n_queries[i] its block size,
  * n_keys[i] the key rows its source held. */
 int infllm_layer_timing(void *layer, int32_t capacity, int32_t stride);

@@ -738,6 +738,7 @@ extern "C" int infllm_layer_read_timing(void *layer, int32_t which, float *ms, i
     StageTimer &t = L->timer[which];
     int n = t.used < capacity ? t.used : capacity;
     for (int i = 0; i < n; ++i) {
+        HIP_OK(hipEventSynchronize(t.ev[2 * i + 1]), "layer_read_timing");            // no wait when the launch has finished
         HIP_OK(hipEventElapsedTime(&ms[i], t.ev[2 * i], t.ev[2 * i + 1]), "layer_read_timing");
         if (n_queries) n_queries[i] = t.n_queries[i];
         if (n_keys) n_keys[i] = t.n_keys[i];
