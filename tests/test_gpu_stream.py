@@ -337,6 +337,8 @@ def test_full_size_stream_is_the_same_with_and_without_the_fetch_ahead(monkeypat
     H, Hkv, T, exc, n_local, n_init, bs, topk = 32, 8, 131072, 512, 4096, 128, 128, 16
     q, k, v = _stream(T, H, Hkv, seed=101)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    monkeypatch.delenv("INFLLM_NO_DMA_FETCH", raising=False)      # the engines where the process can use them ...
+    monkeypatch.setenv("INFLLM_FETCH_AHEAD_ALWAYS", "1")          # ... and guesses also where it cannot
 
     def run(ahead):
         monkeypatch.setattr(ContextManager, "fetch_ahead", ahead)
