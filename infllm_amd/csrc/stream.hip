@@ -1382,6 +1382,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     // ---- 4. what the next block's retrieval waits for: scores of the tokens that leave the ring now,
     //         init peeling, representatives of the new units
     bool carved = false;
+    int carved_slot = 0;
     L->main_stream = st;
     const int64_t new_cursor = a->cursor + a->init_take + (int64_t)a->n_carve * bs;
     const int64_t urgent_hi = new_cursor < b1 ? new_cursor : b1;
@@ -1412,9 +1413,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         // (from there they go to pinned host memory, off the critical path)
         INFLLM_REQUIRE(a->d_rep_out && a->h_carve_dst, "block_back: null carve outputs");
         for (int i = 0; i < a->n_carve; ++i) INFLLM_REQUIRE(a->h_carve_dst[i], "block_back: null carve destination");
-        if (L->off.pending) {
-            // the units of an earlier block are still waiting: their copy into staging was queued a whole block ago, so
-            // the host gets through this wait at once and the engine can take them; else the copy stream does
+        if (L->off.pending && d.carve_slots < 2) {      // one staging slot: the earlier units have to leave it first
             int drc = 0;
             if (L->dma_ok) {
                 drc = carve_wait(L);
@@ -1439,14 +1438,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
                                     unit_all, (int64_t)bs * kD, stream);
         if (rc) return rc;
         carved = true;
-        L->off.after_seq = 0;
-        L->off.has_event = false;
-        L->off.pending = true;
-        L->off.slot = slot;
-        L->off.first_unit = a->n_units;
-        L->off.count = a->n_carve;
-        L->off.dst.assign(a->h_carve_dst, a->h_carve_dst + a->n_carve);
-        L->copy_stream = cs;
+        carved_slot = slot;
     }
     // ---- 5. the next block's retrieval (its prologue ran in block_front)
     const int32_t seq_before = L->topk_seq;
@@ -1471,6 +1463,30 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     }
     L->cand_units = -1;
     if (carved) {
+        // host work that the selection just launched does not have to wait for
+        if (L->off.pending) {
+            // the units of an earlier block are still waiting: their copy into staging was queued a whole block ago, so
+            // the host gets through this wait at once and the engine can take them; else the copy stream does
+            int drc = 0;
+            if (L->dma_ok) {
+                drc = carve_wait(L);
+                if (drc) return drc;
+                drc = issue_offload_dma(L);
+                if (drc < 0) return drc;
+            }
+            if (drc == 0) {
+                rc = issue_offload(L, cs);
+                if (rc) return rc;
+            }
+        }
+        L->off.after_seq = 0;
+        L->off.has_event = false;
+        L->off.pending = true;
+        L->off.slot = carved_slot;
+        L->off.first_unit = a->n_units;
+        L->off.count = a->n_carve;
+        L->off.dst.assign(a->h_carve_dst, a->h_carve_dst + a->n_carve);
+        L->copy_stream = cs;
         // An event record costs the stream 2-3 us.  When a selection kernel that publishes a sequence number follows
         // the copy into staging, that number tells the host as much; otherwise the event does.
         if (L->dma_ok && L->topk_seq != seq_before) L->off.after_seq = L->topk_seq;
