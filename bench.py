@@ -76,21 +76,56 @@ def run_stream(q, k, v, chunk, timing=False):
     return cm, out
 
 
-# HBM bytes per launch from hardware counters (FETCH_SIZE, WRITE_SIZE; one profiler run per counter, each scaled by
-# what the counter reads for a 256 MiB elementwise pass: x2.0 and x1.0).  The summaries of those runs sit in
-# profiles/*.hbm_bytes.txt; the figures hold for the default geometry only.
-LOCAL_STAGE_HBM_BYTES = int((20241.0 * 2.0 + 16640.0) * 1024)      # steady-state local stage: 39.5 MiB read + 16.25 MiB written (fp16 partials)
-UNIT_SCORES_HBM_BYTES = int((32860.6 * 2.0 + 64.0) * 1024)         # 8194 x 4096 representatives: 64.2 MiB read
+def counted_traffic(summary, key):
+    """HBM bytes per launch from hardware counters (FETCH_SIZE, WRITE_SIZE; one profiler run per counter, each scaled
+    by what the counter reads for a 256 MiB elementwise pass).  The figure is not measured in this run: it is read from
+    the rocprofv3 summary under profiles/ that derives it, which carries a line `<key> = <bytes>`; None when the
+    summary is not there (the figures hold for the default geometry only)."""
+    import re
+    try:
+        with open(os.path.join(ROOT, "profiles", summary)) as f:
+            m = re.search(r"^%s\s*=\s*(\d+)" % re.escape(key), f.read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
-def decode_workload(args, dev):
-    """BASELINE config 3: 256 single-token steps over a prepared memory of 8192 units (1,048,576 past tokens)
-    with precomputed representatives.  Prints its own JSON line; not the headline metric."""
+def hbm_leg(dev, n_units=8192, tables=8, launches=200):
+    """The HBM half of the metric, measured in this run: unit scoring (context_manager.py:159-163) over n_units
+    representatives of H*D bf16 each, the shape of BASELINE config 3 - N*H*D*2 algorithmic bytes per launch (64 MiB),
+    read once.  The launches rotate over `tables` distinct tables (512 MiB together, more than the 256 MB of last-level
+    cache), so every launch reads from HBM; the figure is the MEAN over all launches, timed with events on the stream
+    the kernel runs on."""
     from infllm_amd import ops
-    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
-    n_units, bs, n_local, n_init, topk = args.decode_units, KNOBS["block_size"], KNOBS["n_local"], KNOBS["n_init"], KNOBS["topk"]
+    C = H * D
+    reps = torch.randn((tables, n_units, C), device=dev, dtype=torch.bfloat16)
+    qbar = torch.randn((C,), device=dev)
+    scores = torch.empty((n_units,), dtype=torch.float32, device=dev)
+    for i in range(2 * tables):
+        ops.score_topk(reps[i % tables], n_units, qbar, 0, scores, None)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(launches):
+        ops.score_topk(reps[i % tables], n_units, qbar, 0, scores, None)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / launches
+    nbytes = n_units * C * 2
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0,
+            "traffic": counted_traffic("unit_scores__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"),
+            "kernel": f"unit_scores_rows_kernel ({n_units} x {C} bf16 representatives = {nbytes / 2 ** 20:.0f} MiB per launch, "
+                      f"{tables} tables in rotation)",
+            "avg_launch_ms": ms, "launches_timed": launches}
+
+
+def make_decode_state(dev, n_units, seed=3):
+    """A prepared memory for the decode shape (BASELINE config 3): n_units units of mixture keys with representatives
+    (the mean of each unit's first repr_topk keys), a full local window and the init tokens.  Returns the state
+    ContextManager.load_state takes, and a function drawing further (q, k, v) tokens from the same generator."""
+    bs, n_local, n_init = KNOBS["block_size"], KNOBS["n_local"], KNOBS["n_init"]
     T0 = n_init + n_units * bs + n_local
-    g = torch.Generator(device=dev).manual_seed(3)
+    g = torch.Generator(device=dev).manual_seed(seed)
     means = torch.randn((HKV, 64, D), generator=g, device=dev)
 
     def mixture_keys(n):
@@ -110,14 +145,27 @@ def decode_workload(args, dev):
     state = dict(length=T0, tail_k=mixture_keys(n_local), tail_v=torch.randn((1, HKV, n_local, D), generator=g, device=dev).bfloat16(),
                  tail_score=None, init_k=mixture_keys(n_init), init_v=torch.randn((1, HKV, n_init, D), generator=g, device=dev).bfloat16(),
                  units=units, reps=reps)
+
+    def tokens(n):
+        q = torch.randn((1, H, n, D), generator=g, device=dev).bfloat16()
+        return q, mixture_keys(n), torch.randn((1, HKV, n, D), generator=g, device=dev).bfloat16()
+
+    return state, tokens
+
+
+def decode_workload(args, dev):
+    """BASELINE config 3: 256 single-token steps over a prepared memory of 8192 units (1,048,576 past tokens)
+    with precomputed representatives.  Prints its own JSON line; not the headline metric."""
+    from infllm_amd import ops
+    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
+    n_units, bs, n_local, n_init, topk = args.decode_units, KNOBS["block_size"], KNOBS["n_local"], KNOBS["n_init"], KNOBS["topk"]
+    state, tokens = make_decode_state(dev, n_units)
     rope = RotaryEmbeddingESM(D, base=ROPE_BASE, device=dev)
     cm = ContextManager(rope, n_init, n_local, bs, KNOBS["max_cached_block"], topk, KNOBS["exc_block_size"], None, True,
                         KNOBS["repr_topk"], "lru", None, True, True).load_state(state)
-    del units, state
+    del state
     steps = args.decode_steps
-    q = torch.randn((1, H, steps + 8, D), generator=g, device=dev).bfloat16()
-    k = mixture_keys(steps + 8)
-    v = torch.randn((1, HKV, steps + 8, D), generator=g, device=dev).bfloat16()
+    q, k, v = tokens(steps + 8)
     for i in range(8):                                      # warm-up steps
         cm.append(q[:, :, i:i + 1], k[:, :, i:i + 1], v[:, :, i:i + 1], q[:, :, i:i + 1], k[:, :, i:i + 1], v[:, :, i:i + 1])
     torch.cuda.synchronize()
@@ -147,7 +195,8 @@ def decode_workload(args, dev):
         "n_gpus": 1, "steps": steps, "ms_per_step": dt / steps * 1e3, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"config 3: {steps} single-token steps, {N} units x {bs} tokens, topk {topk}, n_local {n_local}, "
                                f"max_cached {KNOBS['max_cached_block']}"},
-        "roofline": {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": UNIT_SCORES_HBM_BYTES,
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0,
+                     "traffic": counted_traffic("unit_scores__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"),
                      "kernel": f"unit_scores_kernel ({N} x {H * D} bf16 representatives, {N * H * D * 2 / 2 ** 20:.1f} MiB per retrieval)",
                      "avg_launch_ms": ms},
         "cache": cm.stats}))
@@ -209,21 +258,25 @@ def model_workload(args, dev):
         "layer0_cache": cm.stats, "layer0_units": cm.num_global_block}))
 
 
-def cpu_baseline(tokens, threads):
-    """The fp32 oracle (restating the reference's torch path) on the first `tokens` tokens of the same
-    kind of stream, on the host cores."""
+def cpu_baseline(tokens, threads, seed=1):
+    """BASELINE config 1: the reference's torch path restated (the fp32 oracle; the reference's own files hard-code
+    "cuda") on the host cores - q, k, v i.i.d. N(0,1) from `seed`, fp32, the first `tokens` tokens of the
+    16,384-token stream (all of it by default)."""
     from oracle.rope import RopeOracle
     from oracle.stream import StreamOracle
     torch.set_num_threads(threads)
-    q, k, v = make_stream(tokens, 1, "cpu")
-    q, k, v = q.float(), k.float(), v.float()
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((1, H, tokens, D), generator=g)
+    k = torch.randn((1, HKV, tokens, D), generator=g)
+    v = torch.randn((1, HKV, tokens, D), generator=g)
     ora = StreamOracle(RopeOracle(D, base=ROPE_BASE), KNOBS["n_init"], KNOBS["n_local"], KNOBS["block_size"],
-                       KNOBS["max_cached_block"], KNOBS["topk"], KNOBS["exc_block_size"], repr_topk=KNOBS["repr_topk"])
+                       32, KNOBS["topk"], KNOBS["exc_block_size"], repr_topk=KNOBS["repr_topk"])
     t0 = time.perf_counter()
     ora.append(q, k, v)
     dt = time.perf_counter() - t0
     return dict(value=tokens / dt, unit="tokens/s", cores=threads, kind="port",
-                sample=f"first {tokens} tokens of the same stream shape (config 1 is 16384), fp32 oracle, {dt:.1f} s")
+                sample=f"config 1: {tokens} of 16384 tokens, q/k/v i.i.d. N(0,1) (torch.Generator seed {seed}), fp32, one append() call, "
+                       f"{dt:.1f} s")
 
 
 def main():
@@ -233,7 +286,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--chunk", type=int, default=8192, help="tokens per append() call")
-    ap.add_argument("--cpu-tokens", type=int, default=32768, help="0 disables the CPU baseline")
+    ap.add_argument("--cpu-tokens", type=int, default=16384, help="tokens of config 1 the CPU baseline runs (0 disables it)")
+    ap.add_argument("--no-hbm-leg", action="store_true", help="skip the unit-scoring (HBM roofline) measurement")
     ap.add_argument("--workload", choices=["prefill", "decode", "model"], default="prefill",
                     help="prefill = the headline 128K-token stream (config 2); decode = config 3, model = config 4 "
                          "(each with its own JSON line)")
@@ -315,7 +369,8 @@ def main():
                                + (f", queries favour {args.favour} components per block" if args.favour else ""),
                    "append_chunk": args.chunk},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS, "traffic": LOCAL_STAGE_HBM_BYTES,
+                     "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": counted_traffic("attn_stage__stream32k.hbm_bytes.txt", "local_stage_traffic_bytes"),
                      "kernel": "attn_stage_kernel<false> (local stage, 512 q x 4096 visible keys x 32 heads)",
                      "avg_launch_ms": avg_ms, "launches_timed": len(steady),
                      "global_stage_avg_ms": sum(glob) / max(len(glob), 1)},
@@ -324,8 +379,10 @@ def main():
         # were the selection, and how long the main stream still waited for units (the wait itself costs ~6 us)
         "fetch_ahead": {"guesses": guesses[0], "confirmed": guesses[1], "stream_wait_avg_ms": sum(waits) / max(len(waits), 1)},
     }
+    if not args.no_hbm_leg:
+        res["roofline_hbm"] = hbm_leg(dev)
     if args.cpu_tokens > 0:
-        res["cpu_baseline"] = cpu_baseline(args.cpu_tokens, min(os.cpu_count() or 1, 16))
+        res["cpu_baseline"] = cpu_baseline(min(args.cpu_tokens, 16384), min(os.cpu_count() or 1, 16))
     print(json.dumps(res))
 
 

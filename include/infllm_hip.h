@@ -190,15 +190,17 @@ int infllm_local_score(const infllm_score_args *a, void *stream);
  * Replaces VectorTensor.get_topk and calc_block_topk
  * (context_manager.py:159-163, 366-383).
  *   scores[n] = sum_c reps[n,c] * qbar[c]   (bf16 reps, fp32 qbar, fp32 out)
- *   idx[0..k)  = indices of the k largest scores, ascending index order;
- *                ties at the boundary go to the lower index.
+ *   idx[0..k)  = indices of the k largest scores in descending score order, as torch.topk
+ *                returns them (the residency policy inserts a block's missed units in this
+ *                order, context_manager.py:495-515); equal scores go to the lower index
+ *                first, at the boundary and in the order.
  * reps [N,C] bf16 row stride rep_stride; C = H*128.  k <= 1024.
  */
 int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C,
                       const float *d_qbar, int32_t k,
                       float *d_scores, int32_t *d_idx, void *stream);
 /* The selection over ALL units from two parts (what the stream does between blocks): d_cand[n_cand] are the k best,
- * ids ascending, of units [0, first_new) (infllm_topk over their scores, taken while other work was in flight);
+ * in any order, of units [0, first_new) (infllm_topk over their scores, taken while other work was in flight);
  * this scores the n_new units [first_new, first_new + n_new) (d_scores[first_new ...] = reps . qbar, the same
  * arithmetic as infllm_unit_scores) and ranks them against the candidates in the same launch: d_idx[k] as
  * infllm_topk over all first_new + n_new scores would give (a unit of the overall top-k that is not new is among

@@ -156,8 +156,7 @@ class ContextManager:
         layer, self._layer = getattr(self, "_layer", None), None
         if layer:
             try:
-                torch.cuda.synchronize()
-                _lib.load().infllm_layer_destroy(layer)
+                _lib.load().infllm_layer_destroy(layer)       # waits for this layer's own work, not for the device
             except Exception:
                 pass
 
@@ -170,6 +169,8 @@ class ContextManager:
             raise ValueError(f"the HIP kernels are built for head_dim {HEAD_DIM}, got {D}")
         if self.topk > self.max_cached_block:
             raise ValueError("topk must not exceed max_cached_block")
+        if self.topk > 64:
+            raise ValueError("this build selects at most 64 units per block (topk <= 64)")
         if self.repr_topk > self.block_size:
             raise ValueError("repr_topk must not exceed block_size")
         self.batch_size = self.num_units = B
@@ -440,7 +441,8 @@ class ContextManager:
         if self.cache_strategy == "lru-s" and n_sel:
             self._mass_units = selected
         if self.record_trace:
-            self.trace_blocks.append(dict(b0=b0, b1=b1, selected=[sorted(s) for s in selected], n_units=N, init_len=init_len))
+            self.trace_blocks.append(dict(b0=b0, b1=b1, selected=[sorted(s) for s in selected], order=[list(s) for s in selected],
+                                          n_units=N, init_len=init_len))
             if c:
                 self.trace_units.append((N, c, idx_out))
         stats["blocks"] += 1
@@ -584,12 +586,13 @@ class ContextManager:
     # ------------------------------------------------------- state in / out
     # The reference keeps its state only in the live object (context_manager.py:292-363); these two
     # methods let a harness start from a prepared memory (e.g. 8192 units with representatives) or resume.
-    def export_state(self):
-        """Snapshot after an append(): everything a fresh ContextManager needs to continue the stream."""
+    def export_state(self, with_units=True):
+        """Snapshot after an append(): everything a fresh ContextManager needs to continue the stream.
+        with_units=False leaves the units out (4 GiB at a million tokens): host_unit(u) still reads them in place."""
         torch.cuda.synchronize()
         T, cur, cap = self.length, self.cursor, self.ring_cap
         rows = torch.arange(cur, T, device=self.device) % cap
-        units = [self.host_unit(u).clone() for u in range(self.num_global_block)]
+        units = [self.host_unit(u).clone() for u in range(self.num_global_block)] if with_units else []
         return dict(length=T, n_units=self.num_global_block, init_len=self.init_len,
                     tail_k=self.ring_k_raw[:, :, rows].clone(), tail_v=self.ring_v[:, :, rows].clone(),
                     tail_score=self.ring_score[:, :, rows].clone(),

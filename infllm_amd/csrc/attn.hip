@@ -3,9 +3,9 @@
 // (inf_llm/attention/dot_production_attention/torch_impl.py:15-96).
 //
 // Work split.  For one kv head the query heads that share it (GQA) are laid out as
-// "wave tasks" (query tile of 32 rows, head-in-group); a workgroup of 4 waves takes 4
+// "wave tasks" (query tile of 32 rows, head-in-group); a workgroup of 8 waves takes 8
 // consecutive tasks ordered tile-major/head-minor, so with 4 query heads per kv head
-// the 4 waves hold the same 32 queries of the 4 heads and walk the same keys.
+// the 8 waves hold two tiles of 32 queries of the 4 heads and walk the same keys.
 // K and V tiles of 64 keys are staged through LDS once per workgroup.
 //
 // MFMA formulation (v_mfma_f32_32x32x16_bf16), all operands read as 16-byte vectors:
@@ -135,15 +135,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     const int b = (int)fdiv(by, geo.hkv), g = by - b * a.Hkv;
     const int split = bz;
     const int n_tasks = geo.n_tasks;
-#ifdef INFLLM_PHASES
-    long long *ph = (long long *)a.d_lse_part + 1024 * 1024;     // debug build only: stamps beyond the lse partials
-    int ph_n = 0;
-    const bool ph_on = bx == 3 && by == 1 && bz == 1 && tid == 0;
-#define PH_STAMP() do { if (ph_on && ph_n < 512) ph[ph_n++] = clock64(); } while (0)
-#else
-#define PH_STAMP() do { } while (0)
-#endif
-    PH_STAMP();
 
     // ---- this wave's task and the tiles it needs
     const int task = bx * kWaves + wave;
@@ -363,9 +354,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                     s[ks][r] = vis ? s[ks][r] : -INFINITY;
                 }
         }
-#ifdef INFLLM_DBG_STAMP_INNER
-        PH_STAMP();
-#endif
         float tmax = -INFINITY;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
@@ -387,7 +375,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             m_run = m_new;
             neg_ms = (m_run == -INFINITY) ? 0.f : -m_run * scale;
         }
-        float psum = 0.f;
+        // The row sum is taken over the probabilities AS ROUNDED to bf16, the values the second MFMA multiplies: the
+        // output is then an exact convex combination of value rows (a row on which one key carries nearly all the
+        // weight comes out as that value row, whatever the rounding of its weight), and a pair costs one dot
+        // instruction instead of two additions.
+        float psum[2] = {0.f, 0.f};
         uint32_t pw[2][8];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks)
@@ -395,13 +387,10 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
             for (int r = 0; r < 16; r += 2) {
                 float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r], scale, neg_ms));
                 float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r + 1], scale, neg_ms));
-                psum += p0 + p1;
                 pw[ks][r >> 1] = pack_bf16x2(p0, p1);
+                psum[ks] = sum_bf16x2(pw[ks][r >> 1], psum[ks]);
             }
-        l_run += psum;
-#ifdef INFLLM_DBG_STAMP_INNER
-        PH_STAMP();
-#endif
+        l_run += psum[0] + psum[1];
         {
             // 4 steps of 16 keys, 4 MFMAs each; the V^T operands of a step are requested from LDS while the
             // MFMAs of the previous step run
@@ -459,19 +448,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     __syncthreads();
     for (int t = g_t0; t < g_t1; t += 2) {
         const int buf = (t - g_t0) & 3;                          // 0 or 2
-        PH_STAMP();
         if (t + 2 < g_t1) load_tile(t + 2, buf ^ 2);
         if (t + 3 < g_t1) load_tile(t + 3, (buf ^ 2) + 1);
-        PH_STAMP();
         if (t >= w_t0 && t < w_t1) tile_math(buf, t);          // wave-uniform; barriers stay outside
         if (t + 1 < g_t1 && t + 1 >= w_t0 && t + 1 < w_t1) tile_math(buf + 1, t + 1);
-        PH_STAMP();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        PH_STAMP();
         __syncthreads();
     }
 
-    PH_STAMP();
     // ---- epilogue: normalised partial + base-2 log-sum-exp.  The accumulators hold O^T (a lane owns a query and
     //      scattered 4-float pieces of its row); they go through this wave's 16 KB of the now idle tile buffers so
     //      that every store instruction writes two whole 512-byte rows.
@@ -507,7 +491,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     }
     if (qi >= a.Lq) return;
     if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run * scale + log2f(l_tot) : -INFINITY;
-    PH_STAMP();
 }
 
 // one thread per (row, 8 dims): P fp16 partials -> bf16 output row + final lse

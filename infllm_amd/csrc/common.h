@@ -53,6 +53,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     f32x2_t v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
+// acc + lo + hi of a packed bf16 pair, exactly (v_dot2c_f32_bf16 against a pair of ones)
+__device__ __forceinline__ float sum_bf16x2(uint32_t pair, float acc) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), acc, false);
+}
 __device__ __forceinline__ float wave_xor32(float x) {
     return __shfl_xor(x, 32, 64);
 }

@@ -12,8 +12,9 @@ struct Rot8 {
     u32x4 lo, hi;
 };
 
-// rotate 8 pairs (lo[i], hi[i]) by (c[i], s[i]); fp32 math, one rounding to bf16
-__device__ __forceinline__ Rot8 rotate8(u32x4 xlo, u32x4 xhi, const float2 *cs) {
+// rotate 8 pairs (lo[i], hi[i]) by (c[i], s[i]); fp32 math, one rounding to bf16.  `raw` (optional) receives the 16
+// rotated values before that rounding: lo pairs first, then hi pairs.
+__device__ __forceinline__ Rot8 rotate8(u32x4 xlo, u32x4 xhi, const float2 *cs, float *raw = nullptr) {
     Rot8 r;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -21,39 +22,38 @@ __device__ __forceinline__ Rot8 rotate8(u32x4 xlo, u32x4 xhi, const float2 *cs) 
         float b0 = bf16_bits_to_f32(xhi[w] & 0xffffu), b1 = bf16_bits_to_f32(xhi[w] >> 16);
         float2 c0 = cs[2 * w], c1 = cs[2 * w + 1];
         // x*cos + rotate_half(x)*sin, rotate_half = (-hi, lo)
-        r.lo[w] = pack_bf16x2(a0 * c0.x - b0 * c0.y, a1 * c1.x - b1 * c1.y);
-        r.hi[w] = pack_bf16x2(b0 * c0.x + a0 * c0.y, b1 * c1.x + a1 * c1.y);
+        const float l0 = a0 * c0.x - b0 * c0.y, l1 = a1 * c1.x - b1 * c1.y;
+        const float h0 = b0 * c0.x + a0 * c0.y, h1 = b1 * c1.x + a1 * c1.y;
+        r.lo[w] = pack_bf16x2(l0, l1);
+        r.hi[w] = pack_bf16x2(h0, h1);
+        if (raw) {
+            raw[2 * w] = l0, raw[2 * w + 1] = l1;
+            raw[8 + 2 * w] = h0, raw[8 + 2 * w + 1] = h1;
+        }
     }
     return r;
 }
 
 // grid = (position tiles of 16, batch rows, kv heads): a workgroup rotates the query heads of one
 // kv-head group plus that group's key head, copies its value head, and leaves the sum of its
-// rotated-to-one-position queries over its positions in d_qpart (for the block's mean query).
+// rotated-to-one-position queries over its positions in d_qpart (for the block's mean query; summed
+// before the rounding to bf16, so the mean query carries no rounding of its own).
+//
+// Angles.  cos / sin of (position x frequency) are needed for 16 positions x 64 frequencies per workgroup.
+// Only the workgroup's FIRST position and the step of one position are evaluated (fp64 sincos, one call
+// per thread for 128 threads); the other 15 positions follow by the angle-addition recurrence in fp64,
+// whose error after 15 steps is a few 1e-16 - far below the fp32 value the rotation consumes.  The rows
+// the workgroup will rotate are requested from memory BEFORE that arithmetic, so the two overlap.
 __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
     __shared__ float2 cs_pos[kPosPerBlock][kHalf];
     __shared__ float2 cs_glb[kHalf];
+    __shared__ double2 cs_step[kHalf];                // (cos, sin) of one position's step per frequency
     __shared__ float red[4][kPosPerBlock][kD];        // q_glb of 4 heads x 16 positions, for the partial sums
     const int tid = threadIdx.x;
     const int b = blockIdx.y, g = blockIdx.z;
     const int G = a.H / a.Hkv;
     const int p0 = blockIdx.x * kPosPerBlock;
     const int np = min(kPosPerBlock, a.n - p0);
-
-    for (int e = tid; e < kPosPerBlock * kHalf; e += 256) {
-        int p = e / kHalf, f = e % kHalf;
-        double ang = (double)(a.pos0 + p0 + p) * a.distance_scale * (double)a.d_inv_freq[f];
-        double s, c;
-        sincos(ang, &s, &c);
-        cs_pos[p][f] = make_float2((float)c, (float)s);
-    }
-    if (tid < kHalf) {
-        double ang = (double)a.glb_pos * a.distance_scale * (double)a.d_inv_freq[tid];
-        double s, c;
-        sincos(ang, &s, &c);
-        cs_glb[tid] = make_float2((float)c, (float)s);
-    }
-    __syncthreads();
 
     const bf16_t *q = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb;
     const bf16_t *k = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh;
@@ -66,29 +66,81 @@ __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
     bf16_t *rv = (bf16_t *)a.d_ring_v + ring_g;
     const int n_tiles = (a.n + kPosPerBlock - 1) / kPosPerBlock;
 
+    // ---- requests first: the first group of (up to) 4 query heads, the key head, the value head
+    constexpr int kQItems = 2;                        // 4 heads x 16 positions x 8 chunk pairs = 512 items over 256 threads
+    u32x4 q_lo[kQItems], q_hi[kQItems], k_lo, k_hi, v_row;
+    const int nh0 = min(4, G);
+#pragma unroll
+    for (int i = 0; i < kQItems; ++i) {
+        const int e = tid + i * 256;
+        if (e < nh0 * np * 8) {
+            const int c = e & 7, p = (e >> 3) % np, hl = (e >> 3) / np;
+            const bf16_t *src = q + (int64_t)(g * G + hl) * a.q_sh + (int64_t)(p0 + p) * a.q_sl;
+            q_lo[i] = *(const u32x4 *)(src + c * 8);
+            q_hi[i] = *(const u32x4 *)(src + kHalf + c * 8);
+        }
+    }
+    if (tid < np * 8) {
+        const bf16_t *src = k + (int64_t)(p0 + (tid >> 3)) * a.k_sl;
+        k_lo = *(const u32x4 *)(src + (tid & 7) * 8);
+        k_hi = *(const u32x4 *)(src + kHalf + (tid & 7) * 8);
+    }
+    if (tid < np * 16) v_row = *(const u32x4 *)(v + (int64_t)(p0 + (tid >> 4)) * a.v_sl + (tid & 15) * 8);
+
+    // ---- angles
+    if (tid < kHalf) {
+        const double w = a.distance_scale * (double)a.d_inv_freq[tid];
+        double s, c;
+        sincos((double)(a.pos0 + p0) * w, &s, &c);
+        cs_pos[0][tid] = make_float2((float)c, (float)s);
+        cs_step[tid] = make_double2(c, s);            // parked here until the step values arrive
+    } else if (tid < 2 * kHalf) {
+        const int f = tid - kHalf;
+        double s, c;
+        sincos((double)a.glb_pos * a.distance_scale * (double)a.d_inv_freq[f], &s, &c);
+        cs_glb[f] = make_float2((float)c, (float)s);
+    }
+    double2 step = make_double2(1.0, 0.0);
+    if (tid < kHalf) {
+        double s, c;
+        sincos(a.distance_scale * (double)a.d_inv_freq[tid], &s, &c);
+        step = make_double2(c, s);
+        double2 cur = cs_step[tid];
+        for (int p = 1; p < kPosPerBlock; ++p) {      // (cos, sin)(x + w) from (cos, sin)(x)
+            const double c2 = cur.x * step.x - cur.y * step.y, s2 = cur.y * step.x + cur.x * step.y;
+            cur = make_double2(c2, s2);
+            cs_pos[p][tid] = make_float2((float)c2, (float)s2);
+        }
+    }
+    __syncthreads();
+
     // query heads of the group, 4 at a time: 8 threads per (head, position) row
     for (int hg0 = 0; hg0 < G; hg0 += 4) {
         const int nh = min(4, G - hg0);
-        for (int e = tid; e < nh * np * 8; e += 256) {
+#pragma unroll
+        for (int i = 0; i < kQItems; ++i) {
+            const int e = tid + i * 256;
+            if (e >= nh * np * 8) continue;
             const int c = e & 7, p = (e >> 3) % np, hl = (e >> 3) / np;
             const int h = g * G + hg0 + hl;
-            const bf16_t *src = q + (int64_t)h * a.q_sh + (int64_t)(p0 + p) * a.q_sl;
-            u32x4 lo = *(const u32x4 *)(src + c * 8), hi = *(const u32x4 *)(src + kHalf + c * 8);
+            u32x4 lo = q_lo[i], hi = q_hi[i];
+            if (hg0 > 0) {
+                const bf16_t *src = q + (int64_t)h * a.q_sh + (int64_t)(p0 + p) * a.q_sl;
+                lo = *(const u32x4 *)(src + c * 8), hi = *(const u32x4 *)(src + kHalf + c * 8);
+            }
             int64_t o = ((int64_t)h * a.n + p0 + p) * kD;
             Rot8 r = rotate8(lo, hi, &cs_pos[p][c * 8]);
             *(u32x4 *)(q_loc + o + c * 8) = r.lo;
             *(u32x4 *)(q_loc + o + kHalf + c * 8) = r.hi;
-            r = rotate8(lo, hi, &cs_glb[c * 8]);
+            float raw[16];
+            r = rotate8(lo, hi, &cs_glb[c * 8], raw);
             *(u32x4 *)(q_glb + o + c * 8) = r.lo;
             *(u32x4 *)(q_glb + o + kHalf + c * 8) = r.hi;
             if (a.d_qpart) {
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    red[hl][p][c * 8 + 2 * w] = bf16_bits_to_f32(r.lo[w] & 0xffffu);
-                    red[hl][p][c * 8 + 2 * w + 1] = bf16_bits_to_f32(r.lo[w] >> 16);
-                    red[hl][p][kHalf + c * 8 + 2 * w] = bf16_bits_to_f32(r.hi[w] & 0xffffu);
-                    red[hl][p][kHalf + c * 8 + 2 * w + 1] = bf16_bits_to_f32(r.hi[w] >> 16);
-                }
+                *(f32x4 *)&red[hl][p][c * 8] = f32x4{raw[0], raw[1], raw[2], raw[3]};
+                *(f32x4 *)&red[hl][p][c * 8 + 4] = f32x4{raw[4], raw[5], raw[6], raw[7]};
+                *(f32x4 *)&red[hl][p][kHalf + c * 8] = f32x4{raw[8], raw[9], raw[10], raw[11]};
+                *(f32x4 *)&red[hl][p][kHalf + c * 8 + 4] = f32x4{raw[12], raw[13], raw[14], raw[15]};
             }
         }
         if (a.d_qpart) {
@@ -103,23 +155,17 @@ __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
         }
     }
     // key head: raw copy + rotated copy into the rings
-    for (int e = tid; e < np * 8; e += 256) {
-        const int c = e & 7, p = e >> 3;
-        const bf16_t *src = k + (int64_t)(p0 + p) * a.k_sl;
-        u32x4 lo = *(const u32x4 *)(src + c * 8), hi = *(const u32x4 *)(src + kHalf + c * 8);
+    if (tid < np * 8) {
+        const int c = tid & 7, p = tid >> 3;
         const int64_t o = ((a.pos0 + p0 + p) % a.ring_cap) * kD;
-        *(u32x4 *)(rk_raw + o + c * 8) = lo;
-        *(u32x4 *)(rk_raw + o + kHalf + c * 8) = hi;
-        Rot8 r = rotate8(lo, hi, &cs_pos[p][c * 8]);
+        *(u32x4 *)(rk_raw + o + c * 8) = k_lo;
+        *(u32x4 *)(rk_raw + o + kHalf + c * 8) = k_hi;
+        Rot8 r = rotate8(k_lo, k_hi, &cs_pos[p][c * 8]);
         *(u32x4 *)(rk_rot + o + c * 8) = r.lo;
         *(u32x4 *)(rk_rot + o + kHalf + c * 8) = r.hi;
     }
     // value head: plain copy, 16 threads per row
-    for (int e = tid; e < np * 16; e += 256) {
-        const int c = e & 15, p = e >> 4;
-        const bf16_t *src = v + (int64_t)(p0 + p) * a.v_sl;
-        *(u32x4 *)(rv + ((a.pos0 + p0 + p) % a.ring_cap) * kD + c * 8) = *(const u32x4 *)(src + c * 8);
-    }
+    if (tid < np * 16) *(u32x4 *)(rv + ((a.pos0 + p0 + (tid >> 4)) % a.ring_cap) * kD + (tid & 15) * 8) = v_row;
     // the score track of a new token starts at zero (context_manager.py:733-741)
     for (int e = tid; e < G * np; e += 256) {
         const int p = e % np, h = g * G + e / np;

@@ -157,10 +157,28 @@ __device__ __forceinline__ void publish(int32_t *flag, int32_t value) {
     if (threadIdx.x == 0) __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// The k selected (id, key) pairs sit in LDS in ascending id; they leave in the order torch.topk returns them
+// (context_manager.py:163: descending score), equal keys in ascending id.  The residency policy inserts a block's
+// missed units in that order (context_manager.py:495-515), so the order decides later evictions.
+__device__ __forceinline__ void emit_descending(const int32_t *sel_id, const uint32_t *sel_key, int k, int32_t *idx_out,
+                                                int32_t *idx_out2) {
+    const int t = threadIdx.x;
+    if (t >= k) return;
+    const uint32_t mine = sel_key[t];
+    int rank = 0;
+    for (int j = 0; j < k; ++j) {
+        const uint32_t kj = sel_key[j];
+        rank += (kj > mine || (kj == mine && j < t)) ? 1 : 0;
+    }
+    put_id(idx_out, idx_out2, rank, sel_id[t]);
+}
+
 __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *idx_out2,
                                                            int32_t *flag, int32_t flag_value) {
     __shared__ int hist[256];
     __shared__ int wave_tot[kSelThreads / 64];
+    __shared__ int32_t sel_id[kSelThreads];
+    __shared__ uint32_t sel_key[kSelThreads];
     __shared__ uint32_t sh_prefix;
     __shared__ int sh_need;
     const int tid = threadIdx.x;
@@ -202,17 +220,19 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
         const int eq_rank = eq_base + block_exclusive_scan(is_eq, wave_tot, &tot_eq);
         const int sel = (n < N && (key > prefix || (is_eq && eq_rank < need))) ? 1 : 0;
         const int pos = out_base + block_exclusive_scan(sel, wave_tot, &tot_sel);
-        if (sel && pos < k) put_id(idx_out, idx_out2, pos, n);
+        if (sel && pos < k) sel_id[pos] = n, sel_key[pos] = key;
         eq_base += tot_eq;
         out_base += tot_sel;
     }
+    __syncthreads();
+    emit_descending(sel_id, sel_key, k, idx_out, idx_out2);
     publish(flag, flag_value);
 }
 
 // Tables of up to 16384 scores: every thread keeps its R consecutive keys in registers, so the scores are read
 // once.  Three digit passes (12, 12 and 8 bits from the top; 4096 bins spread the keys of one binade over
 // many LDS counters) find the key of the k-th largest; a pass whose bucket is wanted whole ends the search.
-// Output contract as above: indices ascending, lowest indices among keys equal to the k-th.
+// Output contract as above: lowest indices among keys equal to the k-th; ids leave in descending score.
 template <int R>
 __global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *idx_out2,
                                                                 int32_t *flag, int32_t flag_value) {
@@ -289,39 +309,47 @@ __global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *sco
     int excl = incl - packed;
     for (int w = 0; w < kSelThreads / 64; ++w) excl += w < wave ? wave_tot[w] : 0;
     int g_before = excl & 0xffff, e_before = excl >> 16;
+    // the histogram is free now: ids and keys of the selection in ascending id, then out in descending score
+    int32_t *sel_id = hist;
+    uint32_t *sel_key = (uint32_t *)hist + kSelThreads;
 #pragma unroll
     for (int j = 0; j < R; ++j) {
         if (j >= n_valid) break;
         const uint32_t mk = key[j] & pmask;
         if (mk > prefix) {
-            put_id(idx_out, idx_out2, g_before + min(e_before, need), tid * R + j);
+            const int pos = g_before + min(e_before, need);
+            sel_id[pos] = tid * R + j, sel_key[pos] = key[j];
             ++g_before;
         } else if (mk == prefix) {
-            if (e_before < need) put_id(idx_out, idx_out2, g_before + e_before, tid * R + j);
+            if (e_before < need) {
+                const int pos = g_before + e_before;
+                sel_id[pos] = tid * R + j, sel_key[pos] = key[j];
+            }
             ++e_before;
         }
     }
+    __syncthreads();
+    emit_descending(sel_id, sel_key, k, idx_out, idx_out2);
     publish(flag, flag_value);
 }
 
-// The selection over ALL units from two parts: the k best of the units that existed earlier (`cand`, ids ascending,
+// The selection over ALL units from two parts: the k best of the units that existed earlier (`cand`, any order,
 // chosen by the kernels above while other work was still in flight) and the n_new units carved since, whose scores
 // arrive last.  A unit of the overall top-k that is not new is among the k best of the old ones, so ranking these
-// n_cand + n_new <= 64 candidates by (key, lower id first) gives the same set, written in ascending id as above.
+// n_cand + n_new <= 64 candidates by (key, lower id first) gives the same list, in the same order, as above.
 __global__ __launch_bounds__(64) void topk_merge_kernel(const float *scores, const int32_t *cand, int n_cand, int first_new,
                                                         int n_new, int k, int32_t *idx_out, int32_t *flag, int32_t flag_value) {
     const int lane = threadIdx.x, n = n_cand + n_new;
     const bool valid = lane < n;
-    const int id = lane < n_cand ? cand[lane] : first_new + (lane - n_cand);       // ascending in the lane
+    const int id = lane < n_cand ? cand[lane] : first_new + (lane - n_cand);
     const uint32_t key = valid ? order_key(scores[id]) : 0u;
     int rank = 0;
     for (int j = 0; j < n; ++j) {
         const uint32_t kj = __shfl(key, j, 64);
-        rank += (kj > key || (kj == key && j < lane)) ? 1 : 0;
+        const int idj = __shfl(id, j, 64);
+        rank += (kj > key || (kj == key && idj < id)) ? 1 : 0;
     }
-    const bool sel = valid && rank < k;
-    const uint64_t mask = __ballot(sel);
-    if (sel) idx_out[__popcll(mask & ((1ull << lane) - 1))] = id;
+    if (valid && rank < k) idx_out[rank] = id;              // descending score, equal scores in ascending id
     publish(flag, flag_value);
 }
 
@@ -365,16 +393,15 @@ __global__ __launch_bounds__(256) void score_new_rank_kernel(const bf16_t *reps,
     if (wave == 0) {
         const int n = n_cand + n_new;
         const bool valid = lane < n;
-        const int id = lane < n_cand ? cand[lane] : first_new + (lane - n_cand);       // ascending in the lane
+        const int id = lane < n_cand ? cand[lane] : first_new + (lane - n_cand);
         const uint32_t key = !valid ? 0u : order_key(lane < n_cand ? scores[id] : fresh[lane - n_cand]);
         int rank = 0;
         for (int j = 0; j < n; ++j) {
             const uint32_t kj = __shfl(key, j, 64);
-            rank += (kj > key || (kj == key && j < lane)) ? 1 : 0;
+            const int idj = __shfl(id, j, 64);
+            rank += (kj > key || (kj == key && idj < id)) ? 1 : 0;
         }
-        const bool sel = valid && rank < k;
-        const uint64_t mask = __ballot(sel);
-        if (sel) idx_out[__popcll(mask & ((1ull << lane) - 1))] = id;
+        if (valid && rank < k) idx_out[rank] = id;          // descending score, equal scores in ascending id
     }
     publish(flag, flag_value);
 }

@@ -51,7 +51,8 @@ struct Layer {
         bool has_event = false;
     } off;
     int32_t seen_seq = 0;                 // last selection sequence number the host has read
-    hipStream_t main_stream = nullptr;    // of the last infllm_block_back
+    hipStream_t main_stream = nullptr;    // of the last infllm_block_front / infllm_block_back
+    bool main_stream_known = false;
     // The same copy through the DMA engine (see issue_offload_dma): agents of this layer's GPU and of the host,
     // one completion signal per carve staging slot, and which units a slot's copy in flight carries
     bool dma_ok = false;
@@ -101,6 +102,9 @@ struct Layer {
     int32_t *d_cand = nullptr;
     int cand_units = -1;
     bool has_global = false;
+    bool global_unmarked = false;         // the last global stage ran without recording global_done (see block_back)
+    hipEvent_t idle_main = nullptr, idle_copy = nullptr;      // recorded by layer_flush: this layer's work up to there
+    bool idle_recorded = false;
     bool topk_pending = false;
     int slot = 0;                         // workspace slot written last
     int cur_slot = 0;                     // workspace slot of the block between front() and back()
@@ -629,6 +633,7 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         !d.d_q_glb || !d.d_qbar || !d.d_qpart || !d.d_o_part || !d.d_lse_part || !d.d_lse || !d.d_topk_idx || !d.d_pages ||
         !d.h_pages || !d.d_carve_stage || !d.d_inv_freq)
         return bad("null buffer");
+    if (d.topk > 64) return bad("topk above 64 (the selection lists of a block are fixed 64-entry arrays)");
     if (d.max_splits < 1 || d.max_splits > 64 || d.num_cus < 1 || d.page_slots < 1 || d.carve_slots < 1 || d.max_carve < 1 ||
         d.max_pages < 1 || d.init_cap < 1)
         return bad("bad capacities");
@@ -638,7 +643,9 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
               hipEventCreateWithFlags(&L->global_done, hipEventDisableTiming) == hipSuccess &&
               hipEventCreateWithFlags(&L->fetch_done, hipEventDisableTiming) == hipSuccess &&
               hipEventCreateWithFlags(&L->carve_ready, hipEventDisableTiming) == hipSuccess &&
-              hipEventCreateWithFlags(&L->mass_done, hipEventDisableTiming) == hipSuccess;
+              hipEventCreateWithFlags(&L->mass_done, hipEventDisableTiming) == hipSuccess &&
+              hipEventCreateWithFlags(&L->idle_main, hipEventDisableTiming) == hipSuccess &&
+              hipEventCreateWithFlags(&L->idle_copy, hipEventDisableTiming) == hipSuccess;
     L->page_evt.resize(d.page_slots, nullptr);
     L->carve_evt.resize(d.carve_slots, nullptr);
     L->page_busy.assign(d.page_slots, 0);
@@ -681,7 +688,13 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
 extern "C" int infllm_layer_destroy(void *layer) {
     if (!layer) return 0;
     Layer *L = (Layer *)layer;
-    for (hipEvent_t e : {L->topk_done, L->global_done, L->fetch_done, L->carve_ready, L->mass_done})
+    // The caller frees the layer's buffers next: wait for the work that uses them - what layer_flush marked on the two
+    // streams (every append ends with it), not for the device, which may be busy with other layers.
+    if (L->idle_recorded) {
+        (void)hipEventSynchronize(L->idle_main);
+        (void)hipEventSynchronize(L->idle_copy);
+    }
+    for (hipEvent_t e : {L->topk_done, L->global_done, L->fetch_done, L->carve_ready, L->mass_done, L->idle_main, L->idle_copy})
         if (e) (void)hipEventDestroy(e);
     for (hipEvent_t e : L->page_evt)
         if (e) (void)hipEventDestroy(e);
@@ -879,6 +892,8 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     INFLLM_REQUIRE(a->n_units >= 0 && a->b0 >= 0, "block_front: negative state");
     INFLLM_REQUIRE(a->n_next >= 0 && a->n_next <= d.exc, "block_front: bad next block size %d", a->n_next);
     int rc;
+    L->main_stream = st;
+    L->main_stream_known = true;
 
     // ---- this block's prologue and retrieval, unless the previous block prepared them
     if (!(L->prepared && L->prepared_b0 == a->b0 && L->prepared_n == a->n)) {
@@ -1127,6 +1142,13 @@ extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, voi
         const int wrc = infllm_layer_wait_topk(layer);
         if (wrc) return wrc;
     }
+    if (L->global_unmarked && !a->wait_topk && L->main_stream) {
+        // The previous global stage left no event behind because the host was expected to read this block's selection
+        // (which the stream produces after that stage) before fetching.  A caller that brings its own selection has not
+        // waited for anything: the slots may still be read, so wait here.
+        HIP_OK(hipStreamSynchronize(L->main_stream), "block_select: wait for the previous global stage");
+    }
+    L->global_unmarked = false;
     L->last_n_sel = a->n_sel;
     if (a->n_sel > 0) L->last_sel.assign(a->h_selected, a->h_selected + (int64_t)d.B * a->n_sel);
     else L->last_sel.clear();
@@ -1342,7 +1364,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         if ((side || L->efetch_ok) && !L->guessing) {
             HIP_OK(hipEventRecord(L->global_done, st), "block_back: event");
             L->has_global = true;
-        }
+            L->global_unmarked = false;
+        } else
+            L->global_unmarked = side || L->efetch_ok;
         parts += at.nsplit;
     }
     // Only the joint log-sum-exp is needed on the way to the next selection, and only by the small score launch of
@@ -1534,6 +1558,11 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
     for (size_t s = 0; s < L->dma_busy.size(); ++s) {       // engine copies are not ordered by any stream: finish them here
         const int wrc = dma_wait_slot(L, (int)s, "layer_flush");
         if (wrc) return wrc;
+    }
+    if (L->main_stream_known) {
+        HIP_OK(hipEventRecord(L->idle_main, L->main_stream), "layer_flush: event");
+        HIP_OK(hipEventRecord(L->idle_copy, (hipStream_t)copy_stream), "layer_flush: event");
+        L->idle_recorded = true;
     }
     return 0;
 }

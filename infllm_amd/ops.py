@@ -184,7 +184,7 @@ def local_score(q, k, lse, score, *, cap=None, j_lo=0, j_hi=None, mask=MASK_NONE
 
 
 def score_topk(reps, n, qbar, k, scores, idx):
-    """scores[:n] = reps[:n] @ qbar; idx[:k] = ascending indices of the k largest."""
+    """scores[:n] = reps[:n] @ qbar; idx[:k] = indices of the k largest, descending score."""
     check(_lib.load().infllm_score_topk(reps.data_ptr(), reps.stride(0), n, reps.shape[1], qbar.data_ptr(), k,
                                         scores.data_ptr(), idx.data_ptr() if idx is not None else None, _stream()),
           "infllm_score_topk")
@@ -192,14 +192,14 @@ def score_topk(reps, n, qbar, k, scores, idx):
 
 def score_new_topk(reps, qbar, scores, cand, first_new, n_new, k, idx):
     """scores[first_new:first_new+n_new] = reps[those rows] @ qbar, then idx[:k] = the top-k over all first_new + n_new
-    scores, given cand = the top-k (ascending ids) of the first first_new."""
+    scores, given cand = the top-k of the first first_new."""
     check(_lib.load().infllm_score_new_topk(reps.data_ptr(), reps.stride(0), reps.shape[1], qbar.data_ptr(), scores.data_ptr(),
                                             cand.data_ptr(), cand.numel(), first_new, n_new, k, idx.data_ptr(), _stream()),
           "infllm_score_new_topk")
 
 
 def topk(scores, n, k, idx):
-    """idx[:k] = ascending indices of the k largest of scores[:n] (lowest indices among equal scores)."""
+    """idx[:k] = indices of the k largest of scores[:n] in descending score (lower index first among equal scores)."""
     check(_lib.load().infllm_topk(scores.data_ptr(), n, k, idx.data_ptr(), _stream()), "infllm_topk")
 
 

@@ -28,7 +28,20 @@ Per append() call (context_manager.py:682-813):
 Two hooks let a test follow another implementation's discrete choices where
 the acceptance rule allows them to differ (near-ties): ``topk_hook`` and
 ``repr_hook``.  They receive the oracle's own fp32 scores and may return the
-choice to adopt, or None to keep the oracle's.
+choice to adopt, or None to keep the oracle's.  A selection is an ORDERED list,
+in the order torch.topk returns it (descending score, :163): the residency
+policy inserts a block's missed units in that order (:495-515), and the order
+breaks ties between equal stamps at later evictions (:253-265).
+
+``rep_dtype`` rounds every representative to that dtype when it is stored: the
+reference keeps them in a VectorTensor of the model dtype (:321-328, 675), so
+torch.bfloat16 restates its bf16 runs; None keeps the compute dtype.
+
+``StreamOracle.from_state`` starts from a snapshot (window, un-carved tail with
+its score track, init tokens, units, representatives - the fields of
+context_manager.py:309-363 restated in absolute terms) instead of an empty
+stream, so that a few execution blocks at the end of a stream too long for the
+CPU can be recomputed.
 """
 import torch
 
@@ -80,7 +93,7 @@ class UnitCacheModel:
             for b in selected:
                 self.cached[b] = 0
         assert len(self.cached) <= self.capacity, "unit cache overflow (topk > max_cached_block)"
-        self.events.append(dict(selected=sorted(selected), misses=sorted(misses), evicted=evicted))
+        self.events.append(dict(selected=sorted(selected), order=list(selected), misses=sorted(misses), evicted=evicted))
 
     def add_scores(self, units, unit_scores):
         """lru-s (context_manager.py:454-470): decay every value, add the block's mass."""
@@ -93,7 +106,7 @@ class UnitCacheModel:
 class StreamOracle:
     def __init__(self, rope, n_init, n_local, block_size, max_cached_block, topk,
                  exc_block_size, score_decay=None, repr_topk=1, cache_strategy="lru",
-                 perhead=False, topk_hook=None, repr_hook=None, chunk_topk_calc=None):
+                 perhead=False, topk_hook=None, repr_hook=None, chunk_topk_calc=None, rep_dtype=None):
         assert exc_block_size <= n_local                      # context_manager.py:219
         self.chunk_topk_calc = chunk_topk_calc
         self.rope = rope
@@ -106,6 +119,7 @@ class StreamOracle:
         self.score_decay = score_decay
         self.perhead = perhead
         self.topk_hook, self.repr_hook = topk_hook, repr_hook
+        self.rep_dtype = rep_dtype
         self.length = 0
         self.ready = False
         self._chunk_plan = None
@@ -132,6 +146,41 @@ class StreamOracle:
     def size(self):
         return self.length
 
+    def from_state(self, state, dtype=torch.float32):
+        """Continue a stream from a snapshot.  ``state``: length T; tail_k / tail_v [B,Hkv,T-cursor,D], the tokens
+        not carved yet (context_manager.py:333-336: the remainder, whose last n_local tokens are the local window,
+        :330-331); tail_score [B,H,T-cursor] or None (:338); init_k / init_v [B,Hkv,init_len,D] (:341-343); units:
+        anything indexable by unit id that yields [B,2,Hkv,bs,D] (K at index 0, V at 1; :317, 652-662), with n_units
+        entries; reps [B,n_units,H*D] (:321-328).  The counts must satisfy the closed forms of :614-679.  The unit
+        cache starts empty.  Unit tensors are kept as they are given and converted when a block reads them."""
+        assert not self.ready and self.length == 0
+        f = lambda t: t.detach().to("cpu").to(dtype)
+        tail_k, tail_v = f(state["tail_k"]), f(state["tail_v"])
+        T = int(state["length"])
+        self.B, self.Hkv, n_tail, self.D = tail_k.shape
+        reps = state.get("reps")
+        self.H = reps.shape[2] // self.D if reps is not None and reps.numel() else int(state["num_heads"])
+        init_len = min(self.n_init, max(T - self.n_local, 0))
+        n_units = max(0, (T - self.n_init - self.n_local) // self.block_size)
+        assert n_tail == T - init_len - n_units * self.block_size, (n_tail, T, init_len, n_units)
+        self.win_k, self.win_v = tail_k[:, :, -self.n_local:], tail_v[:, :, -self.n_local:]
+        self.rem_k, self.rem_v = tail_k, tail_v
+        sc = state.get("tail_score")
+        self.rem_score = f(sc) if sc is not None else torch.zeros(self.B, self.H, n_tail, dtype=dtype)
+        assert self.rem_score.shape == (self.B, self.H, n_tail)
+        self.init_k, self.init_v = f(state["init_k"]), f(state["init_v"])
+        assert self.init_k.shape[2] == init_len
+        self.init_full = init_len == self.n_init
+        units = state.get("units")
+        self.units = [[(units[i][u, 0], units[i][u, 1]) for i in range(n_units)] for u in range(self.B)]
+        reps_f = f(reps[:, :n_units]) if n_units else None
+        self.reps = [[reps_f[u, i] for i in range(n_units)] for u in range(self.B)]
+        self.n_units = n_units
+        self.cache = [UnitCacheModel(self.max_cached_block, self.cache_strategy, self.score_decay) for _ in range(self.B)]
+        self.length = T
+        self.ready = True
+        return self
+
     def _group(self, x):
         """[B, Hkv, L, D] -> [B, H, L, D] (context_manager.py:280-289)."""
         if self.H == self.Hkv:
@@ -155,11 +204,11 @@ class StreamOracle:
             for u in range(self.B):
                 reps = torch.stack(self.reps[u]).reshape(self.n_units, self.H, self.D)
                 sc = torch.einsum("nhd,hd->nh", reps, mean_q[u]).mean(dim=1)
-                pick = sorted(sc.topk(self.topk).indices.tolist())
+                pick = sc.topk(self.topk).indices.tolist()                     # descending score, as :586 / :604 return it
                 if self.topk_hook is not None:
                     other = self.topk_hook(len(self.block_trace) + j, u, sc * self.H)
                     if other is not None:
-                        pick = sorted(other)
+                        pick = list(other)
                 chosen.append(pick)
                 scores.append(sc * self.H)
             out.append((chosen, scores))
@@ -177,11 +226,11 @@ class StreamOracle:
             for u in range(self.B):
                 reps = torch.stack(self.reps[u])                       # [N, H*D]
                 s = reps @ mean_q[u]
-                pick = sorted(s.topk(self.topk).indices.tolist())
+                pick = s.topk(self.topk).indices.tolist()                      # descending score (:163)
                 if self.topk_hook is not None:
                     other = self.topk_hook(len(self.block_trace), u, s)
                     if other is not None:
-                        pick = sorted(other)
+                        pick = list(other)
                 chosen.append(pick)
                 scores.append(s)
         return chosen, scores
@@ -195,7 +244,10 @@ class StreamOracle:
                 idx = torch.as_tensor(other, dtype=torch.int64)
         k_full = self._group(unit_k[None])[0]                                  # [H, bs, D]
         rows = torch.gather(k_full, 1, idx[:, :, None].expand(-1, -1, self.D))
-        return rows.mean(dim=1).reshape(self.H * self.D), idx
+        rep = rows.mean(dim=1).reshape(self.H * self.D)
+        if self.rep_dtype is not None:
+            rep = rep.to(self.rep_dtype).to(rows.dtype)
+        return rep, idx
 
     # ------------------------------------------------------------- one block
     def _block(self, q, win_k, win_v, gq, cur_st, cur_ed):
@@ -211,8 +263,9 @@ class StreamOracle:
         overflow = max(cur_ed - cur_st + len_q - self.n_local, 0)
         parts_k, parts_v = [], []
         for u in range(self.B):
-            ks = [self.units[u][b][0] for b in chosen[u]]
-            vs = [self.units[u][b][1] for b in chosen[u]]
+            as_mine = lambda t: t.to(device=q.device, dtype=q.dtype)               # units given to from_state stay as they came
+            ks = [as_mine(self.units[u][b][0]) for b in sorted(chosen[u])]         # :399 sorts before placing the units
+            vs = [as_mine(self.units[u][b][1]) for b in sorted(chosen[u])]
             ks += [self.init_k[u], self.rem_k[u, :, cur_st:cur_st + overflow]]
             vs += [self.init_v[u], self.rem_v[u, :, cur_st:cur_st + overflow]]
             parts_k.append(torch.cat(ks, dim=-2))
@@ -229,10 +282,10 @@ class StreamOracle:
             per_unit = glob_score[:, :, :n_unit_keys].reshape(self.B, self.H, len(chosen[0]), self.block_size)
             per_unit = per_unit.sum(dim=-1).sum(dim=1)
             for u in range(self.B):
-                self.cache[u].add_scores(chosen[u], per_unit[u].tolist())
+                self.cache[u].add_scores(sorted(chosen[u]), per_unit[u].tolist())
 
         self.block_trace.append(dict(
-            selected=[list(c) for c in chosen], unit_scores=unit_scores, n_units=self.n_units,
+            selected=[sorted(c) for c in chosen], order=[list(c) for c in chosen], unit_scores=unit_scores, n_units=self.n_units,
             init_len=self.init_k.shape[-2], overflow=overflow, global_len=glob_k.shape[-2],
             local_len=win_k.shape[-2]))
         return out, loc_score

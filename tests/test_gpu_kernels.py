@@ -88,9 +88,11 @@ def test_ingest_partial_sums_give_the_mean_global_query():
     ops.ingest(q.cuda(), k.cuda(), v.cuda(), 3, 63, rope.inv_freq.cuda(), 1.0, rk_raw, rk_rot, rv, rscore, q_loc, q_glb, qpart)
     qbar = torch.zeros((B, H * D), dtype=torch.float32, device="cuda")
     ops.reduce_partials(qpart, 1.0 / n, qbar)
-    want = q_glb.float().mean(dim=2).reshape(B, H * D)
-    assert torch.allclose(qbar, want, atol=1e-5)
-    assert torch.allclose(want.cpu(), rope.one_angle(q.float(), 64).mean(dim=2).reshape(B, H * D), atol=1e-2)
+    # the sums are taken before q_glb is rounded to bf16: the mean query is the fp32 oracle's up to fp32 rounding,
+    # and the bf16 rows' own mean differs from it by their rounding (2^-9 relative per element, averaged down)
+    want = rope.one_angle(q.float(), 64).mean(dim=2).reshape(B, H * D)
+    assert torch.allclose(qbar.cpu(), want, atol=2e-6)
+    assert torch.allclose(q_glb.float().mean(dim=2).reshape(B, H * D).cpu(), want, atol=2e-3)
 
 
 def test_block_mean():
@@ -233,7 +235,9 @@ def test_two_stage_joint_softmax_with_ring_and_pages():
     out2, lse2 = torch.empty_like(out), torch.empty_like(lse)
     ops.attn_fwd(la, ga, out2, lse2)
     _check_out(out2, want)
-    assert torch.allclose(lse2, lse, atol=1e-4)
+    # the row sums are taken over bf16-rounded probabilities (what the second MFMA multiplies), so the log-sum-exp
+    # depends on how the keys were split at the 2^-9 / sqrt(keys) level
+    assert torch.allclose(lse2, lse, atol=1e-3)
     out3 = torch.empty_like(out)
     ops.attn_fwd(None, ga, out3, None)                       # one stage alone
     ops.attn_merge(o_part[1:2], lse_part[1:2], 1, out2, None)
@@ -314,10 +318,11 @@ def test_score_topk_matches_bruteforce(N, k):
     got_scores = scores.cpu().double().numpy()
     assert np.allclose(got_scores, want, rtol=1e-4, atol=1e-3)
     got = idx.cpu().tolist()
-    assert got == sorted(got) and len(set(got)) == k
-    # exactly the top-k of the kernel's own fp32 scores (ties at the boundary -> lower index) ...
-    order = sorted(range(N), key=lambda i: (-float(scores[i]), i))
-    assert got == sorted(order[:k])
+    assert len(set(got)) == k
+    # exactly the top-k of the kernel's own fp32 scores, in descending score like torch.topk (equal scores -> lower index first) ...
+    host_scores = scores.cpu().tolist()
+    order = sorted(range(N), key=lambda i: (-host_scores[i], i))
+    assert got == order[:k]
     # ... and equal to the oracle's set except for candidates within 1e-3 relative of the boundary
     want_set = set(np.argsort(-want, kind="stable")[:k].tolist())
     kth = np.sort(want)[-k]
@@ -359,7 +364,7 @@ def test_topk_with_exact_ties_takes_lowest_indices():
     scores = torch.empty((N,), dtype=torch.float32, device="cuda")
     idx = torch.empty((16,), dtype=torch.int32, device="cuda")
     ops.score_topk(reps.cuda(), N, qbar.cuda(), 16, scores, idx)
-    assert idx.cpu().tolist() == [0, 1, 2, 3, 4, 5] + list(range(200, 210))
+    assert idx.cpu().tolist() == list(range(200, 210)) + [0, 1, 2, 3, 4, 5]
     neg = (-reps).cuda()
     ops.score_topk(neg, N, qbar.cuda(), 4, scores, idx)
     assert idx.cpu().tolist()[:4] == [0, 1, 2, 3]
@@ -369,7 +374,7 @@ def test_topk_with_exact_ties_takes_lowest_indices():
                                         (30000, 50, 7)])
 def test_topk_on_heavily_tied_scores_is_the_stable_descending_prefix(N, k, levels):
     """Few distinct score values (negative, zero and positive): the selection must be the first k of a stable
-    descending sort, returned in ascending index order, whichever digit pass the search stops in."""
+    descending sort, returned in that order, whichever digit pass the search stops in."""
     ops = _ops()
     g = torch.Generator().manual_seed(N + k)
     vals = torch.randint(0, levels, (N,), generator=g).float() - levels // 2
@@ -378,7 +383,7 @@ def test_topk_on_heavily_tied_scores_is_the_stable_descending_prefix(N, k, level
     idx = torch.full((k,), -1, dtype=torch.int32, device="cuda")
     ops.topk(scores, N, k, idx)
     order = sorted(range(N), key=lambda i: (-float(vals[i]), i))
-    assert idx.cpu().tolist() == sorted(order[:k])
+    assert idx.cpu().tolist() == order[:k]
 
 
 @pytest.mark.parametrize("bs,r,H,Hkv", [(128, 4, 32, 8), (8, 2, 4, 2), (100, 1, 3, 3), (64, 64, 2, 1)])

@@ -53,10 +53,11 @@ def test_cache_policy_equals_oracle_model(strategy):
     n_units = 3
     for step in range(300):
         n_units += rng.randint(0, 2)
-        sel = sorted(rng.sample(range(n_units), min(3, n_units)))
+        sel = rng.sample(range(n_units), min(3, n_units))           # an ordered list, as torch.topk returns it
         misses, evicted = pol.touch(sel)
         model.touch(sel)
         assert sorted(misses) == model.events[-1]["misses"]
+        assert misses == [u for u in sel if u in misses]              # misses are reported in selection order
         assert evicted == model.events[-1]["evicted"]
         assert pol.cached == model.cached
         assert set(pol.slot_of) == set(pol.cached)
@@ -84,11 +85,12 @@ def test_trying_a_selection_out_on_a_copy_leaves_the_policy_as_the_oracle_model_
     try:
         for step in range(400):
             n_units += rng.randint(0, 2)
-            guess = sorted(rng.sample(range(n_units), k))
+            guess = rng.sample(range(n_units), k)
             real = guess
             if rng.random() < 0.4:                       # as in the stream: a fresh unit displaces one of the guess
                 others = [u for u in range(n_units) if u not in guess]
-                real = sorted(rng.sample(guess, k - 1) + [rng.choice(others)])
+                real = rng.sample(guess, k - 1)
+                real.insert(rng.randrange(k), rng.choice(others))
             before = dict(pol.slot_of)
             assert lib.infllm_cache_copy(shadow, pol.handle) == 0
             g_slots, g_mu, g_ms, g_ev, g_nev = (I * k)(), (I * k)(), (I * k)(), (I * cap)(), I(0)
@@ -125,11 +127,38 @@ def test_trying_a_selection_out_on_a_copy_leaves_the_policy_as_the_oracle_model_
     assert lib.infllm_cache_copy(other.handle, pol.handle) != 0          # different capacity: refused
 
 
+def test_units_missed_in_one_block_are_inserted_in_selection_order():
+    """context_manager.py:495-515 walks the torch.topk list (descending score), so the units a block loads together
+    enter the dict in that order, and the order decides which of them leaves first once their stamps tie
+    (:253-265, a stable sort).  Capacity 4, selections [5,2], [7,8], [9,7]: the third block must evict 5, the unit
+    inserted first; with the ids sorted it would be 2."""
+    pol, model = CachePolicy(4, "lru", None), UnitCacheModel(4, "lru", None)
+    for sel, want in (([5, 2], []), ([7, 8], []), ([9, 7], [5])):
+        misses, evicted = pol.touch(sel)
+        model.touch(sel)
+        assert evicted == want == model.events[-1]["evicted"]
+    assert list(pol.cached) == list(model.cached) == [2, 7, 8, 9]
+    # the reference's dict in plain Python, for the same three blocks
+    cached, clock = {}, 0
+    for sel in ([5, 2], [7, 8], [9, 7]):
+        surplus = len(cached) - 4 + sum(b not in cached for b in sel)
+        for unit, _ in sorted(cached.items(), key=lambda kv: kv[1]):
+            if surplus <= 0:
+                break
+            if unit not in sel:
+                del cached[unit]
+                surplus -= 1
+        clock += 1
+        for b in sel:
+            cached[b] = clock
+    assert list(cached) == [2, 7, 8, 9]
+
+
 def test_cache_policy_lru_s_equals_oracle_model():
     rng = random.Random(6)
     pol, model = CachePolicy(5, "lru-s", 0.9), UnitCacheModel(5, "lru-s", 0.9)
     for step in range(200):
-        sel = sorted(rng.sample(range(12), 3))
+        sel = rng.sample(range(12), 3)
         _, evicted = pol.touch(sel)
         model.touch(sel)
         assert evicted == model.events[-1]["evicted"]

@@ -200,7 +200,7 @@ def test_cache_model_lru_hand_worked():
     c.touch([1, 4])          # two misses, capacity 3 -> evict 2 (stamp 2) then 0 (stamp 3)
     assert c.events[-1]["evicted"] == [2, 0] and set(c.cached) == {3, 1, 4}
     c.touch([3, 1])          # hits only
-    assert c.events[-1] == dict(selected=[1, 3], misses=[], evicted=[])
+    assert c.events[-1] == dict(selected=[1, 3], order=[3, 1], misses=[], evicted=[])
 
 
 def test_cache_model_ties_break_in_insertion_order_and_selected_are_kept():
@@ -294,3 +294,67 @@ def test_oracle_still_produces_its_frozen_vectors():
             assert np.allclose(frozen[name], fresh[name], atol=1e-5), name
         else:
             assert np.array_equal(frozen[name], fresh[name]), name
+
+
+# ------------------------------------------------------------- resume from a snapshot
+def _snapshot(cm):
+    """The oracle's own state in the form StreamOracle.from_state takes (the fields of context_manager.py:309-363)."""
+    units = [torch.stack([torch.stack(cm.units[u][i]) for u in range(cm.B)]) for i in range(cm.n_units)]
+    reps = torch.stack([torch.stack(cm.reps[u]) if cm.n_units else torch.zeros(0, cm.H * cm.D) for u in range(cm.B)])
+    return dict(length=cm.length, tail_k=cm.rem_k, tail_v=cm.rem_v, tail_score=cm.rem_score, init_k=cm.init_k, init_v=cm.init_v,
+                units=units, reps=reps, num_heads=cm.H)
+
+
+@pytest.mark.parametrize("T0,calls", [(150, [90]), (20, [100, 3]), (36, [1] * 30), (97, [64, 1, 40])])
+def test_resume_from_a_snapshot_equals_the_uninterrupted_stream(T0, calls):
+    """from_state + append against one oracle that saw the whole stream: outputs, selections, representatives,
+    final state - before the window is full, mid init peeling, and with units already carved."""
+    T = T0 + sum(calls)
+    q, k, v = _stream(T, seed=T, B=2)
+    whole_out, whole = _run(q, k, v, [T0] + calls)
+    _, first = _run(q, k, v, [T0])
+    resumed = StreamOracle(RopeOracle(q.shape[-1], base=10000), **GEOM).from_state(_snapshot(first))
+    assert resumed.length == T0 and resumed.n_units == first.n_units
+    outs, pos = [], T0
+    for L in calls:
+        outs.append(resumed.append(q[:, :, pos:pos + L], k[:, :, pos:pos + L], v[:, :, pos:pos + L]))
+        pos += L
+    assert torch.allclose(torch.cat(outs, dim=-2), whole_out[:, :, T0:], atol=1e-6)
+    n_first = len(first.block_trace)
+    assert [b["order"] for b in resumed.block_trace] == [b["order"] for b in whole.block_trace[n_first:]]
+    assert resumed.n_units == whole.n_units and resumed.length == whole.length
+    for u in range(2):
+        for mine, theirs in zip(resumed.reps[u], whole.reps[u]):
+            assert torch.allclose(mine, theirs, atol=1e-6)
+    assert torch.equal(resumed.rem_k, whole.rem_k) and torch.allclose(resumed.rem_score, whole.rem_score, atol=1e-6)
+    assert torch.equal(resumed.init_k, whole.init_k)
+
+
+def test_selections_are_ordered_lists_and_the_order_reaches_the_cache_model():
+    """torch.topk order (descending score) is what the residency policy sees (context_manager.py:163, 495-515)."""
+    q, k, v = _stream(400, seed=3)
+    _, cm = _run(q, k, v, [400], topk=3, max_cached_block=4)
+    seen = 0
+    for blk, ev in zip(cm.block_trace, cm.cache[0].events):
+        assert ev["order"] == blk["order"][0] and sorted(blk["order"][0]) == blk["selected"][0]
+        sc = blk["unit_scores"][0]
+        if sc is not None:
+            vals = [float(sc[i]) for i in blk["order"][0]]
+            assert vals == sorted(vals, reverse=True)
+            seen += vals != sorted(vals) and blk["order"][0] != blk["selected"][0]
+    assert seen > 3
+
+
+def test_representatives_can_be_kept_in_the_model_dtype():
+    """rep_dtype=bfloat16 (the reference's VectorTensor of the model dtype, context_manager.py:321-328): every stored
+    representative is the bf16 rounding of the fp32 one, and nothing else changes while the selections agree."""
+    q, k, v = _stream(300, seed=5)
+    _, a = _run(q, k, v, [300])
+    _, b = _run(q, k, v, [300], rep_dtype=torch.bfloat16)
+    assert a.n_units == b.n_units > 0
+    same = 0
+    for ra, rb, ta, tb in zip(a.reps[0], b.reps[0], a.unit_trace, b.unit_trace):
+        if torch.equal(ta["repr_idx"], tb["repr_idx"]):
+            assert torch.equal(rb, ra.bfloat16().float())
+            same += 1
+    assert same >= a.n_units // 2
