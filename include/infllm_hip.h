@@ -158,6 +158,19 @@ int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t
 int infllm_attn_fwd(const infllm_attn_args *local, const infllm_attn_args *global,
                     void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse, void *stream);
 
+/* infllm_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The stages' partial rows, which
+ * infllm_attn_fwd takes from the caller as a workspace (d_o_part / d_lse_part), live in an array inside the library's
+ * own image instead: the d_o_part / d_lse_part fields of both argument blocks are ignored, everything else is as for
+ * infllm_attn_fwd, and the results are the same bit for bit.  The call allocates nothing (no hipMalloc / hipFree, no
+ * allocating library routine).  Limit: (local nsplit + global nsplit) * B * H * Lq <= INFLLM_NOALLOC_MAX_PART_ROWS
+ * partial rows (260 bytes each: 16.25 MiB of device memory per GPU, held until the process ends); larger calls are
+ * rejected with an error.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams,
+ * two threads) race - serialise them, or use infllm_attn_fwd with workspaces of your own. */
+#define INFLLM_NOALLOC_MAX_PART_ROWS 65536
+int infllm_attn_fwd_noalloc(const infllm_attn_args *local, const infllm_attn_args *global,
+                            void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse, void *stream);
+
 /* ---------------------------------------------------------------------------
  * Column sums of the final probabilities of one linear stage
  * (torch_impl.py:27-28; triton_impl.py:232-335):

@@ -646,6 +646,12 @@ __global__ __launch_bounds__(256) void attn_merge_lse_wide_kernel(const float *l
 
 }  // namespace
 
+#define HIP_OK_ATTN(call, what)                                                         \
+    do {                                                                                \
+        hipError_t e_ = (call);                                                         \
+        if (e_ != hipSuccess) return infllm_fail(-2, "%s: %s", what, hipGetErrorString(e_)); \
+    } while (0)
+
 extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
     INFLLM_REQUIRE(a != nullptr, "attn_stage: null argument block");
     INFLLM_REQUIRE(a->d_q && a->d_o_part && a->d_lse_part, "attn_stage: null q / output pointer");
@@ -717,6 +723,61 @@ extern "C" int infllm_attn_fwd(const infllm_attn_args *local, const infllm_attn_
     if (rc) return rc;
     return infllm_attn_merge(first->d_o_part, first->d_lse_part, parts, first->B, first->H, first->Lq, d_out, o_sb, o_sh, o_sl,
                              d_lse, stream);
+}
+
+// ---- the forward for callers that cannot allocate
+// The stages' partial rows are scratch memory: infllm_attn_fwd takes them from the caller.  A caller under HIP graph
+// capture, in a tight serving loop or in a harness that forbids hipMalloc has nowhere to get them from, so this
+// variant keeps them in an array of the library's own image.  Every GPU the library runs on holds its own copy of the
+// array (at its own address) until the process ends; every call on a GPU uses that GPU's copy, so calls that overlap on
+// one GPU race.  Nothing has to be cleared between calls: each split writes all of its rows and log-sum-exps before
+// the merge reads them.
+constexpr int64_t kStaticPartRows = INFLLM_NOALLOC_MAX_PART_ROWS;            // (split, batch row, head, query) rows
+static __device__ __align__(256) unsigned char attn_static_scratch[kStaticPartRows * (kD * 2 + 4)];
+constexpr int kMaxDevices = 64;
+static unsigned char *static_scratch_ptr[kMaxDevices];                       // per device: where ITS copy of the array lives
+static bool static_scratch_known[kMaxDevices];
+
+extern "C" int infllm_attn_fwd_noalloc(const infllm_attn_args *local, const infllm_attn_args *global, void *d_out, int64_t o_sb,
+                                       int64_t o_sh, int64_t o_sl, float *d_lse, void *stream) {
+    INFLLM_REQUIRE(local || global, "attn_fwd_noalloc: no stage given");
+    const infllm_attn_args *first = local ? local : global;
+    INFLLM_REQUIRE(first->B > 0 && first->H > 0 && first->Lq > 0, "attn_fwd_noalloc: bad geometry");
+    if (local && global)
+        INFLLM_REQUIRE(local->B == global->B && local->H == global->H && local->Lq == global->Lq,
+                       "attn_fwd_noalloc: the two stages disagree on B / H / Lq");
+    const int parts = (local ? local->nsplit : 0) + (global ? global->nsplit : 0);
+    const int64_t rows = (int64_t)first->B * first->H * first->Lq;
+    INFLLM_REQUIRE(parts >= 1 && parts <= 128, "attn_fwd_noalloc: %d key splits", parts);
+    INFLLM_REQUIRE(parts * rows <= kStaticPartRows,
+                   "attn_fwd_noalloc: %d splits x %lld rows exceed the built-in scratch of %lld partial rows (use infllm_attn_fwd "
+                   "with a workspace of your own)", parts, (long long)rows, (long long)kStaticPartRows);
+    int dev = -1;
+    HIP_OK_ATTN(hipGetDevice(&dev), "attn_fwd_noalloc");
+    INFLLM_REQUIRE(dev >= 0 && dev < kMaxDevices, "attn_fwd_noalloc: device %d", dev);
+    if (!static_scratch_known[dev]) {          // once per device, with that device current: the symbol's address THERE
+        void *p = nullptr;
+        HIP_OK_ATTN(hipGetSymbolAddress(&p, HIP_SYMBOL(attn_static_scratch)), "attn_fwd_noalloc: hipGetSymbolAddress");
+        INFLLM_REQUIRE(p != nullptr, "attn_fwd_noalloc: no address for the scratch array");
+        static_scratch_ptr[dev] = (unsigned char *)p;
+        static_scratch_known[dev] = true;
+    }
+    // o partials first (fp16 rows), the log-sum-exps behind all of them; the global stage's follow the local stage's
+    uint16_t *o_part = (uint16_t *)static_scratch_ptr[dev];
+    float *lse_part = (float *)(static_scratch_ptr[dev] + kStaticPartRows * kD * 2);
+    infllm_attn_args l{}, g{};
+    if (local) {
+        l = *local;
+        l.d_o_part = o_part;
+        l.d_lse_part = lse_part;
+    }
+    if (global) {
+        g = *global;
+        const int64_t skip = local ? (int64_t)local->nsplit * rows : 0;
+        g.d_o_part = o_part + skip * kD;
+        g.d_lse_part = lse_part + skip;
+    }
+    return infllm_attn_fwd(local ? &l : nullptr, global ? &g : nullptr, d_out, o_sb, o_sh, o_sl, d_lse, stream);
 }
 
 extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,

@@ -155,6 +155,17 @@ def attn_fwd(local_args, global_args, out, lse):
                                       lse.data_ptr() if lse is not None else None, _stream()), "infllm_attn_fwd")
 
 
+NOALLOC_MAX_PART_ROWS = 65536       # INFLLM_NOALLOC_MAX_PART_ROWS
+
+
+def attn_fwd_noalloc(local_args, global_args, out, lse):
+    """attn_fwd with the partial rows in the library's built-in scratch array (the argument blocks' o_part / lse_part
+    are ignored); allocates nothing.  Calls on one GPU must not overlap."""
+    _need(out.stride(-1) == 1 and out.dtype == torch.bfloat16, "bad merge output")
+    check(_lib.load().infllm_attn_fwd_noalloc(local_args, global_args, out.data_ptr(), out.stride(0), out.stride(1), out.stride(2),
+                                              lse.data_ptr() if lse is not None else None, _stream()), "infllm_attn_fwd_noalloc")
+
+
 def attn_merge(o_part, lse_part, P, out, lse):
     """Join P partials: out bf16 [B,H,Lq,D] (any strides with contiguous rows), lse fp32 [B,H,Lq]."""
     B, H, Lq, D = out.shape

@@ -1,0 +1,89 @@
+"""infllm_attn_fwd_noalloc: the attention forward whose partial rows live in the library's built-in scratch array,
+for callers that cannot allocate.  Checked through the C ABI against infllm_attn_fwd (caller-provided workspace) on
+the same inputs: bit-equal outputs and log-sum-exps, on two calls in a row of which the second is smaller (the
+array keeps the first call's contents), and a call beyond the built-in limit is rejected with a clear error."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+D = 128
+
+
+def _rand(shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g).bfloat16()
+
+
+def _case(ops, B, H, Hkv, Lq, n_local, n_glob, nsplit_l, nsplit_g, seed):
+    cap = (n_local + Lq + 63) // 64 * 64 + 64
+    b0 = 3000
+    lo, b1 = b0 - n_local, b0 + Lq
+    q, qg = _rand((B, H, Lq, D), seed).cuda(), _rand((B, H, Lq, D), seed + 1).cuda()
+    ring_k, ring_v = _rand((B, Hkv, cap, D), seed + 2).cuda(), _rand((B, Hkv, cap, D), seed + 3).cuda()
+    pool_k, pool_v = _rand((Hkv, n_glob, D), seed + 4).cuda(), _rand((Hkv, n_glob, D), seed + 5).cuda()
+    ent, pos = [], 0
+    while pos < n_glob:
+        n = min(64, n_glob - pos)
+        ent.append((pool_k.data_ptr() + pos * D * 2, pool_v.data_ptr() + pos * D * 2, n_glob * D, n))
+        pos += n
+    arr = ops.make_pages(ent * B)
+    host = torch.empty((len(ent) * B * 32,), dtype=torch.uint8)
+    ctypes.memmove(host.data_ptr(), arr, len(ent) * B * 32)
+    pages = host.cuda()
+    P = nsplit_l + nsplit_g
+    o_part = torch.empty((P, B, H, Lq, D), dtype=torch.float16, device="cuda")
+    lse_part = torch.empty((P, B, H, Lq), dtype=torch.float32, device="cuda")
+
+    def blocks(op, lp):
+        la = ops.linear_stage_args(q, ring_k, ring_v, op[:nsplit_l], lp[:nsplit_l], cap=cap, j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW,
+                                   offset=b0, window=n_local, nsplit=nsplit_l)
+        ga = ops.paged_stage_args(qg, pages, len(ent), Hkv, op[nsplit_l:], lp[nsplit_l:], nsplit=nsplit_g)
+        return la, ga
+
+    keep = (q, qg, ring_k, ring_v, pool_k, pool_v, pages, o_part, lse_part)
+    return blocks, o_part, lse_part, (B, H, Lq), keep
+
+
+def _both_ways(ops, case):
+    blocks, o_part, lse_part, (B, H, Lq), _ = case
+    want, want_lse = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda"), torch.empty((B, H, Lq), device="cuda")
+    ops.attn_fwd(*blocks(o_part, lse_part), want, want_lse)
+    got, got_lse = torch.full_like(want, float("nan")), torch.full_like(want_lse, float("nan"))
+    dummy_o, dummy_l = torch.empty((1,), dtype=torch.float16, device="cuda"), torch.empty((1,), dtype=torch.float32, device="cuda")
+    la, ga = blocks(o_part, lse_part)
+    la.d_o_part = la.d_lse_part = ga.d_o_part = ga.d_lse_part = None         # ignored by the entry point: show it
+    ops.attn_fwd_noalloc(la, ga, got, got_lse)
+    torch.cuda.synchronize()
+    assert torch.isfinite(want.float()).all() and torch.isfinite(want_lse).all()
+    assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
+    return got
+
+
+def test_noalloc_forward_equals_the_workspace_forward_twice_in_a_row():
+    from infllm_amd import ops
+    from infllm_amd._lib import InfLLMHipError
+    big = _case(ops, B=2, H=8, Hkv=2, Lq=96, n_local=512, n_glob=64 * 5 + 17, nsplit_l=3, nsplit_g=2, seed=70)
+    small = _case(ops, B=1, H=4, Hkv=4, Lq=7, n_local=200, n_glob=100, nsplit_l=1, nsplit_g=2, seed=80)
+    first = _both_ways(ops, big)                      # 5 x 1536 partial rows
+    second = _both_ways(ops, small)                   # 3 x 28 rows, into the array the first call left full
+    assert first.shape != second.shape
+    again = _both_ways(ops, big)                      # and the large one once more
+    assert torch.equal(again, first)
+    # beyond the built-in scratch: rejected, nothing launched
+    B, H, Lq, P = 1, 32, 512, 8
+    assert P * B * H * Lq > ops.NOALLOC_MAX_PART_ROWS
+    huge = _case(ops, B=B, H=H, Hkv=8, Lq=Lq, n_local=1024, n_glob=256, nsplit_l=4, nsplit_g=4, seed=90)
+    la, ga = huge[0](huge[1], huge[2])
+    out = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(InfLLMHipError, match="exceed the built-in scratch"):
+        ops.attn_fwd_noalloc(la, ga, out, None)
+    # one stage alone is a valid call as well
+    la, _ = small[0](small[1], small[2])
+    want, got = torch.empty((1, 4, 7, D), dtype=torch.bfloat16, device="cuda"), torch.empty((1, 4, 7, D), dtype=torch.bfloat16, device="cuda")
+    ops.attn_fwd(la, None, want, None)
+    ops.attn_fwd_noalloc(la, None, got, None)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
