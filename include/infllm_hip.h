@@ -158,6 +158,15 @@ int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t
 int infllm_attn_fwd(const infllm_attn_args *local, const infllm_attn_args *global,
                     void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse, void *stream);
 
+/* Both stages of the operator in ONE launch (attn.append(local...) + attn.append(global..., end=True),
+ * context_manager.py:486-489, 526-533; the reference's fused implementation carries the softmax state across its
+ * stages the same way, triton_impl.py:488-556): the linear stage's tiles and the paged stage's pages form one list
+ * that `nsplit` key splits divide between them, each with the queries of its own stage (local->d_q, global->d_q).
+ * Both blocks must agree on B, H, Hkv, Lq and softmax_scale; nsplit and the partial buffers are taken from `local`:
+ * d_o_part [nsplit,B,H,Lq,128] fp16, d_lse_part [nsplit,B,H,Lq] - one set of partials for both stages, to be joined
+ * by infllm_attn_merge with P = nsplit. */
+int infllm_attn_stages_fused(const infllm_attn_args *local, const infllm_attn_args *global, void *stream);
+
 /* infllm_attn_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The stages' partial rows, which
  * infllm_attn_fwd takes from the caller as a workspace (d_o_part / d_lse_part), live in an array inside the library's

@@ -131,6 +131,7 @@ SYMBOLS = {
     "infllm_attn_stage": (c_i32, [C.POINTER(AttnArgs), c_vp]),
     "infllm_attn_merge": (c_i32, [c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
     "infllm_attn_fwd": (c_i32, [C.POINTER(AttnArgs), C.POINTER(AttnArgs), c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
+    "infllm_attn_stages_fused": (c_i32, [C.POINTER(AttnArgs), C.POINTER(AttnArgs), c_vp]),
     "infllm_attn_fwd_noalloc": (c_i32, [C.POINTER(AttnArgs), C.POINTER(AttnArgs), c_vp, c_i64, c_i64, c_i64, c_vp, c_vp]),
     "infllm_local_score": (c_i32, [C.POINTER(ScoreArgs), c_vp]),
     "infllm_unit_scores": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp]),

@@ -16,6 +16,8 @@
 // pi(r) = 16*(r>>4) + 8*((r>>2)&1) + 4*((r>>3)&1) + (r&3); with that binding the 16
 // accumulator registers of a lane are two runs of 8 consecutive keys, which is exactly
 // the k-slice the second MFMA wants from the lane.  V is transposed on its way into LDS.
+#include <cstdlib>
+
 #include "common.h"
 
 namespace {
@@ -108,13 +110,22 @@ struct IntC {
     static constexpr int value = N;
 };
 
-template <bool PAGED>
-__global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a, StageGeom geo) {
+// MODE: what the launch walks.  kLinear: the linear source of `a`; kPaged: the page table of `a`; kBoth: the linear
+// source of `a`, then the page table of `a2` with `a2`'s queries - both stages of the operator in one launch, as ONE
+// list of tiles that the key splits divide between them (one set of partials, one fixed cost instead of two).
+enum { kLinear = 0, kPaged = 1, kBoth = 2 };
+
+template <int MODE>
+__global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a, infllm_attn_args a2, StageGeom geo) {
+    constexpr bool HAS_LIN = MODE != kPaged, HAS_PAG = MODE != kLinear;
+    const infllm_attn_args &ap = MODE == kBoth ? a2 : a;                 // the paged stage's arguments
     extern __shared__ __attribute__((aligned(16))) char lds_dyn[];      // kStages K tiles, then kStages V tiles
     char *const Ks = lds_dyn, *const Vs = lds_dyn + kStages * kTileBytes;
     __shared__ int wg_lo[kWaves], wg_hi[kWaves];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    // the wave index is the same in every lane: said so, what derives from it (the wave's queries, tile range, mask
+    // distances) stays in scalar registers
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
     const int G = (int)geo.group.d;
     // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  Renumber so that
@@ -143,45 +154,42 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     const int h = g * G + hg;
     const int i0 = qt * kQTile, i1 = min(i0 + kQTile, a.Lq) - 1;
 
-    int w_t0, w_t1;                      // this wave's tile range
-    if (PAGED) {
-        w_t0 = 0;
-        w_t1 = live ? a.n_pages : 0;
-    } else {
+    int w_t0 = 0, w_t1 = 0;              // this wave's range of LINEAR tiles (absolute tile numbers)
+    if (HAS_LIN && live) {
         StageRange r = visible_range(a, i0, i1);
-        if (!live || r.hi <= r.lo) {
-            w_t0 = w_t1 = 0;
-        } else {
+        if (r.hi > r.lo) {
             w_t0 = floordiv64(r.lo);
             w_t1 = floordiv64(r.hi - 1) + 1;
         }
     }
-    // ---- workgroup range = union over its waves; the split takes a contiguous share of it
+    // ---- workgroup range of linear tiles = union over its waves
     if (lane == 0) {
         wg_lo[wave] = w_t1 > w_t0 ? w_t0 : INT32_MAX;
         wg_hi[wave] = w_t1 > w_t0 ? w_t1 : INT32_MIN;
     }
     __syncthreads();
-    int g_t0 = INT32_MAX, g_t1 = INT32_MIN;
+    int lin_t0 = INT32_MAX, lin_t1 = INT32_MIN;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-        g_t0 = min(g_t0, wg_lo[w]);
-        g_t1 = max(g_t1, wg_hi[w]);
+        lin_t0 = min(lin_t0, wg_lo[w]);
+        lin_t1 = max(lin_t1, wg_hi[w]);
     }
-    if (g_t1 <= g_t0) g_t0 = g_t1 = 0;
+    if (lin_t1 <= lin_t0) lin_t0 = lin_t1 = 0;
+    // The unified tile list: u in [0, n_lin) is linear tile lin_t0 + u, u in [n_lin, n_lin + n_pag) is page u - n_lin.
+    const int n_lin = lin_t1 - lin_t0, n_pag = HAS_PAG ? ap.n_pages : 0;
+    int g_t0, g_t1;                      // this split's share of the list
     {
         // n / nsplit tiles each; the n % nsplit left over go one each to a run of splits in the middle: the first and
         // the last split hold the tiles that need the mask (window start, causal diagonal) and take 1-2 us longer over
         // the same number of tiles, so with the extras at the ends the whole launch waited for them
-        const uint32_t n = (uint32_t)(g_t1 - g_t0), per = fdiv(n, geo.nsplit), rem = n - per * a.nsplit;
+        const uint32_t n = (uint32_t)(n_lin + n_pag), per = fdiv(n, geo.nsplit), rem = n - per * a.nsplit;
         const int first_extra = (int)((a.nsplit - rem) >> 1);
         const int before = min(max(split - first_extra, 0), (int)rem);            // extras given to lower splits
         const int mine = (split >= first_extra && split < first_extra + (int)rem) ? 1 : 0;
-        int t_begin = g_t0 + (int)per * split + before;
-        int t_end = t_begin + (int)per + mine;
-        g_t0 = t_begin;
-        g_t1 = t_end;
+        g_t0 = (int)per * split + before;
+        g_t1 = g_t0 + (int)per + mine;
     }
+    const int wu0 = w_t0 - lin_t0, wu1 = w_t1 - lin_t0;     // this wave's linear tiles in list indices
 
     bf16x8 qreg[kD / 16];                     // Q as the B operand: lane = (query col, k-group); loaded behind the first tiles
 
@@ -204,48 +212,52 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     // ---- tile loads: wave w, instruction i fills LDS rows 8*w + 4*i .. +3; lane -> (row, position).
     //      The wave-uniform tile base advances with the loop; the per-lane offsets are loop invariant.
     constexpr int kLd = kTile / (4 * kWaves);  // load instructions per wave and tile, for K and for V
-    uint32_t gk_off[kLd], gv_off[kLd];        // element offsets inside a tile
+    uint32_t gk_off[kLd], gv_off[kLd];        // element offsets inside a linear tile
+    uint32_t pk_off[kLd], pv_off[kLd];        // ... inside a page (rows of kD elements)
     int gk_row[kLd], gv_row[kLd];
     {
         const int ld_pos = lane & 15, ld_sub = lane >> 4;
-        const int64_t k_sl = PAGED ? kD : a.k_sl, v_sl = PAGED ? kD : a.v_sl;
 #pragma unroll
         for (int i = 0; i < kLd; ++i) {
             const int R = 4 * kLd * wave + 4 * i + ld_sub, chunk = ld_pos ^ swz(R);
             gk_row[i] = k_lds_row(R);
             gv_row[i] = R;
-            gk_off[i] = (uint32_t)(gk_row[i] * k_sl + chunk * 8);
-            gv_off[i] = (uint32_t)(R * v_sl + chunk * 8);
+            if (HAS_LIN) {
+                gk_off[i] = (uint32_t)(gk_row[i] * a.k_sl + chunk * 8);
+                gv_off[i] = (uint32_t)(R * a.v_sl + chunk * 8);
+            }
+            if (HAS_PAG) {
+                pk_off[i] = (uint32_t)(gk_row[i] * kD + chunk * 8);
+                pv_off[i] = (uint32_t)(R * kD + chunk * 8);
+            }
         }
     }
     const bf16_t *k_head = nullptr, *v_head = nullptr;          // linear source: row 0 of this kv head
-    int64_t ring_row = 0;                                        // ring row of the tile to load next
-    if (!PAGED) {
+    int64_t ring_row = 0;                                        // ring row of the linear tile to load next
+    if (HAS_LIN) {
         k_head = (const bf16_t *)a.d_k + (int64_t)b * a.k_sb + (int64_t)g * a.k_sh;
         v_head = (const bf16_t *)a.d_v + (int64_t)b * a.v_sb + (int64_t)g * a.v_sh;
-        ring_row = (int64_t)(g_t0 - (int)(fdiv(g_t0, geo.cap_tiles) * geo.cap_tiles.d)) * kTile;
+        const int first = lin_t0 + min(g_t0, n_lin);
+        ring_row = (int64_t)(first - (int)(fdiv(first, geo.cap_tiles) * geo.cap_tiles.d)) * kTile;
     }
     // The page table is read through the constant address space: the index is wave-uniform, so these become scalar
     // loads.  As vector loads they would share the vmcnt counter with the tile transfers, and waiting for a page
     // entry would wait for every tile in flight.  The table is written by an earlier kernel and is read-only here.
     const __attribute__((address_space(4))) infllm_page *page_table =
-        (const __attribute__((address_space(4))) infllm_page *)(uintptr_t)a.d_pages;
-    auto load_tile = [&](int t, int buf) {
+        (const __attribute__((address_space(4))) infllm_page *)(uintptr_t)ap.d_pages + (int64_t)b * n_pag;
+    auto load_tile = [&](int u, int buf) {     // list index; linear tiles are requested in ascending order
         const bf16_t *kbase, *vbase;
         int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
-        if (PAGED) {
-            const __attribute__((address_space(4))) infllm_page *entry = page_table + ((int64_t)b * a.n_pages + t);
-            infllm_page pg;
-            pg.k = entry->k;
-            pg.v = entry->v;
-            pg.head_stride = entry->head_stride;
-            pg.n_valid = entry->n_valid;
-            kbase = (const bf16_t *)pg.k + (int64_t)g * pg.head_stride;
-            vbase = (const bf16_t *)pg.v + (int64_t)g * pg.head_stride;
+        const bool paged = MODE == kPaged || (MODE == kBoth && u >= n_lin);
+        if (paged) {
+            const __attribute__((address_space(4))) infllm_page *entry = page_table + (u - n_lin);
+            const int64_t hs = entry->head_stride;
+            kbase = (const bf16_t *)entry->k + (int64_t)g * hs;
+            vbase = (const bf16_t *)entry->v + (int64_t)g * hs;
             row_lo = 0;
-            row_hi = pg.n_valid;
+            row_hi = entry->n_valid;
         } else {
-            const int64_t j0 = (int64_t)t * kTile;
+            const int64_t j0 = (int64_t)(lin_t0 + u) * kTile;
             kbase = k_head + ring_row * a.k_sl;       // cap is a multiple of the tile, so a tile never wraps
             vbase = v_head + ring_row * a.v_sl;
             ring_row += kTile;
@@ -257,16 +269,16 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         if (row_lo == 0 && row_hi == kTile) {          // the common case: no per-lane predicate
 #pragma unroll
             for (int i = 0; i < kLd; ++i) {
-                load_to_lds16(kbase + gk_off[i], (bf16_t *)(kdst + i * 1024));
-                load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
+                load_to_lds16(kbase + (paged ? pk_off[i] : gk_off[i]), (bf16_t *)(kdst + i * 1024));
+                load_to_lds16(vbase + (paged ? pv_off[i] : gv_off[i]), (bf16_t *)(vdst + i * 1024));
             }
         } else {
 #pragma unroll
             for (int i = 0; i < kLd; ++i) {
                 // rows outside the source are written as zeros: their keys are masked, but 0 * stale must stay 0
-                if (gk_row[i] >= row_lo && gk_row[i] < row_hi) load_to_lds16(kbase + gk_off[i], (bf16_t *)(kdst + i * 1024));
+                if (gk_row[i] >= row_lo && gk_row[i] < row_hi) load_to_lds16(kbase + (paged ? pk_off[i] : gk_off[i]), (bf16_t *)(kdst + i * 1024));
                 else *(u32x4 *)(kdst + i * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
-                if (gv_row[i] >= row_lo && gv_row[i] < row_hi) load_to_lds16(vbase + gv_off[i], (bf16_t *)(vdst + i * 1024));
+                if (gv_row[i] >= row_lo && gv_row[i] < row_hi) load_to_lds16(vbase + (paged ? pv_off[i] : gv_off[i]), (bf16_t *)(vdst + i * 1024));
                 else *(u32x4 *)(vdst + i * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
             }
         }
@@ -319,11 +331,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         bool need_mask;
         int row_lo = 0, row_hi = kTile;
         int d0 = 0;                            // dist of (this lane's query, key 0 of the tile)
-        if (PAGED) {
-            row_hi = page_table[(int64_t)b * a.n_pages + t].n_valid;
+        const bool paged = MODE == kPaged || (MODE == kBoth && t >= n_lin);
+        if (paged) {
+            row_hi = page_table[t - n_lin].n_valid;
             need_mask = row_hi < kTile;
         } else {
-            const int64_t j0 = (int64_t)t * kTile;
+            const int64_t j0 = (int64_t)(lin_t0 + t) * kTile;
             row_lo = (int)max((int64_t)0, a.j_lo - j0);
             row_hi = (int)min((int64_t)kTile, a.j_hi - j0);
             need_mask = row_lo > 0 || row_hi < kTile;
@@ -347,7 +360,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                     // expressed relative to the per-lane bases so that no per-register value is kept
                     const int kc = ks * 32 + 16 * (r >> 3) + (r & 7);
                     bool vis = (kc >= lo_l) && (kc < hi_l);
-                    if (!PAGED) {
+                    if (!paged) {
                         if (a.mask == INFLLM_MASK_WINDOW) vis = vis && (kc <= dl) && (kc > dl - win);
                         if (a.mask == INFLLM_MASK_COMPLEMENT) vis = vis && (kc <= dl - win);
                     }
@@ -428,16 +441,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     static_assert(kStages == 4, "two buffer pairs");
     for (int p = 0; p < 2; ++p)
         if (g_t0 + p < g_t1) load_tile(g_t0 + p, p);
-    {
+    auto load_q = [&](const infllm_attn_args &src) {
         const int qi = i0 + col;
-        const bool ok = live && qi < a.Lq;
-        const bf16_t *qrow = (const bf16_t *)a.d_q + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh + (int64_t)qi * a.q_sl;
+        const bool ok = live && qi < src.Lq;
+        const bf16_t *qrow = (const bf16_t *)src.d_q + (int64_t)b * src.q_sb + (int64_t)h * src.q_sh + (int64_t)qi * src.q_sl;
 #pragma unroll
         for (int kk = 0; kk < kD / 16; ++kk) {
             u32x4 raw = ok ? *(const u32x4 *)(qrow + kk * 16 + grp * 8) : u32x4{0, 0, 0, 0};
             qreg[kk] = __builtin_bit_cast(bf16x8, raw);
         }
-    }
+    };
+    // the queries of the stage this split starts in; a split that crosses from the linear tiles into the pages swaps
+    // them for the paged stage's queries at its first page (once per workgroup: that wait also covers the tiles in flight)
+    bool q_paged = MODE == kPaged || (MODE == kBoth && g_t0 >= n_lin);
+    load_q(q_paged ? ap : a);
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // The compiler does not know that the wait above also covered the query rows; passing them through an empty
@@ -446,12 +463,22 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
 #pragma unroll
     for (int kk = 0; kk < kD / 16; ++kk) asm volatile("" : "+v"(qreg[kk]));
     __syncthreads();
+    // does this wave see tile u at all?  (pages: every live wave; linear tiles: the wave's own visible range)
+    auto mine = [&](int u) { return (HAS_PAG && u >= n_lin) ? live : (u >= wu0 && u < wu1); };
     for (int t = g_t0; t < g_t1; t += 2) {
         const int buf = (t - g_t0) & 3;                          // 0 or 2
         if (t + 2 < g_t1) load_tile(t + 2, buf ^ 2);
         if (t + 3 < g_t1) load_tile(t + 3, (buf ^ 2) + 1);
-        if (t >= w_t0 && t < w_t1) tile_math(buf, t);          // wave-uniform; barriers stay outside
-        if (t + 1 < g_t1 && t + 1 >= w_t0 && t + 1 < w_t1) tile_math(buf + 1, t + 1);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {                            // wave-uniform conditions; barriers stay outside
+            const int u = t + e;
+            if (u >= g_t1) break;
+            if (MODE == kBoth && u >= n_lin && !q_paged) {
+                load_q(ap);
+                q_paged = true;
+            }
+            if (mine(u)) tile_math(buf + e, u);
+        }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
@@ -652,50 +679,86 @@ __global__ __launch_bounds__(256) void attn_merge_lse_wide_kernel(const float *l
         if (e_ != hipSuccess) return infllm_fail(-2, "%s: %s", what, hipGetErrorString(e_)); \
     } while (0)
 
-extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
-    INFLLM_REQUIRE(a != nullptr, "attn_stage: null argument block");
-    INFLLM_REQUIRE(a->d_q && a->d_o_part && a->d_lse_part, "attn_stage: null q / output pointer");
+namespace {
+
+int check_linear_stage(const infllm_attn_args *a) {
+    INFLLM_REQUIRE(a->j_hi <= a->j_lo || (a->d_k && a->d_v), "attn_stage: null k / v pointer");
+    INFLLM_REQUIRE(a->cap > 0 && a->cap % kTile == 0, "attn_stage: cap %lld is not a positive multiple of %d",
+                   (long long)a->cap, kTile);
+    INFLLM_REQUIRE(a->j_lo >= 0 && a->j_hi - a->j_lo <= a->cap, "attn_stage: key range [%lld,%lld) exceeds cap %lld",
+                   (long long)a->j_lo, (long long)a->j_hi, (long long)a->cap);
+    INFLLM_REQUIRE(a->mask >= 0 && a->mask <= 2, "attn_stage: unknown mask %d", a->mask);
+    INFLLM_REQUIRE(a->j_hi < (1ll << 36), "attn_stage: key range beyond 2^36 rows");
+    INFLLM_REQUIRE((a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8 | a->v_sl % 8 | a->v_sh % 8 | a->v_sb % 8) == 0,
+                   "attn_stage: k/v strides must be multiples of 8");
+    return 0;
+}
+
+int check_common(const infllm_attn_args *a) {
+    INFLLM_REQUIRE(a->d_q, "attn_stage: null q pointer");
     INFLLM_REQUIRE(a->B > 0 && a->H > 0 && a->Hkv > 0 && a->H % a->Hkv == 0 && a->Lq > 0,
                    "attn_stage: bad geometry B=%d H=%d Hkv=%d Lq=%d", a->B, a->H, a->Hkv, a->Lq);
     INFLLM_REQUIRE(a->nsplit >= 1 && a->nsplit <= 64, "attn_stage: nsplit %d out of range", a->nsplit);
     INFLLM_REQUIRE((a->q_sl % 8 | a->q_sh % 8 | a->q_sb % 8) == 0, "attn_stage: q strides must be multiples of 8");
+    return 0;
+}
+
+// mode: kLinear (a), kPaged (a), kBoth (a = linear stage, a2 = paged stage)
+int launch_stage(int mode, const infllm_attn_args *a, const infllm_attn_args *a2, void *stream) {
     const int G = a->H / a->Hkv;
     const int n_tasks = ((a->Lq + kQTile - 1) / kQTile) * G;
     dim3 grid((n_tasks + kWaves - 1) / kWaves, a->B * a->Hkv, a->nsplit);
     INFLLM_REQUIRE((int64_t)grid.x * grid.y * grid.z < (1ll << 31), "attn_stage: grid too large");
     StageGeom geo{fast_div(grid.x), fast_div(grid.y), fast_div((uint32_t)a->Hkv), fast_div((uint32_t)G),
                   fast_div((uint32_t)a->nsplit), fast_div(1), n_tasks};
+    // tile indices stay below 2^30, so any ring of 2^31 tiles or more never wraps: one divisor stands for all of them
+    if (mode != kPaged) geo.cap_tiles = fast_div((uint32_t)std::min<int64_t>(a->cap / kTile, 1ll << 31));
     constexpr size_t lds_bytes = 2 * kStages * kTileBytes;
-    static bool lds_set[2] = {false, false};           // dynamic LDS above 64 KiB must be enabled once per kernel
-    if (a->d_pages) {
-        INFLLM_REQUIRE(a->n_pages >= 0, "attn_stage: negative page count");
-        if (!lds_set[1]) {
-            hipError_t e = hipFuncSetAttribute((const void *)attn_stage_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
-            lds_set[1] = true;
-        }
-        hipLaunchKernelGGL(attn_stage_kernel<true>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, geo);
-    } else {
-        INFLLM_REQUIRE(a->j_hi <= a->j_lo || (a->d_k && a->d_v), "attn_stage: null k / v pointer");
-        INFLLM_REQUIRE(a->cap > 0 && a->cap % kTile == 0, "attn_stage: cap %lld is not a positive multiple of %d",
-                       (long long)a->cap, kTile);
-        INFLLM_REQUIRE(a->j_lo >= 0 && a->j_hi - a->j_lo <= a->cap, "attn_stage: key range [%lld,%lld) exceeds cap %lld",
-                       (long long)a->j_lo, (long long)a->j_hi, (long long)a->cap);
-        INFLLM_REQUIRE(a->mask >= 0 && a->mask <= 2, "attn_stage: unknown mask %d", a->mask);
-        INFLLM_REQUIRE(a->j_hi < (1ll << 36), "attn_stage: key range beyond 2^36 rows");
-        // tile indices stay below 2^30, so any ring of 2^31 tiles or more never wraps: one divisor stands for all of them
-        geo.cap_tiles = fast_div((uint32_t)std::min<int64_t>(a->cap / kTile, 1ll << 31));
-        INFLLM_REQUIRE((a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8 | a->v_sl % 8 | a->v_sh % 8 | a->v_sb % 8) == 0,
-                       "attn_stage: k/v strides must be multiples of 8");
-        if (!lds_set[0]) {
-            hipError_t e = hipFuncSetAttribute((const void *)attn_stage_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
-            lds_set[0] = true;
-        }
-        hipLaunchKernelGGL(attn_stage_kernel<false>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, geo);
+    static bool lds_set[3] = {false, false, false};           // dynamic LDS above 64 KiB must be enabled once per kernel
+    const void *fn = mode == kLinear ? (const void *)attn_stage_kernel<kLinear>
+                     : mode == kPaged ? (const void *)attn_stage_kernel<kPaged> : (const void *)attn_stage_kernel<kBoth>;
+    if (!lds_set[mode]) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
+        lds_set[mode] = true;
     }
+    const infllm_attn_args &second = a2 ? *a2 : *a;
+    if (mode == kLinear) hipLaunchKernelGGL(attn_stage_kernel<kLinear>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo);
+    else if (mode == kPaged) hipLaunchKernelGGL(attn_stage_kernel<kPaged>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo);
+    else hipLaunchKernelGGL(attn_stage_kernel<kBoth>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo);
     INFLLM_CHECK_LAUNCH("attn_stage");
     return 0;
+}
+
+}  // namespace
+
+extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
+    INFLLM_REQUIRE(a != nullptr, "attn_stage: null argument block");
+    INFLLM_REQUIRE(a->d_o_part && a->d_lse_part, "attn_stage: null output pointer");
+    int rc = check_common(a);
+    if (rc) return rc;
+    if (a->d_pages) {
+        INFLLM_REQUIRE(a->n_pages >= 0, "attn_stage: negative page count");
+        return launch_stage(kPaged, a, nullptr, stream);
+    }
+    rc = check_linear_stage(a);
+    return rc ? rc : launch_stage(kLinear, a, nullptr, stream);
+}
+
+extern "C" int infllm_attn_stages_fused(const infllm_attn_args *local, const infllm_attn_args *global, void *stream) {
+    INFLLM_REQUIRE(local && global, "attn_stages_fused: null argument block");
+    INFLLM_REQUIRE(local->d_o_part && local->d_lse_part, "attn_stages_fused: null output pointer");
+    INFLLM_REQUIRE(!local->d_pages && global->d_pages && global->n_pages >= 0,
+                   "attn_stages_fused: the first stage must be linear, the second paged");
+    INFLLM_REQUIRE(local->B == global->B && local->H == global->H && local->Hkv == global->Hkv && local->Lq == global->Lq,
+                   "attn_stages_fused: the two stages disagree on B / H / Hkv / Lq");
+    INFLLM_REQUIRE(local->softmax_scale == global->softmax_scale, "attn_stages_fused: the two stages disagree on the softmax scale");
+    int rc = check_common(local);
+    if (rc) return rc;
+    rc = check_common(global);
+    if (rc) return rc;
+    rc = check_linear_stage(local);
+    return rc ? rc : launch_stage(kBoth, local, global, stream);
 }
 
 extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,

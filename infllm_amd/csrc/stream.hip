@@ -71,6 +71,9 @@ struct Layer {
     uint32_t efetch_seq = 0;
     bool efetch_wait = false;
     int cur_n = 0;                                     // queries of the block in flight
+    bool local_pending = false;                        // the block's local stage has not been launched yet (block_back does it)
+    bool local_in_front = true;                        // the local stage is launched by block_front; INFLLM_FUSED_STAGES=1:
+                                                       // by block_back, in one launch with the global stage
     bool guessing = false;                             // the last selection settled a fetch made ahead of it
     // The fetch ahead of the selection (see infllm_block_prefetch): the candidates' host copy with the sequence number
     // the kernel publishes behind them, the selection whose global stage may still be running, and the guess in flight.
@@ -676,6 +679,8 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
     {
         const char *any = getenv("INFLLM_FETCH_AHEAD_ALWAYS");
         L->ahead_any_path = any && any[0] && any[0] != '0';
+        const char *fs = getenv("INFLLM_FUSED_STAGES");
+        L->local_in_front = !(fs && fs[0] && fs[0] != '0');
     }
     if (hipHostMalloc((void **)&L->h_cand, ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
         (void)hipGetLastError();
@@ -881,6 +886,27 @@ int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t
     return infllm_local_score(&sc, stream);
 }
 
+// the local stage of a block: causal sliding window over the ring
+infllm_attn_args local_stage_args(Layer *L, int n, int64_t b0, int slot, int nsplit) {
+    const infllm_layer_desc &d = L->d;
+    const int64_t b1 = b0 + n;
+    const int64_t lo = b0 > d.n_local ? b0 - d.n_local : 0;
+    infllm_attn_args at{};
+    at.d_q = (const bf16_t *)d.d_q_loc + (int64_t)slot * d.B * d.H * d.exc * kD;
+    at.q_sl = kD; at.q_sh = (int64_t)n * kD; at.q_sb = (int64_t)d.H * n * kD;
+    at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = n;
+    at.d_k = d.d_ring_k_rot; at.d_v = d.d_ring_v;
+    at.k_sl = at.v_sl = kD;
+    at.k_sh = at.v_sh = d.ring_cap * kD;
+    at.k_sb = at.v_sb = (int64_t)d.Hkv * d.ring_cap * kD;
+    at.cap = d.ring_cap; at.j_lo = lo; at.j_hi = b1;
+    at.mask = INFLLM_MASK_WINDOW; at.offset = b0; at.window = d.n_local;
+    at.nsplit = nsplit;
+    at.softmax_scale = d.softmax_scale;
+    at.d_o_part = d.d_o_part; at.d_lse_part = d.d_lse_part;
+    return at;
+}
+
 }  // namespace
 
 extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void *stream) {
@@ -915,26 +941,21 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     L->cur_n = a->n;
     L->cand_for_units = -1;
 
-    // ---- local stage: causal sliding window over the ring
+    // ---- local stage: causal sliding window over the ring.  Launched here, ahead of the host's wait for the selection
+    //      and of the stream's wait for the fetched units, both of which it covers.  With INFLLM_FUSED_STAGES=1
+    //      block_back launches it instead, in ONE launch with the global stage (measured: the launch is 6 us shorter than
+    //      the two and the merge reads half the partials, but the stream then reaches its wait for the fetch a local
+    //      stage earlier and idles longer than it saved - the missed units' way over PCIe takes 135 us of a 190 us block).
     const int64_t b1 = a->b0 + a->n;
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
-    infllm_attn_args at{};
-    at.d_q = (const bf16_t *)d.d_q_loc + (int64_t)L->cur_slot * d.B * d.H * d.exc * kD;
-    at.q_sl = kD; at.q_sh = (int64_t)a->n * kD; at.q_sb = (int64_t)d.H * a->n * kD;
-    at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = a->n;
-    at.d_k = d.d_ring_k_rot; at.d_v = d.d_ring_v;
-    at.k_sl = at.v_sl = kD;
-    at.k_sh = at.v_sh = d.ring_cap * kD;
-    at.k_sb = at.v_sb = (int64_t)d.Hkv * d.ring_cap * kD;
-    at.cap = d.ring_cap; at.j_lo = lo; at.j_hi = b1;
-    at.mask = INFLLM_MASK_WINDOW; at.offset = a->b0; at.window = d.n_local;
-    at.nsplit = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
-    at.softmax_scale = d.softmax_scale;
-    at.d_o_part = d.d_o_part; at.d_lse_part = d.d_lse_part;
-    const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
-    rc = infllm_attn_stage(&at, stream);
-    timer_end(L, 0, ti, st);
-    if (rc) return rc;
+    L->local_pending = !L->local_in_front;
+    if (L->local_in_front) {
+        infllm_attn_args at = local_stage_args(L, a->n, a->b0, L->cur_slot, splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile)));
+        const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
+        rc = infllm_attn_stage(&at, stream);
+        timer_end(L, 0, ti, st);
+        if (rc) return rc;
+    }
 
     // ---- the next block's prologue and the scores of the units that exist already
     if (a->n_next > 0 && a->d_q_next && a->d_k_next && a->d_v_next) {
@@ -1327,7 +1348,25 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         }
     }
 
-    // ---- 3. global stage and merge
+    // ---- 3. the global stage and merge.  When block_front left the local stage to this call (INFLLM_FUSED_STAGES=1)
+    //         both stages are ONE launch over one list of tiles (ring tiles, then pages) behind the wait for the fetch -
+    //         for every block, not only those whose units are known to be in place: how the keys are cut into partials
+    //         then depends on the block alone, and with it every bit of the result.
+    const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
+    const int lin_tiles = (int)((b1 - lo + kTile - 1) / kTile);
+    const int64_t part_o = (int64_t)d.B * d.H * a->n * kD, part_l = (int64_t)d.B * d.H * a->n;
+    const bool fuse = L->local_pending && n_pages > 0;
+    int rc;
+    int sl = 0;
+    if (L->local_pending && !fuse) {
+        sl = splits_for(d, a->n, lin_tiles);
+        infllm_attn_args at = local_stage_args(L, a->n, a->b0, cur, sl);
+        const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
+        rc = infllm_attn_stage(&at, stream);
+        timer_end(L, 0, ti, st);
+        if (rc) return rc;
+    } else if (!L->local_pending)
+        sl = splits_for(d, a->n, lin_tiles);              // launched by block_front
     const int tw = L->fetch_wait || L->efetch_wait ? timer_begin(L, 2, a->n, a->n_miss, st) : -1;
     if (L->fetch_wait) {
         HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
@@ -1338,11 +1377,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         L->efetch_wait = false;
     }
     timer_end(L, 2, tw, st);
-    const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
-    const int sl = splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile));
     int parts = sl;
-    const int64_t part_o = (int64_t)d.B * d.H * a->n * kD, part_l = (int64_t)d.B * d.H * a->n;
-    int rc;
     if (n_pages > 0) {
         infllm_attn_args at{};
         at.d_q = (const bf16_t *)d.d_q_glb + (int64_t)cur * d.B * d.H * d.exc * kD;
@@ -1350,14 +1385,28 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = a->n;
         at.cap = kTile;
         at.d_pages = d.d_pages; at.n_pages = n_pages;
-        at.nsplit = splits_for(d, a->n, n_pages);
         at.softmax_scale = d.softmax_scale;
-        at.d_o_part = d.d_o_part + sl * part_o;
-        at.d_lse_part = d.d_lse_part + sl * part_l;
-        const int ti = timer_begin(L, 1, a->n, n_pages * kTile, st);
-        rc = infllm_attn_stage(&at, stream);
-        timer_end(L, 1, ti, st);
-        if (rc) return rc;
+        if (fuse) {
+            const int ns = splits_for(d, a->n, lin_tiles + n_pages);
+            infllm_attn_args lt = local_stage_args(L, a->n, a->b0, cur, ns);
+            at.nsplit = ns;
+            at.d_o_part = d.d_o_part; at.d_lse_part = d.d_lse_part;
+            // timed as the block's dominant launch: its key count is the window plus the pages
+            const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo) + n_pages * kTile, st);
+            rc = infllm_attn_stages_fused(&lt, &at, stream);
+            timer_end(L, 0, ti, st);
+            if (rc) return rc;
+            parts = ns;
+        } else {
+            at.nsplit = splits_for(d, a->n, n_pages);
+            at.d_o_part = d.d_o_part + sl * part_o;
+            at.d_lse_part = d.d_lse_part + sl * part_l;
+            const int ti = timer_begin(L, 1, a->n, n_pages * kTile, st);
+            rc = infllm_attn_stage(&at, stream);
+            timer_end(L, 1, ti, st);
+            if (rc) return rc;
+            parts += at.nsplit;
+        }
         // The next fetch (copy stream or DMA engines) must not overtake these reads.  While guesses are being settled
         // no event is needed for that: a fetch ahead never writes a slot of the selection in use, and a fetch behind
         // a selection is issued by a host that has read that selection, which the stream produced after this stage.
@@ -1367,8 +1416,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
             L->global_unmarked = false;
         } else
             L->global_unmarked = side || L->efetch_ok;
-        parts += at.nsplit;
     }
+    L->local_pending = false;
     // Only the joint log-sum-exp is needed on the way to the next selection, and only by the small score launch of
     // step 4, which joins the partial values itself; the merge (output rows and the joint value for the bulk of the
     // scores) runs once that selection is out (step 5b).  The score-decay policy needs the joint value here.

@@ -155,6 +155,11 @@ def attn_fwd(local_args, global_args, out, lse):
                                       lse.data_ptr() if lse is not None else None, _stream()), "infllm_attn_fwd")
 
 
+def attn_stages_fused(local_args, global_args):
+    """Both stages in one launch: one list of tiles, local_args.nsplit partials at local_args' partial buffers."""
+    check(_lib.load().infllm_attn_stages_fused(local_args, global_args, _stream()), "infllm_attn_stages_fused")
+
+
 NOALLOC_MAX_PART_ROWS = 65536       # INFLLM_NOALLOC_MAX_PART_ROWS
 
 

@@ -303,6 +303,55 @@ def test_operator_class_protocol():
     _check_out(attn.get_result()[0], want1)
 
 
+@pytest.mark.parametrize("Lq,n_local,n_glob,nsplit,H,Hkv", [(64, 256, 64 * 3 + 50, 1, 8, 2), (96, 512, 64 * 9, 4, 8, 2), (33, 100, 40, 3, 4, 4),
+                                                        (512, 1024, 64 * 20 + 1, 4, 8, 2), (5, 64, 700, 7, 4, 1)])
+def test_both_stages_in_one_launch_equal_the_oracle_and_the_two_launches(Lq, n_local, n_glob, nsplit, H, Hkv):
+    """infllm_attn_stages_fused: the ring tiles and the pages as one list divided among the key splits (splits that lie
+    in the window, in the pages, or across the seam, where the queries are swapped), against the fp32 oracle and
+    against the two-launch form (same joint softmax; the partials are cut elsewhere, so equal to rounding only)."""
+    ops = _ops()
+    B, cap = 2, (n_local + Lq + 63) // 64 * 64 + 64
+    b0 = 5000
+    lo, b1 = b0 - n_local, b0 + Lq
+    q, qg = _rand((B, H, Lq, D), 60), _rand((B, H, Lq, D), 61)
+    k_win, v_win = _rand((B, Hkv, b1 - lo, D), 62), _rand((B, Hkv, b1 - lo, D), 63)
+    k_g, v_g = _rand((B, Hkv, n_glob, D), 64), _rand((B, Hkv, n_glob, D), 65)
+    ora = MultiStageOracle(q.shape)
+    ora.append(q.float(), k_win.float(), v_win.float(), sliding_window=n_local)
+    ora.append(qg.float(), k_g.float(), v_g.float(), end=True)
+    want, _ = ora.get_result()
+    ring_k = torch.zeros((B, Hkv, cap, D), dtype=torch.bfloat16, device="cuda")
+    ring_v = torch.zeros_like(ring_k)
+    rows = torch.arange(lo, b1) % cap
+    ring_k[:, :, rows] = k_win.cuda()
+    ring_v[:, :, rows] = v_win.cuda()
+    kgd, vgd = k_g.cuda(), v_g.cuda()
+    ent = []
+    for b in range(B):
+        for pos in range(0, n_glob, 64):
+            ent.append((kgd[b].data_ptr() + pos * D * 2, vgd[b].data_ptr() + pos * D * 2, n_glob * D, min(64, n_glob - pos)))
+    n_pages = len(ent) // B
+    arr = ops.make_pages(ent)
+    import ctypes
+    host = torch.empty((len(ent) * 32,), dtype=torch.uint8)
+    ctypes.memmove(host.data_ptr(), arr, len(ent) * 32)
+    pages = host.cuda()
+    qd, qgd = q.cuda(), qg.cuda()
+    o_part = torch.empty((2 * nsplit, B, H, Lq, D), dtype=torch.float16, device="cuda")
+    lse_part = torch.empty((2 * nsplit, B, H, Lq), dtype=torch.float32, device="cuda")
+    la = ops.linear_stage_args(qd, ring_k, ring_v, o_part[:nsplit], lse_part[:nsplit], cap=cap, j_lo=lo, j_hi=b1, mask=ops.MASK_WINDOW,
+                               offset=b0, window=n_local, nsplit=nsplit)
+    ga = ops.paged_stage_args(qgd, pages, n_pages, Hkv, o_part[nsplit:], lse_part[nsplit:], nsplit=nsplit)
+    two, two_lse = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda"), torch.empty((B, H, Lq), device="cuda")
+    ops.attn_fwd(la, ga, two, two_lse)
+    ops.attn_stages_fused(la, ga)
+    one, one_lse = torch.empty_like(two), torch.empty_like(two_lse)
+    ops.attn_merge(o_part[:nsplit], lse_part[:nsplit], nsplit, one, one_lse)
+    _check_out(one, want)
+    assert torch.allclose(one_lse, two_lse, atol=1e-3)
+    assert float((one.float() - two.float()).abs().max()) <= 2.0 ** -6 * max(1.0, float(two.float().abs().max()))
+
+
 # ----------------------------------------------------------------- retrieval
 @pytest.mark.parametrize("N,k", [(17, 16), (991, 16), (8192, 16), (5000, 64), (40, 1), (8194, 16), (16384, 64), (20000, 16),
                                  (3000, 1024), (1024, 1024), (2049, 3)])

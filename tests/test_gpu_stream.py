@@ -22,6 +22,20 @@ def test_small_geometry_follows_oracle(calls):
     assert cm.num_global_block > SMALL["topk"]            # retrieval was exercised
 
 
+def test_both_stages_in_one_launch_follow_the_oracle(monkeypatch):
+    """INFLLM_FUSED_STAGES=1: the local and the global stage of every block as one launch over one list of tiles
+    (infllm_attn_stages_fused) - same acceptance against the oracle, at the small and at the reference geometry, and
+    the same discrete trajectory as the two-launch order."""
+    monkeypatch.setenv("INFLLM_FUSED_STAGES", "1")
+    cm, _, _ = compare(1500, [700, 1, 1, 798], H=8, Hkv=2, base=1e4, seed=41, B=2, **SMALL)
+    assert cm.num_global_block > SMALL["topk"]
+    T = 4096 + 2048
+    cm1, _, _ = compare(T, [4096, 2048], H=32, Hkv=8, base=1e6, seed=42, **REFERENCE)
+    monkeypatch.delenv("INFLLM_FUSED_STAGES")
+    cm2, _, _ = compare(T, [4096, 2048], H=32, Hkv=8, base=1e6, seed=42, **REFERENCE)
+    assert [b["order"] for b in cm1.trace_blocks] == [b["order"] for b in cm2.trace_blocks] and cm1.stats == cm2.stats
+
+
 def test_score_decay_policy_follows_oracle():
     """cache_strategy lru-s: evictions are decided by the decayed attention mass each cached unit received
     (context_manager.py:454-470), which the device computes and the host reads back once per block."""
