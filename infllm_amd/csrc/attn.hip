@@ -20,6 +20,10 @@
 
 #include "common.h"
 
+#include <cstddef>
+#include <cstring>
+#include <type_traits>
+
 namespace {
 
 constexpr int kWaves = 8;                  // 2 per SIMD inside ONE workgroup: a K/V tile in LDS feeds 256 query rows
@@ -115,8 +119,24 @@ struct IntC {
 // list of tiles that the key splits divide between them (one set of partials, one fixed cost instead of two).
 enum { kLinear = 0, kPaged = 1, kBoth = 2 };
 
-template <int MODE>
-__global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a, infllm_attn_args a2, StageGeom geo) {
+// The page table can ride in the launch itself (INLINE): the host passes up to kInlinePages entries by value, and the
+// kernel reads them where they lie in its argument segment - scalar loads through the constant address space, like the
+// table in device memory, but no kernel has to run beforehand to put it there.  The parameter is never touched as a
+// C++ object (that would copy it to scratch memory for the dynamic index).
+constexpr int kInlinePages = 64;
+struct InlinePages {
+    infllm_page p[kInlinePages];
+};
+struct NoInlinePages {};
+struct KernargLayout {                     // the arguments as the launch lays them out: in order, naturally aligned
+    infllm_attn_args a, a2;
+    StageGeom geo;
+    InlinePages pages;
+};
+
+template <int MODE, bool INLINE = false>
+__global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_args a, infllm_attn_args a2, StageGeom geo,
+                                                                 std::conditional_t<INLINE, InlinePages, NoInlinePages>) {
     constexpr bool HAS_LIN = MODE != kPaged, HAS_PAG = MODE != kLinear;
     const infllm_attn_args &ap = MODE == kBoth ? a2 : a;                 // the paged stage's arguments
     extern __shared__ __attribute__((aligned(16))) char lds_dyn[];      // kStages K tiles, then kStages V tiles
@@ -243,8 +263,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     // The page table is read through the constant address space: the index is wave-uniform, so these become scalar
     // loads.  As vector loads they would share the vmcnt counter with the tile transfers, and waiting for a page
     // entry would wait for every tile in flight.  The table is written by an earlier kernel and is read-only here.
-    const __attribute__((address_space(4))) infllm_page *page_table =
-        (const __attribute__((address_space(4))) infllm_page *)(uintptr_t)ap.d_pages + (int64_t)b * n_pag;
+    const __attribute__((address_space(4))) infllm_page *page_table;
+    if constexpr (INLINE)
+        page_table = (const __attribute__((address_space(4))) infllm_page *)((const __attribute__((address_space(4))) char *)
+                                                                             __builtin_amdgcn_kernarg_segment_ptr() +
+                                                                             offsetof(KernargLayout, pages)) + (int64_t)b * n_pag;
+    else
+        page_table = (const __attribute__((address_space(4))) infllm_page *)(uintptr_t)ap.d_pages + (int64_t)b * n_pag;
     auto load_tile = [&](int u, int buf) {     // list index; linear tiles are requested in ascending order
         const bf16_t *kbase, *vbase;
         int row_lo, row_hi;                   // valid rows of this tile: [row_lo, row_hi)
@@ -703,8 +728,9 @@ int check_common(const infllm_attn_args *a) {
     return 0;
 }
 
-// mode: kLinear (a), kPaged (a), kBoth (a = linear stage, a2 = paged stage)
-int launch_stage(int mode, const infllm_attn_args *a, const infllm_attn_args *a2, void *stream) {
+// mode: kLinear (a), kPaged (a), kBoth (a = linear stage, a2 = paged stage); h_pages: NULL, or the paged stage's table
+// [B, n_pages] in HOST memory, B * n_pages <= kInlinePages, which then travels in the launch (d_pages is not read)
+int launch_stage(int mode, const infllm_attn_args *a, const infllm_attn_args *a2, void *stream, const infllm_page *h_pages = nullptr) {
     const int G = a->H / a->Hkv;
     const int n_tasks = ((a->Lq + kQTile - 1) / kQTile) * G;
     dim3 grid((n_tasks + kWaves - 1) / kWaves, a->B * a->Hkv, a->nsplit);
@@ -715,6 +741,25 @@ int launch_stage(int mode, const infllm_attn_args *a, const infllm_attn_args *a2
     if (mode != kPaged) geo.cap_tiles = fast_div((uint32_t)std::min<int64_t>(a->cap / kTile, 1ll << 31));
     constexpr size_t lds_bytes = 2 * kStages * kTileBytes;
     static bool lds_set[3] = {false, false, false};           // dynamic LDS above 64 KiB must be enabled once per kernel
+    const infllm_attn_args &second = a2 ? *a2 : *a;
+    if (h_pages) {
+        const infllm_attn_args &pg = mode == kBoth ? second : *a;
+        INFLLM_REQUIRE(mode != kLinear && pg.n_pages >= 0 && (int64_t)pg.B * pg.n_pages <= kInlinePages,
+                       "attn_stage: %d x %d pages do not fit a launch", pg.B, pg.n_pages);
+        static bool lds_set_inline[3] = {false, false, false};
+        const void *fn = mode == kPaged ? (const void *)attn_stage_kernel<kPaged, true> : (const void *)attn_stage_kernel<kBoth, true>;
+        if (!lds_set_inline[mode]) {
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
+            lds_set_inline[mode] = true;
+        }
+        InlinePages table;
+        memcpy(table.p, h_pages, sizeof(infllm_page) * pg.B * pg.n_pages);
+        if (mode == kPaged) hipLaunchKernelGGL((attn_stage_kernel<kPaged, true>), grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo, table);
+        else hipLaunchKernelGGL((attn_stage_kernel<kBoth, true>), grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo, table);
+        INFLLM_CHECK_LAUNCH("attn_stage");
+        return 0;
+    }
     const void *fn = mode == kLinear ? (const void *)attn_stage_kernel<kLinear>
                      : mode == kPaged ? (const void *)attn_stage_kernel<kPaged> : (const void *)attn_stage_kernel<kBoth>;
     if (!lds_set[mode]) {
@@ -722,10 +767,9 @@ int launch_stage(int mode, const infllm_attn_args *a, const infllm_attn_args *a2
         if (e != hipSuccess) return infllm_fail(-2, "attn_stage: %s", hipGetErrorString(e));
         lds_set[mode] = true;
     }
-    const infllm_attn_args &second = a2 ? *a2 : *a;
-    if (mode == kLinear) hipLaunchKernelGGL(attn_stage_kernel<kLinear>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo);
-    else if (mode == kPaged) hipLaunchKernelGGL(attn_stage_kernel<kPaged>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo);
-    else hipLaunchKernelGGL(attn_stage_kernel<kBoth>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo);
+    if (mode == kLinear) hipLaunchKernelGGL(attn_stage_kernel<kLinear>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo, NoInlinePages{});
+    else if (mode == kPaged) hipLaunchKernelGGL(attn_stage_kernel<kPaged>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo, NoInlinePages{});
+    else hipLaunchKernelGGL(attn_stage_kernel<kBoth>, grid, dim3(kThreads), lds_bytes, (hipStream_t)stream, *a, second, geo, NoInlinePages{});
     INFLLM_CHECK_LAUNCH("attn_stage");
     return 0;
 }
@@ -743,6 +787,24 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
     }
     rc = check_linear_stage(a);
     return rc ? rc : launch_stage(kLinear, a, nullptr, stream);
+}
+
+// library-internal: the paged stage (local == NULL) or both stages in one launch, with the page table [B, n_pages]
+// given in HOST memory and carried by the launch; global->d_pages is not read.  B * n_pages <= infllm_inline_page_limit().
+int infllm_inline_page_limit() { return kInlinePages; }
+int infllm_attn_paged_inline(const infllm_attn_args *local, const infllm_attn_args *global, const infllm_page *h_pages, void *stream) {
+    INFLLM_REQUIRE(global && h_pages && global->d_o_part && global->d_lse_part, "attn_paged_inline: null argument");
+    int rc = check_common(global);
+    if (rc) return rc;
+    if (!local) return launch_stage(kPaged, global, nullptr, stream, h_pages);
+    INFLLM_REQUIRE(local->d_o_part && local->d_lse_part && !local->d_pages, "attn_paged_inline: bad local stage");
+    INFLLM_REQUIRE(local->B == global->B && local->H == global->H && local->Hkv == global->Hkv && local->Lq == global->Lq &&
+                       local->softmax_scale == global->softmax_scale,
+                   "attn_paged_inline: the two stages disagree");
+    rc = check_common(local);
+    if (rc) return rc;
+    rc = check_linear_stage(local);
+    return rc ? rc : launch_stage(kBoth, local, global, stream, h_pages);
 }
 
 extern "C" int infllm_attn_stages_fused(const infllm_attn_args *local, const infllm_attn_args *global, void *stream) {

@@ -141,6 +141,8 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_inline_page_limit();
+int infllm_attn_paged_inline(const infllm_attn_args *local, const infllm_attn_args *global, const infllm_page *h_pages, void *stream);
 int infllm_score_new_rank(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores, const int32_t *d_cand,
                           int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx, int32_t *d_flag,
                           int32_t flag_value, void *stream);
@@ -1243,6 +1245,43 @@ extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, voi
     return n_miss;
 }
 
+namespace {
+
+// The global stage's page table of batch row u, on the host: units (by slot) | init tokens | overflow remainder of the
+// ring.  Writes at most `room` entries to pg and returns how many the row has (slots are checked by the caller).
+int host_pages(const infllm_layer_desc &d, const infllm_back_args *a, int u, int64_t overflow_end, infllm_page *pg, int room) {
+    const int bs = d.block_size;
+    const int64_t unit_elems = (int64_t)d.Hkv * bs * kD, slot_elems = 2 * unit_elems;
+    int n = 0;
+    auto push = [&](const bf16_t *k, const bf16_t *v, int64_t hs, int valid) {
+        if (n < room) pg[n] = infllm_page{k, v, hs, valid, 0};
+        ++n;
+    };
+    for (int s = 0; s < a->n_sel; ++s) {
+        const int sl = a->h_sel_slots[u * a->n_sel + s];
+        const bf16_t *kb = (const bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + sl) * slot_elems;
+        for (int t0 = 0; t0 < bs; t0 += kTile)
+            push(kb + (int64_t)t0 * kD, kb + unit_elems + (int64_t)t0 * kD, (int64_t)bs * kD, bs - t0 < kTile ? bs - t0 : kTile);
+    }
+    const bf16_t *ik = (const bf16_t *)d.d_init_kv + (int64_t)u * 2 * d.Hkv * d.init_cap * kD;
+    const bf16_t *iv = ik + (int64_t)d.Hkv * d.init_cap * kD;
+    for (int t0 = 0; t0 < a->init_len; t0 += kTile)
+        push(ik + (int64_t)t0 * kD, iv + (int64_t)t0 * kD, d.init_cap * kD, a->init_len - t0 < kTile ? a->init_len - t0 : kTile);
+    const bf16_t *rk = (const bf16_t *)d.d_ring_k_raw + (int64_t)u * d.Hkv * d.ring_cap * kD;
+    const bf16_t *rv = (const bf16_t *)d.d_ring_v + (int64_t)u * d.Hkv * d.ring_cap * kD;
+    for (int64_t pos = a->cursor; pos < overflow_end;) {
+        const int64_t row = pos % d.ring_cap;
+        int64_t len = overflow_end - pos;
+        if (len > kTile) len = kTile;
+        if (len > d.ring_cap - row) len = d.ring_cap - row;
+        push(rk + row * kD, rv + row * kD, d.ring_cap * kD, (int)len);
+        pos += len;
+    }
+    return n;
+}
+
+}  // namespace
+
 extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream) {
     INFLLM_REQUIRE(layer && a, "block_back: null argument");
     Layer *L = (Layer *)layer;
@@ -1273,7 +1312,28 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     //         wait for the fetch, so it is out of the way when the units arrive)
     const int64_t overflow_end = b1 - d.n_local > a->cursor ? b1 - d.n_local : a->cursor;
     int n_pages = 0;
-    if (d.B * a->n_sel <= kPageJobSlots) {
+    for (int i = 0; i < d.B * a->n_sel; ++i)
+        INFLLM_REQUIRE(a->h_sel_slots[i] >= 0 && a->h_sel_slots[i] < d.max_cached, "block_back: slot %d out of range", a->h_sel_slots[i]);
+    // A table of up to 64 entries travels in the launch of the stage that reads it; a longer one is written by a small
+    // kernel from the slot list, or uploaded.  INFLLM_PAGE_TABLE_KERNEL=1 keeps the kernel for short tables too.
+    infllm_page inline_pages[64];
+    bool pages_inline = false;
+    static const bool inline_allowed = [] { const char *e = getenv("INFLLM_PAGE_TABLE_KERNEL"); return !(e && e[0] && e[0] != '0'); }();
+    if (inline_allowed) {
+        const int room = infllm_inline_page_limit() < 64 ? infllm_inline_page_limit() : 64;
+        int n0 = host_pages(d, a, 0, overflow_end, inline_pages, room);
+        if (n0 > 0 && (int64_t)d.B * n0 <= room) {
+            INFLLM_REQUIRE(n0 <= d.max_pages, "block_back: %d pages exceed the table (%d)", n0, d.max_pages);
+            for (int u = 1; u < d.B; ++u) {
+                const int nu = host_pages(d, a, u, overflow_end, inline_pages + (int64_t)u * n0, n0);
+                INFLLM_REQUIRE(nu == n0, "block_back: batch rows disagree on the page count");
+            }
+            n_pages = n0;
+            pages_inline = true;
+        }
+    }
+    if (pages_inline) {
+    } else if (d.B * a->n_sel <= kPageJobSlots) {
         PageJob j{};
         j.B = d.B; j.Hkv = d.Hkv; j.bs = bs; j.max_cached = d.max_cached; j.n_sel = a->n_sel; j.init_len = a->init_len;
         j.n_unit_pages = a->n_sel * ((bs + kTile - 1) / kTile);
@@ -1393,7 +1453,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
             at.d_o_part = d.d_o_part; at.d_lse_part = d.d_lse_part;
             // timed as the block's dominant launch: its key count is the window plus the pages
             const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo) + n_pages * kTile, st);
-            rc = infllm_attn_stages_fused(&lt, &at, stream);
+            rc = pages_inline ? infllm_attn_paged_inline(&lt, &at, inline_pages, stream) : infllm_attn_stages_fused(&lt, &at, stream);
             timer_end(L, 0, ti, st);
             if (rc) return rc;
             parts = ns;
@@ -1402,7 +1462,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
             at.d_o_part = d.d_o_part + sl * part_o;
             at.d_lse_part = d.d_lse_part + sl * part_l;
             const int ti = timer_begin(L, 1, a->n, n_pages * kTile, st);
-            rc = infllm_attn_stage(&at, stream);
+            rc = pages_inline ? infllm_attn_paged_inline(nullptr, &at, inline_pages, stream) : infllm_attn_stage(&at, stream);
             timer_end(L, 1, ti, st);
             if (rc) return rc;
             parts += at.nsplit;

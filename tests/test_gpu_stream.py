@@ -36,6 +36,25 @@ def test_both_stages_in_one_launch_follow_the_oracle(monkeypatch):
     assert [b["order"] for b in cm1.trace_blocks] == [b["order"] for b in cm2.trace_blocks] and cm1.stats == cm2.stats
 
 
+def test_page_table_in_the_launch_gives_the_bits_of_the_table_in_memory(monkeypatch):
+    """The global stage reads its page table (selected units | init tokens | overflow rows of the ring) from the
+    arguments of its own launch when the table has at most 64 entries; INFLLM_PAGE_TABLE_KERNEL=1 keeps the small
+    kernel that writes the table to device memory first.  Same entries either way: outputs bit for bit, at the small
+    geometry with two batch rows (2 x 7 pages) and at the reference geometry (37 pages)."""
+    def run(kernel, T, calls, H, Hkv, base, seed, B, kw):
+        if kernel:
+            monkeypatch.setenv("INFLLM_PAGE_TABLE_KERNEL", "1")
+        else:
+            monkeypatch.delenv("INFLLM_PAGE_TABLE_KERNEL", raising=False)
+        q, k, v = make_stream(T, H, Hkv, seed, B=B)
+        out, cm = run_gpu(q, k, v, calls, base, **kw)
+        return out, [b["order"] for b in cm.trace_blocks]
+
+    for args in ((1500, [700, 1, 1, 798], 8, 2, 1e4, 45, 2, SMALL), (4096 + 2048, [4096, 2048], 32, 8, 1e6, 46, 1, REFERENCE)):
+        a, b = run(False, *args), run(True, *args)
+        assert torch.equal(a[0], b[0]) and a[1] == b[1] and len(a[1]) > 10
+
+
 def test_score_decay_policy_follows_oracle():
     """cache_strategy lru-s: evictions are decided by the decayed attention mass each cached unit received
     (context_manager.py:454-470), which the device computes and the host reads back once per block."""
