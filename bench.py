@@ -371,7 +371,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": counted_traffic("attn_stage__stream32k.hbm_bytes.txt", "local_stage_traffic_bytes"),
-                     "kernel": "attn_stage_kernel<false> (local stage, 512 q x 4096 visible keys x 32 heads)",
+                     "kernel": "attn_stage_kernel<0, false> (local stage, 512 q x 4096 visible keys x 32 heads)",
                      "avg_launch_ms": avg_ms, "launches_timed": len(steady),
                      "global_stage_avg_ms": sum(glob) / max(len(glob), 1)},
         "cache": cm_stats,
