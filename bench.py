@@ -351,9 +351,11 @@ def main():
 
     # dominant kernel: the local (sliding-window) attention stage; steady-state launches only
     exc, n_local = KNOBS["exc_block_size"], KNOBS["n_local"]
-    steady = [ms for r in runs for ms, nq, nk in r[0] if nq == exc and nk == n_local + exc]
+    # (one launch covers every block of an append() call: its queries are the call's, each seeing n_local keys)
+    q_launch = max([nq for r in runs for ms, nq, nk in r[0]] or [exc])
+    steady = [ms for r in runs for ms, nq, nk in r[0] if nq == q_launch and nk == n_local + q_launch]
     avg_ms = sum(steady) / max(len(steady), 1)
-    flops_per_launch = 4.0 * H * D * exc * n_local
+    flops_per_launch = 4.0 * H * D * q_launch * n_local
     achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12 if steady else 0.0
     glob_keys = KNOBS["topk"] * KNOBS["block_size"] + KNOBS["n_init"] + exc
     glob = [ms for r in runs for ms, nq, nk in r[1] if nq == exc and nk == glob_keys]
@@ -371,7 +373,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": counted_traffic("attn_stage__stream32k.hbm_bytes.txt", "local_stage_traffic_bytes"),
-                     "kernel": "attn_stage_kernel<0, false> (local stage, 512 q x 4096 visible keys x 32 heads)",
+                     "kernel": f"attn_stage_kernel<0, false> (local stage, {q_launch} q x {n_local} visible keys x {H} heads per launch)",
                      "avg_launch_ms": avg_ms, "launches_timed": len(steady),
                      "global_stage_avg_ms": sum(glob) / max(len(glob), 1)},
         "cache": cm_stats,
@@ -379,6 +381,12 @@ def main():
         # were the selection, and how long the main stream still waited for units (the wait itself costs ~6 us)
         "fetch_ahead": {"guesses": guesses[0], "confirmed": guesses[1], "stream_wait_avg_ms": sum(waits) / max(len(waits), 1)},
     }
+    # what the stream as a whole is bound by: the missed units' way from pinned host memory over PCIe (repairs of wrong
+    # guesses come on top of the misses counted here)
+    unit_bytes = 2 * HKV * KNOBS["block_size"] * D * 2
+    res["host_link"] = {"missed_units_per_step": cm_stats["misses"], "bytes_per_step": cm_stats["misses"] * unit_bytes,
+                        "avg_GBps": cm_stats["misses"] * unit_bytes / (dt / args.steps) / 1e9,
+                        "note": "PCIe 5.0 x16: 64 GB/s raw; 8 DMA engines move 13 x 512 KiB units at 54 GB/s on an idle GPU, 44 GB/s beside the stream's kernels"}
     if not args.no_hbm_leg:
         res["roofline_hbm"] = hbm_leg(dev)
     if args.cpu_tokens > 0:

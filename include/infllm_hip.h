@@ -382,6 +382,36 @@ typedef struct {
     int32_t n_next, flags;                            /* INFLLM_NO_RETRIEVAL: the caller supplies the selection */
 } infllm_front_args;
 int infllm_block_front(void *layer, const infllm_front_args *a, void *stream);
+
+/* A whole append() call prepared in one go.  ContextManager.append (context_manager.py:749-798) works its tokens off
+ * in execution blocks, and the sliding-window half of a block's attention (context_manager.py:474-482) needs nothing
+ * but the block's own rows and the rows before it - so, once the call's rows are in the rings, it can run for several
+ * blocks in one launch, ahead of the blocks' retrieval:
+ *
+ *   infllm_layer_set_batch  hands the layer the buffers this takes (the caller's allocation, like the workspaces of
+ *                           infllm_layer_desc): rotated queries of a call, the blocks' mean queries and the local
+ *                           stage's partial rows.  Needs exc_block_size to be a multiple of 32.
+ *   infllm_call_front       a->d_q/d_k/d_v are the rows of the next a->n <= max_tokens tokens (a->b0 the first one's
+ *                           position); runs the prologue for all of them (the rings must have room: ring_cap >=
+ *                           a->b0 - cursor + a->n), every block's mean query, the first block's retrieval when
+ *                           a->n_units > topk.  The blocks then go through infllm_block_front / select / back as
+ *                           ever, in order; block_front finds their prologue done (its d_q / d_k / d_v and
+ *                           next-block pointers are not read, n_next still says whether a block of this call
+ *                           follows) and launches the local stage for group_blocks blocks at a time, at the first
+ *                           block of each group.  infllm_layer_flush ends the call.
+ * Without these two calls every block runs its own prologue and local stage (block_front). */
+typedef struct {
+    void *d_q_loc, *d_q_glb;          /* [B, H, max_tokens, 128] bf16 each */
+    float *d_qpart;                   /* [B, ceil(max_tokens / 16), H*128] */
+    float *d_qbar;                    /* [ceil(max_tokens / exc), B, H*128] */
+    uint16_t *d_o_part;               /* [part_rows, 128] fp16: partial rows of the local stage, by block */
+    float *d_lse_part;                /* [part_rows] */
+    int64_t part_rows;                /* >= B * H * exc * max(8, 4 * group_blocks) */
+    int32_t max_tokens;
+    int32_t group_blocks;             /* blocks per local-stage launch (0: 2) */
+} infllm_batch_desc;
+int infllm_layer_set_batch(void *layer, const infllm_batch_desc *b);
+int infllm_call_front(void *layer, const infllm_front_args *a, void *stream);
 int infllm_layer_wait_topk(void *layer);
 
 /* flags of infllm_front_args / infllm_back_args: skip mean query, unit scores and top-k (the selection was made

@@ -91,6 +91,14 @@ class FrontArgs(C.Structure):
     ]
 
 
+class BatchDesc(C.Structure):
+    _fields_ = [
+        ("d_q_loc", c_vp), ("d_q_glb", c_vp), ("d_qpart", c_vp), ("d_qbar", c_vp),
+        ("d_o_part", c_vp), ("d_lse_part", c_vp), ("part_rows", c_i64),
+        ("max_tokens", c_i32), ("group_blocks", c_i32),
+    ]
+
+
 class BackArgs(C.Structure):
     _fields_ = [
         ("n", c_i32), ("n_sel", c_i32), ("b0", c_i64),
@@ -148,6 +156,8 @@ SYMBOLS = {
     "infllm_layer_create": (c_vp, [C.POINTER(LayerDesc)]),
     "infllm_layer_destroy": (c_i32, [c_vp]),
     "infllm_block_front": (c_i32, [c_vp, C.POINTER(FrontArgs), c_vp]),
+    "infllm_layer_set_batch": (c_i32, [c_vp, C.POINTER(BatchDesc)]),
+    "infllm_call_front": (c_i32, [c_vp, C.POINTER(FrontArgs), c_vp]),
     "infllm_layer_wait_topk": (c_i32, [c_vp]),
     "infllm_layer_wait_mass": (c_i32, [c_vp]),
     "infllm_block_fetch": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),

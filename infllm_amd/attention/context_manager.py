@@ -31,6 +31,7 @@ cache policy and fetch) and infllm_block_back, plus infllm_block_prefetch for
 the next block.
 """
 import ctypes
+import os
 
 import torch
 
@@ -39,6 +40,7 @@ from .._lib import BackArgs, FrontArgs, LayerDesc, check
 from ..ops import HEAD_DIM, KEY_TILE
 
 _SIDE_STREAM = None          # one process-wide side stream, like GLOBAL_STREAM (context_manager.py:193)
+_CALL_BUFFERS = {}           # (device, stream, geometry) -> the buffers of a call prepared in one go, see _bind_call_buffers
 _HOST_CHUNK_UNITS = 64       # units per pinned host allocation
 _MAX_SPLITS = 16             # key splits of one attention stage
 _NUM_CUS = 256               # MI355X
@@ -117,6 +119,10 @@ class CachePolicy:
 class ContextManager:
     select_in_steps = False     # True: drive wait / policy / fetch from here (slower), instead of infllm_block_select
     fetch_ahead = True          # start the next block's fetch from its candidates (infllm_block_prefetch)
+    call_tokens = 8192          # tokens of an append() call prepared in one go (prologue, mean queries and the local
+                                # stage of all their blocks: infllm_call_front); 0: every block runs its own.
+                                # INFLLM_CALL_TOKENS overrides it.  Needs exc_block_size to be a multiple of 32.
+    local_group_blocks = 2      # blocks of a prepared call per launch of the local stage (INFLLM_LOCAL_GROUP overrides it)
 
     def __init__(self, position_embedding, n_init, n_local, block_size, max_cached_block, topk, exc_block_size,
                  score_decay=None, fattn=False, repr_topk=1, cache_strategy="lru", chunk_topk_calc=None,
@@ -180,7 +186,11 @@ class ContextManager:
         self.dtype = q.dtype
         self.device = dev
         bs, exc, topk = self.block_size, self.exc_block_size, self.topk
-        cap = self.n_local + 2 * exc + bs          # one block is prepared ahead of the one being attended
+        ct = int(os.environ.get("INFLLM_CALL_TOKENS", self.call_tokens))
+        self._call_tokens = min(ct, 16 * exc) // exc * exc if (ct >= exc and exc % 32 == 0) else 0
+        # the rings hold the local window, the remainder that waits to fill a unit, and what is prepared ahead of the
+        # block being attended: one block, or the rest of a call prepared in one go
+        cap = self.n_local + exc + bs + max(exc, self._call_tokens)
         self.ring_cap = cap = (cap + KEY_TILE - 1) // KEY_TILE * KEY_TILE + KEY_TILE
         bf = dict(dtype=torch.bfloat16, device=dev)
         f32 = dict(dtype=torch.float32, device=dev)
@@ -256,6 +266,7 @@ class ContextManager:
             raise _lib.InfLLMHipError("infllm_layer_create failed: " + (self._lib.infllm_last_error() or b"").decode())
         if self._timing_cap:
             check(self._lib.infllm_layer_timing(self._layer, self._timing_cap, self._timing_stride), "infllm_layer_timing")
+        self._call_stream = None               # stream the call buffers were taken for (they are bound at the first append)
         # argument blocks and host arrays reused by every block
         self._fa, self._ba = FrontArgs(), BackArgs()
         self._sel_slots = (ctypes.c_int32 * (B * max(topk, 1)))()
@@ -294,6 +305,33 @@ class ContextManager:
         self._sa_ref = ctypes.byref(sa)
         self._fa_ref, self._ba_ref = ctypes.byref(self._fa), ctypes.byref(self._ba)
         self.initialized = True
+
+    def _bind_call_buffers(self, stream):
+        """Buffers of a call prepared in one go: the rotated queries of up to call_tokens tokens, the blocks' mean
+        queries and the local stage's partial rows.  They are dead between append() calls, so the layers that work on
+        one stream (one after the other, as the layers of a model do) share one set."""
+        B, H, D, exc, T = self.num_units, self.unit_size, self.dim_head, self.exc_block_size, self._call_tokens
+        group = int(os.environ.get("INFLLM_LOCAL_GROUP", self.local_group_blocks))
+        blocks = max(8, 4 * group)            # partial rows: two groups of blocks, up to two key splits each
+        dev = self.device.index if self.device.index is not None else torch.cuda.current_device()
+        key = (dev, stream, B, H, D, T, exc, blocks)
+        buf = _CALL_BUFFERS.get(key)
+        if buf is None:
+            bf = dict(dtype=torch.bfloat16, device=self.device)
+            f32 = dict(dtype=torch.float32, device=self.device)
+            buf = _CALL_BUFFERS[key] = dict(
+                q_loc=torch.empty((B, H, T, D), **bf), q_glb=torch.empty((B, H, T, D), **bf),
+                qpart=torch.empty((B, (T + 15) // 16, H * D), **f32), qbar=torch.empty((T // exc, B, H * D), **f32),
+                o_part=torch.empty((blocks * B * H * exc, D), dtype=torch.float16, device=self.device),
+                lse_part=torch.empty((blocks * B * H * exc,), **f32))
+        self._call_buf = buf
+        bd = _lib.BatchDesc()
+        bd.d_q_loc, bd.d_q_glb = buf["q_loc"].data_ptr(), buf["q_glb"].data_ptr()
+        bd.d_qpart, bd.d_qbar = buf["qpart"].data_ptr(), buf["qbar"].data_ptr()
+        bd.d_o_part, bd.d_lse_part = buf["o_part"].data_ptr(), buf["lse_part"].data_ptr()
+        bd.part_rows, bd.max_tokens, bd.group_blocks = blocks * B * H * exc, T, group
+        check(self._lib.infllm_layer_set_batch(self._layer, ctypes.byref(bd)), "infllm_layer_set_batch")
+        self._call_stream = stream
 
     def size(self, *args, **kwargs):
         return self.length
@@ -558,6 +596,8 @@ class ContextManager:
         main = torch.cuda.current_stream()
         self._main_raw = main.cuda_stream
         self._copy_raw = _SIDE_STREAM.cuda_stream if self.async_global_stream else self._main_raw
+        if self._call_tokens and self._call_stream != self._main_raw:
+            self._bind_call_buffers(self._main_raw)
         out_ptr, out_step = out.data_ptr(), out.stride(2) * 2
         exc = self.exc_block_size
         use_chunks = self.chunk_topk_calc is not None and input_length > 1      # context_manager.py:749-760
@@ -567,8 +607,20 @@ class ContextManager:
             if cuts[-1] < input_length:
                 cuts.append(input_length)
             cut_i, plan, plan_pos = -1, None, 0
+        call_end = 0
         for st in range(0, input_length, exc):
             n = min(exc, input_length - st)
+            if self._call_tokens and st == call_end:
+                # the next stretch of the call in one go: prologue, mean queries, first retrieval, local stage
+                call_end = min(st + self._call_tokens, input_length)
+                assert self.length + call_end - self.cursor <= self.ring_cap
+                fa.d_q, fa.d_k, fa.d_v = (self._q_ptr + st * self._q_step, self._k_ptr + st * self._k_step,
+                                          self._v_ptr + st * self._v_step)
+                fa.n, fa.n_units, fa.b0 = call_end - st, self.num_global_block, self.length + st
+                fa.flags = _lib.NO_RETRIEVAL if use_chunks else 0
+                check(self._lib.infllm_call_front(self._layer, self._fa_ref, self._main_raw), "infllm_call_front")
+            elif not self._call_tokens:
+                call_end = input_length
             chosen = None
             if use_chunks:
                 if cuts[cut_i + 1] < st + n:
@@ -576,7 +628,7 @@ class ContextManager:
                     plan, plan_pos = self._chunk_topk(q, cuts[cut_i], cuts[cut_i + 1]), 0
                 chosen = plan[plan_pos]
                 plan_pos += 1
-            self._block(st, n, out_ptr + st * out_step, min(exc, input_length - st - n), chosen)
+            self._block(st, n, out_ptr + st * out_step, min(exc, call_end - st - n), chosen)
         self.length += input_length
         check(self._lib.infllm_layer_flush(self._layer, self._copy_raw), "infllm_layer_flush")
         if self.perhead:

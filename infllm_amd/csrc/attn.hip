@@ -69,6 +69,12 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f) { return 
 struct StageGeom {
     FastDiv gx, gy, hkv, group, nsplit, cap_tiles;
     int32_t n_tasks;
+    // Partial rows by execution block (out_exc > 0): the queries are those of several consecutive execution blocks of
+    // out_exc rows (the last one may be shorter), and block k's partials form a [nsplit, B, H, n_k, 128] array of their
+    // own at row k * out_block_rows of the partial buffers - where the merge of that block expects them.
+    int32_t out_exc;
+    int64_t out_block_rows;
+    FastDiv out_exc_div;
 };
 
 // LDS layouts.  Tiles go from global memory straight into LDS (global_load_lds_dwordx4: lane l of a
@@ -515,7 +521,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     const float l_tot = l_run + wave_xor32(l_run);
     const int qi = i0 + col;
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int64_t row0 = (((int64_t)split * a.B + b) * a.H + h) * a.Lq + i0;      // row of this wave's first query
+    int64_t row0 = (((int64_t)split * a.B + b) * a.H + h) * a.Lq + i0;            // row of this wave's first query
+    int rows_left = a.Lq - i0;                                                     // valid queries of this tile
+    if (geo.out_exc > 0) {                    // a query tile lies inside one execution block (out_exc is a multiple of the tile)
+        const int blk = (int)fdiv(i0, geo.out_exc_div), in_blk = i0 - blk * geo.out_exc;
+        const int n_blk = min(geo.out_exc, a.Lq - blk * geo.out_exc);
+        row0 = (int64_t)blk * geo.out_block_rows + (((int64_t)split * a.B + b) * a.H + h) * n_blk + in_blk;
+        rows_left = n_blk - in_blk;
+    }
     const int64_t row = row0 + col;
     {
         // fp16 keeps 11 bits of a value that ends up rounded to bf16's 8, and halves what the partials cost in HBM
@@ -531,7 +544,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                 const int chunk = dt * 4 + q4;                                     // 16-byte chunk of the row; grp picks its half
                 *(f16x4 *)(stage + col * (kD * 2) + ((chunk ^ col) & 15) * 16 + grp * 8) = o4;
             }
-        const int rows_left = a.Lq - i0;                                           // valid queries of this tile
         const int piece = lane & 15;
         _Float16 *o_part = (_Float16 *)a.d_o_part;
 #pragma unroll
@@ -545,10 +557,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run * scale + log2f(l_tot) : -INFINITY;
 }
 
+// The partials of a merge may lie in two places: the first n_first of them behind the pointers the kernel is given,
+// the rest wherever the second stage wrote them.  skip_l / skip_o are what has to be added to an index into the first
+// buffers (log-sum-exps; fp16 elements beyond the row term) to land in the second.
+struct PartSets {
+    int32_t n_first;
+    int64_t skip_l, skip_o;
+    __device__ __forceinline__ int64_t l(int p, int64_t rows) const { return (int64_t)p * rows + (p >= n_first ? skip_l : 0); }
+    __device__ __forceinline__ int64_t o(int p) const { return p >= n_first ? skip_o : 0; }
+};
+
 // one thread per (row, 8 dims): P fp16 partials -> bf16 output row + final lse
 __global__ __launch_bounds__(256) void attn_merge_kernel(const _Float16 *o_part, const float *lse_part, int P, int B, int H,
                                                          int Lq, bf16_t *out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
-                                                         float *lse_out) {
+                                                         float *lse_out, PartSets ps) {
     const int64_t rows = (int64_t)B * H * Lq;
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t row = e >> 4;
@@ -560,7 +582,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const _Float16 *o_part,
     for (int p0 = 0; p0 < P; p0 += 8) {
         float l8[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) l8[i] = p0 + i < P ? lse_part[(p0 + i) * rows + row] : -INFINITY;
+        for (int i = 0; i < 8; ++i) l8[i] = p0 + i < P ? lse_part[ps.l(p0 + i, rows) + row] : -INFINITY;
 #pragma unroll
         for (int i = 0; i < 8; ++i) m = fmaxf(m, l8[i]);
     }
@@ -575,8 +597,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const _Float16 *o_part,
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const bool on = p0 + i < P;
-                l8[i] = on ? lse_part[(p0 + i) * rows + row] : -INFINITY;
-                o8[i] = on ? *(const f16x8 *)(o_part + ((p0 + i) * rows + row) * kD + c * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                l8[i] = on ? lse_part[ps.l(p0 + i, rows) + row] : -INFINITY;
+                o8[i] = on ? *(const f16x8 *)(o_part + (ps.l(p0 + i, rows) + row) * kD + ps.o(p0 + i) + c * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -596,14 +618,14 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(const _Float16 *o_part,
 }
 
 // the log-sum-exp half of the merge alone: one thread per row
-__global__ __launch_bounds__(256) void attn_merge_lse_kernel(const float *lse_part, int P, int64_t rows, float *lse_out) {
+__global__ __launch_bounds__(256) void attn_merge_lse_kernel(const float *lse_part, int P, int64_t rows, float *lse_out, PartSets ps) {
     const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (row >= rows) return;
     float m = -INFINITY, den = 0.f;
     for (int p0 = 0; p0 < P; p0 += 8) {                 // online over batches of 8 independent loads
         float l8[8], m8 = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) l8[i] = p0 + i < P ? lse_part[(p0 + i) * rows + row] : -INFINITY;
+        for (int i = 0; i < 8; ++i) l8[i] = p0 + i < P ? lse_part[ps.l(p0 + i, rows) + row] : -INFINITY;
 #pragma unroll
         for (int i = 0; i < 8; ++i) m8 = fmaxf(m8, l8[i]);
         if (m8 == -INFINITY) continue;
@@ -632,7 +654,7 @@ __device__ __forceinline__ float group16_sum(float v) {
 
 __global__ __launch_bounds__(256) void attn_merge_wide_kernel(const _Float16 *o_part, const float *lse_part, int P, int B, int H,
                                                               int Lq, bf16_t *out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
-                                                              float *lse_out) {
+                                                              float *lse_out, PartSets ps) {
     const int64_t rows = (int64_t)B * H * Lq;
     const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;       // (row, 8 dims)
     const int pl = threadIdx.x & 15;
@@ -647,8 +669,8 @@ __global__ __launch_bounds__(256) void attn_merge_wide_kernel(const _Float16 *o_
     for (int i = 0; i < kMine; ++i) {
         const int p = pl + 16 * i;
         const bool on = p < P;
-        l[i] = on ? lse_part[p * rows + row] : -INFINITY;
-        o[i] = on ? *(const f16x8 *)(o_part + (p * rows + row) * kD + c * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        l[i] = on ? lse_part[ps.l(p, rows) + row] : -INFINITY;
+        o[i] = on ? *(const f16x8 *)(o_part + (ps.l(p, rows) + row) * kD + ps.o(p) + c * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
         m = fmaxf(m, l[i]);
     }
     m = group16_max(m);
@@ -674,7 +696,7 @@ __global__ __launch_bounds__(256) void attn_merge_wide_kernel(const _Float16 *o_
     if (c == 0 && lse_out) lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
 }
 
-__global__ __launch_bounds__(256) void attn_merge_lse_wide_kernel(const float *lse_part, int P, int64_t rows, float *lse_out) {
+__global__ __launch_bounds__(256) void attn_merge_lse_wide_kernel(const float *lse_part, int P, int64_t rows, float *lse_out, PartSets ps) {
     const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
     const int pl = threadIdx.x & 15;
     if (row >= rows) return;
@@ -683,7 +705,7 @@ __global__ __launch_bounds__(256) void attn_merge_lse_wide_kernel(const float *l
 #pragma unroll
     for (int i = 0; i < kMine; ++i) {
         const int p = pl + 16 * i;
-        l[i] = p < P ? lse_part[p * rows + row] : -INFINITY;
+        l[i] = p < P ? lse_part[ps.l(p, rows) + row] : -INFINITY;
         m = fmaxf(m, l[i]);
     }
     m = group16_max(m);
@@ -730,13 +752,14 @@ int check_common(const infllm_attn_args *a) {
 
 // mode: kLinear (a), kPaged (a), kBoth (a = linear stage, a2 = paged stage); h_pages: NULL, or the paged stage's table
 // [B, n_pages] in HOST memory, B * n_pages <= kInlinePages, which then travels in the launch (d_pages is not read)
-int launch_stage(int mode, const infllm_attn_args *a, const infllm_attn_args *a2, void *stream, const infllm_page *h_pages = nullptr) {
+int launch_stage(int mode, const infllm_attn_args *a, const infllm_attn_args *a2, void *stream, const infllm_page *h_pages = nullptr,
+                 int out_exc = 0, int64_t out_block_rows = 0) {
     const int G = a->H / a->Hkv;
     const int n_tasks = ((a->Lq + kQTile - 1) / kQTile) * G;
     dim3 grid((n_tasks + kWaves - 1) / kWaves, a->B * a->Hkv, a->nsplit);
     INFLLM_REQUIRE((int64_t)grid.x * grid.y * grid.z < (1ll << 31), "attn_stage: grid too large");
     StageGeom geo{fast_div(grid.x), fast_div(grid.y), fast_div((uint32_t)a->Hkv), fast_div((uint32_t)G),
-                  fast_div((uint32_t)a->nsplit), fast_div(1), n_tasks};
+                  fast_div((uint32_t)a->nsplit), fast_div(1), n_tasks, out_exc, out_block_rows, fast_div((uint32_t)(out_exc > 0 ? out_exc : 1))};
     // tile indices stay below 2^30, so any ring of 2^31 tiles or more never wraps: one divisor stands for all of them
     if (mode != kPaged) geo.cap_tiles = fast_div((uint32_t)std::min<int64_t>(a->cap / kTile, 1ll << 31));
     constexpr size_t lds_bytes = 2 * kStages * kTileBytes;
@@ -787,6 +810,19 @@ extern "C" int infllm_attn_stage(const infllm_attn_args *a, void *stream) {
     }
     rc = check_linear_stage(a);
     return rc ? rc : launch_stage(kLinear, a, nullptr, stream);
+}
+
+// library-internal: a linear stage over the queries of several consecutive execution blocks of `exc` rows (the last
+// may be shorter); block k's partial rows and log-sum-exps start at row k * block_rows of d_o_part / d_lse_part and
+// are laid out [nsplit, B, H, n_k, 128] / [nsplit, B, H, n_k], as infllm_attn_merge takes them for that block.
+int infllm_attn_stage_blocked(const infllm_attn_args *a, int32_t exc, int64_t block_rows, void *stream) {
+    INFLLM_REQUIRE(a && a->d_o_part && a->d_lse_part && !a->d_pages, "attn_stage_blocked: null argument or paged source");
+    INFLLM_REQUIRE(exc > 0 && exc % kQTile == 0, "attn_stage_blocked: blocks of %d rows are not whole query tiles", exc);
+    INFLLM_REQUIRE(block_rows >= (int64_t)a->nsplit * a->B * a->H * (a->Lq < exc ? a->Lq : exc), "attn_stage_blocked: block stride too small");
+    int rc = check_common(a);
+    if (rc) return rc;
+    rc = check_linear_stage(a);
+    return rc ? rc : launch_stage(kLinear, a, nullptr, stream, nullptr, exc, block_rows);
 }
 
 // library-internal: the paged stage (local == NULL) or both stages in one launch, with the page table [B, n_pages]
@@ -905,10 +941,22 @@ extern "C" int infllm_attn_fwd_noalloc(const infllm_attn_args *local, const infl
     return infllm_attn_fwd(local ? &l : nullptr, global ? &g : nullptr, d_out, o_sb, o_sh, o_sl, d_lse, stream);
 }
 
-extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
-                                 int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
-                                 void *stream) {
+// library-internal: the merge over two sets of partials, P1 behind (d_o_part, d_lse_part) and P2 behind
+// (d_o_part2, d_lse_part2), in that order; P2 == 0 is the plain merge
+int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2,
+                       const float *d_lse_part2, int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb,
+                       int64_t o_sh, int64_t o_sl, float *d_lse, void *stream) {
     INFLLM_REQUIRE(d_o_part && d_lse_part, "attn_merge: null pointer");
+    INFLLM_REQUIRE(P1 >= 1 && P2 >= 0 && (P2 == 0 || (d_o_part2 && d_lse_part2)), "attn_merge: bad partial sets %d + %d", P1, P2);
+    const int32_t P = P1 + P2;
+    PartSets ps{P, 0, 0};
+    if (P2 > 0) {
+        const int64_t rows_ = (int64_t)B * H * Lq;
+        ps.n_first = P1;
+        // index (p * rows + row) of the first buffers -> index ((p - P1) * rows + row) of the second
+        ps.skip_l = (int64_t)(((intptr_t)d_lse_part2 - (intptr_t)d_lse_part) / (intptr_t)sizeof(float)) - (int64_t)P1 * rows_;
+        ps.skip_o = (int64_t)(((intptr_t)d_o_part2 - (intptr_t)d_o_part) / 2) - (int64_t)P1 * rows_ * kD - ps.skip_l * kD;
+    }
     INFLLM_REQUIRE(P >= 1 && B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes P=%d B=%d H=%d Lq=%d", P, B, H, Lq);
     INFLLM_REQUIRE((o_sl % 8 | o_sh % 8 | o_sb % 8) == 0, "attn_merge: output strides must be multiples of 8");
     // few rows, many partials (decode-sized blocks): 16 lanes per row piece, each taking every 16th partial
@@ -918,20 +966,26 @@ extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_pa
         const int64_t rows = (int64_t)B * H * Lq;
         if (wide)
             hipLaunchKernelGGL(attn_merge_lse_wide_kernel, dim3((unsigned)((rows * 16 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                               d_lse_part, P, rows, d_lse);
+                               d_lse_part, P, rows, d_lse, ps);
         else
             hipLaunchKernelGGL(attn_merge_lse_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d_lse_part,
-                               P, rows, d_lse);
+                               P, rows, d_lse, ps);
         INFLLM_CHECK_LAUNCH("attn_merge (lse)");
         return 0;
     }
     const int64_t threads = (int64_t)B * H * Lq * 16;
     if (wide)
         hipLaunchKernelGGL(attn_merge_wide_kernel, dim3((unsigned)((threads * 16 + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                           (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
+                           (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse, ps);
     else
         hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                           (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse);
+                           (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse, ps);
     INFLLM_CHECK_LAUNCH("attn_merge");
     return 0;
+}
+
+extern "C" int infllm_attn_merge(const uint16_t *d_o_part, const float *d_lse_part, int32_t P, int32_t B, int32_t H,
+                                 int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
+                                 void *stream) {
+    return infllm_attn_merge2(d_o_part, d_lse_part, P, nullptr, nullptr, 0, B, H, Lq, d_out, o_sb, o_sh, o_sl, d_lse, stream);
 }

@@ -176,12 +176,20 @@ __global__ __launch_bounds__(256) void ingest_kernel(infllm_ingest_args a) {
 // out[b, c] = scale * sum_p parts[b, p, c], p ascending.  A workgroup owns 64 columns; its 4 waves fetch different
 // partials, so that 32 of them are one round trip to memory (a chain of dependent loads is all latency, and that
 // latency multiplies while a unit fetch keeps the memory fabric busy); the sum itself runs in the fixed order.
+// With blockIdx.z > 0 the partials are those of several execution blocks ingested by one launch: block z owns
+// blk_parts consecutive partials (the last block what is left of n_parts) and exc positions (the last what is left of
+// n_rows), its mean goes to out[z, b, :] and its scale is 1 / (its positions).
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float *parts, int n_parts, int C, float scale,
-                                                              float *out) {
+                                                              float *out, int blk_parts, int n_rows, int exc) {
     __shared__ float stage[32][64];
     const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
-    const int c = blockIdx.x * 64 + lane, b = blockIdx.y;
-    const float *src = parts + (int64_t)b * n_parts * C + c;
+    const int c = blockIdx.x * 64 + lane, b = blockIdx.y, z = blockIdx.z;
+    const float *src = parts + ((int64_t)b * n_parts + (int64_t)z * blk_parts) * C + c;
+    out += (int64_t)z * gridDim.y * C;
+    if (blk_parts < n_parts) {
+        n_parts = min(blk_parts, n_parts - z * blk_parts);
+        scale = 1.f / (float)min(exc, n_rows - z * exc);
+    }
     float s = 0.f;
     for (int p0 = 0; p0 < n_parts; p0 += 32) {
         float v[8];
@@ -340,8 +348,20 @@ extern "C" int infllm_reduce_partials(const float *d_parts, int32_t B, int32_t n
     INFLLM_REQUIRE(d_parts && d_out, "reduce_partials: null pointer");
     INFLLM_REQUIRE(B > 0 && n_parts > 0 && C > 0, "reduce_partials: bad sizes B=%d n_parts=%d C=%d", B, n_parts, C);
     hipLaunchKernelGGL(reduce_partials_kernel, dim3((C + 63) / 64, B), dim3(256), 0, (hipStream_t)stream, d_parts, n_parts, C,
-                       scale, d_out);
+                       scale, d_out, n_parts, 0, 0);
     INFLLM_CHECK_LAUNCH("reduce_partials");
+    return 0;
+}
+
+// library-internal: the mean rotated query of every execution block of one ingest launch over n positions (blocks of
+// exc, a multiple of the ingest tile; the last may be shorter): d_parts [B, ceil(n / tile), C] -> d_out [blocks, B, C]
+int infllm_reduce_partials_blocks(const float *d_parts, int32_t B, int32_t n, int32_t exc, int32_t C, float *d_out, void *stream) {
+    INFLLM_REQUIRE(d_parts && d_out, "reduce_partials_blocks: null pointer");
+    INFLLM_REQUIRE(B > 0 && n > 0 && C > 0 && exc > 0 && exc % kPosPerBlock == 0, "reduce_partials_blocks: bad sizes B=%d n=%d exc=%d C=%d", B, n, exc, C);
+    const int n_parts = (n + kPosPerBlock - 1) / kPosPerBlock, n_blocks = (n + exc - 1) / exc;
+    hipLaunchKernelGGL(reduce_partials_kernel, dim3((C + 63) / 64, B, n_blocks), dim3(256), 0, (hipStream_t)stream, d_parts, n_parts, C,
+                       1.f / (float)n, d_out, n_blocks > 1 ? exc / kPosPerBlock : n_parts, n, exc);
+    INFLLM_CHECK_LAUNCH("reduce_partials_blocks");
     return 0;
 }
 

@@ -110,7 +110,28 @@ struct Layer {
     bool idle_recorded = false;
     bool topk_pending = false;
     int slot = 0;                         // workspace slot written last
-    int cur_slot = 0;                     // workspace slot of the block between front() and back()
+    // Where a block's rotated queries, mean query and (when its local stage already ran) local partials are: a slot of
+    // the per-block workspaces, or a slice of the buffers of a call that was prepared in one go (infllm_call_front).
+    struct QView {
+        const bf16_t *q_loc = nullptr, *q_glb = nullptr;
+        int64_t q_sh = 0, q_sb = 0;
+        const float *qbar = nullptr;
+        bool batched = false;
+        const uint16_t *o_loc = nullptr;   // batched: the block's local partials [nsplit, B, H, n, 128] and log-sum-exps
+        const float *lse_loc = nullptr;
+        int nsplit = 0;
+    };
+    QView fresh;                          // the block whose prologue ran last
+    QView cur;                            // the block between front() and back()
+    infllm_batch_desc bd{};               // buffers for calls prepared in one go
+    bool batch_ok = false;
+    bool batch_live = false;              // a prepared call whose blocks are being worked off
+    int64_t batch_b0 = 0;
+    int batch_n = 0, batch_nsplit = 0;
+    int64_t batch_block_rows = 0;
+    bool batch_retrieved = false;         // the first block's retrieval was launched by infllm_call_front
+    int batch_group = 1;                  // blocks per local-stage launch of the prepared call
+    int batch_regions = 1;                // block-sized regions of the partial rows, used in turn (a multiple of the group)
     bool prepared = false;                // the next block's prologue already ran
     int64_t prepared_b0 = 0;
     int prepared_n = 0;
@@ -142,6 +163,11 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
 int infllm_inline_page_limit();
+int infllm_attn_stage_blocked(const infllm_attn_args *a, int32_t exc, int64_t block_rows, void *stream);
+int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2, const float *d_lse_part2,
+                       int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
+                       void *stream);
+int infllm_reduce_partials_blocks(const float *d_parts, int32_t B, int32_t n, int32_t exc, int32_t C, float *d_out, void *stream);
 int infllm_attn_paged_inline(const infllm_attn_args *local, const infllm_attn_args *global, const infllm_page *h_pages, void *stream);
 int infllm_score_new_rank(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores, const int32_t *d_cand,
                           int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx, int32_t *d_flag,
@@ -505,7 +531,11 @@ int fetch_by_engines(Layer *L, int n_miss, const void *const *srcs, int64_t nbyt
         (void)hipGetLastError();
         HIP_OK(hipEventSynchronize(L->global_done), "fetch: wait global");
     }
-    int rc = efetch_wait_signal(L->efetch_flag_sig, "fetch");             // the previous fetch's flag copy (long done)
+    // One fetch at a time: the host waits here until the previous one has landed (in a long prefill that is some 40 us
+    // of every block - the link is busy three quarters of the time).  Letting the next fetch start while this one is
+    // in flight (a second set of signals) was measured: its copies take bandwidth from the stragglers of the fetch the
+    // stream is waiting for, the waits grow and the stream is no faster.
+    int rc = efetch_wait_signal(L->efetch_flag_sig, "fetch");
     if (rc) return rc;
     const uint32_t seq = ++L->efetch_seq;
     uint32_t *val = L->h_efetch_val + (seq % kEfetchVals);
@@ -787,18 +817,46 @@ int run_ingest(Layer *L, const infllm_front_args *a, const void *q, const void *
     const int C = d.H * kD;
     float *qpart = d.d_qpart + (int64_t)slot * d.B * ((d.exc + 15) / 16) * C;
     in.d_qpart = want_mean ? qpart : nullptr;
+    Layer::QView qv;
+    qv.q_loc = (const bf16_t *)in.d_q_loc; qv.q_glb = (const bf16_t *)in.d_q_glb;
+    qv.q_sh = (int64_t)n * kD; qv.q_sb = (int64_t)d.H * n * kD;
+    qv.qbar = d.d_qbar + (int64_t)slot * d.B * C;
+    L->fresh = qv;
     int rc = infllm_ingest(&in, stream);
     if (rc || !want_mean) return rc;
     return infllm_reduce_partials(qpart, d.B, (n + 15) / 16, C, 1.f / (float)n, d.d_qbar + (int64_t)slot * d.B * C, stream);
 }
 
+// a block of the call that infllm_call_front prepared?
+bool block_in_batch(const Layer *L, int64_t b0, int n) {
+    if (!L->batch_live || b0 < L->batch_b0 || b0 + n > L->batch_b0 + L->batch_n) return false;
+    return (b0 - L->batch_b0) % L->d.exc == 0 && (n == L->d.exc || b0 + n == L->batch_b0 + L->batch_n);
+}
+
+Layer::QView batch_view(const Layer *L, int64_t b0) {
+    const infllm_layer_desc &d = L->d;
+    const int64_t off = b0 - L->batch_b0;
+    const int blk = (int)(off / d.exc);
+    Layer::QView v;
+    v.q_loc = (const bf16_t *)L->bd.d_q_loc + off * kD; v.q_glb = (const bf16_t *)L->bd.d_q_glb + off * kD;
+    v.q_sh = (int64_t)L->batch_n * kD; v.q_sb = (int64_t)d.H * L->batch_n * kD;
+    v.qbar = L->bd.d_qbar + (int64_t)blk * d.B * d.H * kD;
+    v.batched = true;
+    // a block's partials live from its group's launch to its merge: the regions are used in turn
+    const int region = blk % L->batch_regions;
+    v.o_loc = L->bd.d_o_part + (int64_t)region * L->batch_block_rows * kD;
+    v.lse_loc = L->bd.d_lse_part + (int64_t)region * L->batch_block_rows;
+    v.nsplit = L->batch_nsplit;
+    return v;
+}
+
 int run_unit_scores(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_su, float *scores, int64_t scores_sb, int first,
-                    int count, int slot, void *stream) {
+                    int count, const float *qbar, void *stream) {
     const infllm_layer_desc &d = L->d;
     const int C = d.H * kD;
     for (int u = 0; u < d.B; ++u) {
         int rc = infllm_unit_scores((const bf16_t *)reps + (int64_t)u * rep_sb, rep_su, first, count, C,
-                                    d.d_qbar + ((int64_t)slot * d.B + u) * C, scores + (int64_t)u * scores_sb, stream);
+                                    qbar + (int64_t)u * C, scores + (int64_t)u * scores_sb, stream);
         if (rc) return rc;
     }
     return 0;
@@ -858,7 +916,7 @@ int run_score_new_rank(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_s
     if (poll) ++L->topk_seq;
     for (int u = 0; u < d.B; ++u) {
         const bool last = poll && u == d.B - 1;
-        int rc = infllm_score_new_rank((const bf16_t *)reps + (int64_t)u * rep_sb, rep_su, C, d.d_qbar + ((int64_t)L->slot * d.B + u) * C,
+        int rc = infllm_score_new_rank((const bf16_t *)reps + (int64_t)u * rep_sb, rep_su, C, L->fresh.qbar + (int64_t)u * C,
                                        scores + (int64_t)u * scores_sb, L->d_cand + (int64_t)u * d.topk, d.topk, n_old, n_new, d.topk,
                                        d.d_topk_idx + (int64_t)u * d.topk, last ? d.d_topk_flag : nullptr, L->topk_seq, stream);
         if (rc) return rc < 0 ? rc : infllm_fail(-2, "score_new_rank: no kernel after the geometry check");
@@ -872,12 +930,12 @@ int run_score_new_rank(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_s
 }
 
 // n_parts > 0: the stages' partial log-sum-exps are joined inside the launch (d_lse is not ready yet)
-int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t j_hi, int n_parts, void *stream) {
+int run_local_score(Layer *L, int n, int64_t b0, const Layer::QView &qv, int64_t j_lo, int64_t j_hi, int n_parts, void *stream) {
     const infllm_layer_desc &d = L->d;
     if (j_hi <= j_lo) return 0;
     infllm_score_args sc{};
-    sc.d_q = (const bf16_t *)d.d_q_loc + (int64_t)slot * d.B * d.H * d.exc * kD;
-    sc.q_sl = kD; sc.q_sh = (int64_t)n * kD; sc.q_sb = (int64_t)d.H * n * kD;
+    sc.d_q = qv.q_loc;
+    sc.q_sl = kD; sc.q_sh = qv.q_sh; sc.q_sb = qv.q_sb;
     sc.B = d.B; sc.H = d.H; sc.Hkv = d.Hkv; sc.Lq = n;
     sc.d_k = d.d_ring_k_rot;
     sc.k_sl = kD; sc.k_sh = d.ring_cap * kD; sc.k_sb = (int64_t)d.Hkv * d.ring_cap * kD;
@@ -889,13 +947,13 @@ int run_local_score(Layer *L, int n, int64_t b0, int slot, int64_t j_lo, int64_t
 }
 
 // the local stage of a block: causal sliding window over the ring
-infllm_attn_args local_stage_args(Layer *L, int n, int64_t b0, int slot, int nsplit) {
+infllm_attn_args local_stage_args(Layer *L, int n, int64_t b0, const Layer::QView &qv, int nsplit) {
     const infllm_layer_desc &d = L->d;
     const int64_t b1 = b0 + n;
     const int64_t lo = b0 > d.n_local ? b0 - d.n_local : 0;
     infllm_attn_args at{};
-    at.d_q = (const bf16_t *)d.d_q_loc + (int64_t)slot * d.B * d.H * d.exc * kD;
-    at.q_sl = kD; at.q_sh = (int64_t)n * kD; at.q_sb = (int64_t)d.H * n * kD;
+    at.d_q = qv.q_loc;
+    at.q_sl = kD; at.q_sh = qv.q_sh; at.q_sb = qv.q_sb;
     at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = n;
     at.d_k = d.d_ring_k_rot; at.d_v = d.d_ring_v;
     at.k_sl = at.v_sl = kD;
@@ -911,6 +969,94 @@ infllm_attn_args local_stage_args(Layer *L, int n, int64_t b0, int slot, int nsp
 
 }  // namespace
 
+extern "C" int infllm_layer_set_batch(void *layer, const infllm_batch_desc *b) {
+    INFLLM_REQUIRE(layer && b, "layer_set_batch: null argument");
+    Layer *L = (Layer *)layer;
+    const infllm_layer_desc &d = L->d;
+    INFLLM_REQUIRE(b->d_q_loc && b->d_q_glb && b->d_qpart && b->d_qbar && b->d_o_part && b->d_lse_part, "layer_set_batch: null buffer");
+    INFLLM_REQUIRE(d.exc % 32 == 0, "layer_set_batch: execution blocks of %d rows are not whole query tiles", d.exc);
+    INFLLM_REQUIRE(b->max_tokens >= d.exc, "layer_set_batch: %d tokens are less than one execution block", b->max_tokens);
+    INFLLM_REQUIRE(b->group_blocks >= 0 && b->group_blocks <= 64, "layer_set_batch: %d blocks per launch", b->group_blocks);
+    const int group = b->group_blocks > 0 ? b->group_blocks : 2;
+    INFLLM_REQUIRE(b->part_rows >= (int64_t)d.B * d.H * d.exc * (4 * group > 8 ? 4 * group : 8), "layer_set_batch: too few partial rows");
+    INFLLM_REQUIRE(!L->batch_live, "layer_set_batch: a prepared call is still being worked off");
+    L->bd = *b;
+    L->batch_ok = true;
+    return 0;
+}
+
+extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *stream) {
+    INFLLM_REQUIRE(layer && a, "call_front: null argument");
+    Layer *L = (Layer *)layer;
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream;
+    INFLLM_REQUIRE(L->batch_ok, "call_front: no buffers (infllm_layer_set_batch)");
+    INFLLM_REQUIRE(a->n >= 1 && a->n <= L->bd.max_tokens, "call_front: %d tokens do not fit the buffers (%d)", a->n, L->bd.max_tokens);
+    INFLLM_REQUIRE(a->n <= d.ring_cap, "call_front: %d tokens do not fit a ring of %lld rows", a->n, (long long)d.ring_cap);
+    INFLLM_REQUIRE(a->n_units >= 0 && a->b0 >= 0, "call_front: negative state");
+    L->main_stream = st;
+    L->main_stream_known = true;
+    L->batch_live = false;
+    L->prepared = false;
+    const int C = d.H * kD;
+    const int n_blocks = (a->n + d.exc - 1) / d.exc;
+
+    // ---- prologue of every token, mean query of every block
+    infllm_ingest_args in{};
+    in.d_q = a->d_q; in.d_k = a->d_k; in.d_v = a->d_v;
+    in.q_sb = a->q_sb; in.q_sh = a->q_sh; in.q_sl = a->q_sl;
+    in.k_sb = a->k_sb; in.k_sh = a->k_sh; in.k_sl = a->k_sl;
+    in.v_sb = a->v_sb; in.v_sh = a->v_sh; in.v_sl = a->v_sl;
+    in.B = d.B; in.H = d.H; in.Hkv = d.Hkv; in.n = a->n;
+    in.pos0 = a->b0; in.glb_pos = d.n_local - 1;
+    in.d_inv_freq = d.d_inv_freq; in.distance_scale = d.distance_scale;
+    in.d_ring_k_raw = d.d_ring_k_raw; in.d_ring_k_rot = d.d_ring_k_rot; in.d_ring_v = d.d_ring_v;
+    in.d_ring_score = d.d_ring_score; in.ring_cap = d.ring_cap;
+    in.d_q_loc = L->bd.d_q_loc; in.d_q_glb = L->bd.d_q_glb;
+    in.d_qpart = L->bd.d_qpart;
+    int rc = infllm_ingest(&in, stream);
+    if (rc) return rc;
+    rc = infllm_reduce_partials_blocks(L->bd.d_qpart, d.B, a->n, d.exc, C, L->bd.d_qbar, stream);
+    if (rc) return rc;
+
+    // ---- how the local stage cuts its keys: as few splits as fill the chip, and no more than the partial rows hold.
+    //      It is launched for a group of blocks at a time (block_front, at the group's first block), every launch
+    //      with the same number of splits.
+    const int group = L->bd.group_blocks > 0 ? L->bd.group_blocks : 2;
+    const int group_n = a->n < group * d.exc ? a->n : group * d.exc;
+    const int64_t b1 = a->b0 + group_n;
+    const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
+    int nsplit = splits_for(d, group_n, (int)((b1 - lo + kTile - 1) / kTile));
+    // room for the partials of two groups: the one being merged block by block and the one launched ahead of it
+    const int64_t rows_one = (int64_t)d.B * d.H * (n_blocks > 1 ? d.exc : a->n);
+    const int need = n_blocks > 1 ? 2 * group : 1;
+    while (nsplit > 1 && L->bd.part_rows / (nsplit * rows_one) < need) --nsplit;
+    int regions = (int)(L->bd.part_rows / (nsplit * rows_one));
+    INFLLM_REQUIRE(regions >= need, "call_front: partial rows do not fit");
+    regions = regions / group * group;
+    L->batch_live = true;
+    L->batch_b0 = a->b0;
+    L->batch_n = a->n;
+    L->batch_nsplit = nsplit;
+    L->batch_group = group;
+    L->batch_regions = n_blocks > 1 ? regions : 1;
+    L->batch_block_rows = (int64_t)nsplit * d.B * d.H * (n_blocks > 1 ? d.exc : a->n);
+    L->fresh = batch_view(L, a->b0);
+
+    // ---- the first block's retrieval
+    L->topk_pending = false;
+    L->batch_retrieved = false;
+    if (a->n_units > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL)) {
+        INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "call_front: null representative / score buffer");
+        rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
+        if (rc) return rc;
+        rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, stream);
+        if (rc) return rc;
+        L->batch_retrieved = true;
+    }
+    return 0;
+}
+
 extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void *stream) {
     INFLLM_REQUIRE(layer && a, "block_front: null argument");
     Layer *L = (Layer *)layer;
@@ -924,49 +1070,50 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     L->main_stream_known = true;
 
     // ---- this block's prologue and retrieval, unless the previous block prepared them
+    const bool batched = block_in_batch(L, a->b0, a->n);       // its prologue and local stage ran in infllm_call_front
     if (!(L->prepared && L->prepared_b0 == a->b0 && L->prepared_n == a->n)) {
-        L->slot ^= 1;
         const bool retrieve = a->n_units > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL);
-        rc = run_ingest(L, a, a->d_q, a->d_k, a->d_v, a->n, a->b0, L->slot, retrieve, stream);
-        if (rc) return rc;
-        L->topk_pending = false;
-        if (retrieve) {
+        const bool retrieved = batched && L->batch_retrieved && a->b0 == L->batch_b0;
+        if (batched)
+            L->fresh = batch_view(L, a->b0);
+        else {
+            L->slot ^= 1;
+            rc = run_ingest(L, a, a->d_q, a->d_k, a->d_v, a->n, a->b0, L->slot, retrieve, stream);
+            if (rc) return rc;
+        }
+        if (!retrieved) L->topk_pending = false;
+        if (retrieve && !retrieved) {
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
-            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->slot, stream);
+            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
             if (rc) return rc;
             rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, stream);
             if (rc) return rc;
         }
     }
+    L->batch_retrieved = false;
     L->prepared = false;
-    L->cur_slot = L->slot;
+    L->cur = L->fresh;
     L->cur_n = a->n;
     L->cand_for_units = -1;
 
-    // ---- local stage: causal sliding window over the ring.  Launched here, ahead of the host's wait for the selection
-    //      and of the stream's wait for the fetched units, both of which it covers.  With INFLLM_FUSED_STAGES=1
-    //      block_back launches it instead, in ONE launch with the global stage (measured: the launch is 6 us shorter than
-    //      the two and the merge reads half the partials, but the stream then reaches its wait for the fetch a local
-    //      stage earlier and idles longer than it saved - the missed units' way over PCIe takes 135 us of a 190 us block).
     const int64_t b1 = a->b0 + a->n;
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
-    L->local_pending = !L->local_in_front;
-    if (L->local_in_front) {
-        infllm_attn_args at = local_stage_args(L, a->n, a->b0, L->cur_slot, splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile)));
-        const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
-        rc = infllm_attn_stage(&at, stream);
-        timer_end(L, 0, ti, st);
-        if (rc) return rc;
-    }
 
-    // ---- the next block's prologue and the scores of the units that exist already
-    if (a->n_next > 0 && a->d_q_next && a->d_k_next && a->d_v_next) {
-        L->slot ^= 1;
-        rc = run_ingest(L, a, a->d_q_next, a->d_k_next, a->d_v_next, a->n_next, b1, L->slot, true, stream);
-        if (rc) return rc;
+    // ---- the next block's prologue and the scores of the units that exist already.  Ahead of the local stage: the
+    //      host starts the next block's fetch from the candidates chosen here, and everything queued before them
+    //      delays that fetch.
+    const bool next_batched = a->n_next > 0 && block_in_batch(L, b1, a->n_next);
+    if (next_batched || (a->n_next > 0 && a->d_q_next && a->d_k_next && a->d_v_next)) {
+        if (next_batched)
+            L->fresh = batch_view(L, b1);
+        else {
+            L->slot ^= 1;
+            rc = run_ingest(L, a, a->d_q_next, a->d_k_next, a->d_v_next, a->n_next, b1, L->slot, true, stream);
+            if (rc) return rc;
+        }
         if (a->n_units > 0 && !(a->flags & INFLLM_NO_RETRIEVAL)) {
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
-            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->slot, stream);
+            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
             if (rc) return rc;
             // their k best now, while the fetch is in flight: the selection after the block then only has to weigh these
             // against the few units carved in between, instead of running over every unit on the chain
@@ -987,6 +1134,33 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
         L->prepared = true;
         L->prepared_b0 = b1;
         L->prepared_n = a->n_next;
+    }
+
+    // ---- local stage: causal sliding window over the ring.  Launched here, ahead of the host's wait for the selection
+    //      and of the stream's wait for the fetched units, both of which it covers.  With INFLLM_FUSED_STAGES=1
+    //      block_back launches it instead, in ONE launch with the global stage (measured: the launch is 6 us shorter than
+    //      the two and the merge reads half the partials, but the stream then reaches its wait for the fetch a local
+    //      stage earlier and idles longer than it saved - the missed units' way over PCIe takes 135 us of a 190 us block).
+    L->local_pending = !batched && !L->local_in_front;
+    if (batched && ((a->b0 - L->batch_b0) / d.exc) % L->batch_group == 0) {
+        // the local stage of this block and the next ones of its group in one launch (more queries per launch: fewer
+        // key splits, fewer partial rows, the launch's fixed cost once); each block's partials go where its merge
+        // expects them
+        const int64_t left = L->batch_b0 + L->batch_n - a->b0;
+        const int gn = (int)(left < (int64_t)L->batch_group * d.exc ? left : (int64_t)L->batch_group * d.exc);
+        infllm_attn_args at = local_stage_args(L, gn, a->b0, L->cur, L->batch_nsplit);
+        at.d_o_part = (uint16_t *)L->cur.o_loc; at.d_lse_part = (float *)L->cur.lse_loc;
+        const int ti = timer_begin(L, 0, gn, (int)(a->b0 + gn - lo), st);
+        rc = infllm_attn_stage_blocked(&at, d.exc, L->batch_block_rows, stream);
+        timer_end(L, 0, ti, st);
+        if (rc) return rc;
+    }
+    if (!batched && L->local_in_front) {
+        infllm_attn_args at = local_stage_args(L, a->n, a->b0, L->cur, splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile)));
+        const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
+        rc = infllm_attn_stage(&at, stream);
+        timer_end(L, 0, ti, st);
+        if (rc) return rc;
     }
     return 0;
 }
@@ -1299,7 +1473,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     const int64_t b1 = a->b0 + a->n;
     const int64_t unit_elems = (int64_t)d.Hkv * bs * kD;          // K (or V) of one unit
     const int64_t slot_elems = 2 * unit_elems;
-    const int cur = L->cur_slot;
+    const Layer::QView &cur = L->cur;
+    const bool batched = cur.batched;
 
     // ---- 1. fetch missed units into their slots (copy stream), unless infllm_block_fetch already did
     if (!L->fetch_issued) {
@@ -1425,7 +1600,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         rc = infllm_attn_stage(&at, stream);
         timer_end(L, 0, ti, st);
         if (rc) return rc;
-    } else if (!L->local_pending)
+    } else if (batched)
+        sl = cur.nsplit;                                  // launched by infllm_call_front, for the whole call
+    else if (!L->local_pending)
         sl = splits_for(d, a->n, lin_tiles);              // launched by block_front
     const int tw = L->fetch_wait || L->efetch_wait ? timer_begin(L, 2, a->n, a->n_miss, st) : -1;
     if (L->fetch_wait) {
@@ -1440,8 +1617,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     int parts = sl;
     if (n_pages > 0) {
         infllm_attn_args at{};
-        at.d_q = (const bf16_t *)d.d_q_glb + (int64_t)cur * d.B * d.H * d.exc * kD;
-        at.q_sl = kD; at.q_sh = (int64_t)a->n * kD; at.q_sb = (int64_t)d.H * a->n * kD;
+        at.d_q = cur.q_glb;
+        at.q_sl = kD; at.q_sh = cur.q_sh; at.q_sb = cur.q_sb;
         at.B = d.B; at.H = d.H; at.Hkv = d.Hkv; at.Lq = a->n;
         at.cap = kTile;
         at.d_pages = d.d_pages; at.n_pages = n_pages;
@@ -1459,8 +1636,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
             parts = ns;
         } else {
             at.nsplit = splits_for(d, a->n, n_pages);
-            at.d_o_part = d.d_o_part + sl * part_o;
-            at.d_lse_part = d.d_lse_part + sl * part_l;
+            // behind the local stage's partials - unless those lie with the call's (then the merge takes two sets)
+            at.d_o_part = d.d_o_part + (batched ? 0 : sl * part_o);
+            at.d_lse_part = d.d_lse_part + (batched ? 0 : sl * part_l);
             const int ti = timer_begin(L, 1, a->n, n_pages * kTile, st);
             rc = pages_inline ? infllm_attn_paged_inline(nullptr, &at, inline_pages, stream) : infllm_attn_stage(&at, stream);
             timer_end(L, 1, ti, st);
@@ -1482,8 +1660,16 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     // step 4, which joins the partial values itself; the merge (output rows and the joint value for the bulk of the
     // scores) runs once that selection is out (step 5b).  The score-decay policy needs the joint value here.
     const bool lse_now = a->d_unit_mass && a->n_sel > 0;
-    if (lse_now) {
-        rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, nullptr, 0, 0, 0, d.d_lse, stream);
+    const bool one_pass = L->guessing && !lse_now;
+    // partials in two places cannot be joined by the score launch: the joint value comes first then as well
+    const bool lse_early = lse_now || (batched && !one_pass);
+    auto merge = [&](void *out, float *lse) {
+        return batched ? infllm_attn_merge2(cur.o_loc, cur.lse_loc, sl, d.d_o_part, d.d_lse_part, parts - sl, d.B, d.H, a->n, out, a->o_sb,
+                                            a->o_sh, a->o_sl, lse, stream)
+                       : infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, out, a->o_sb, a->o_sh, a->o_sl, lse, stream);
+    };
+    if (lse_early) {
+        rc = merge(nullptr, d.d_lse);
         if (rc) return rc;
     }
 
@@ -1493,8 +1679,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         for (int u = 0; u < d.B; ++u)
             for (int i = 0; i < a->n_sel; ++i) {
                 infllm_score_args sc{};
-                sc.d_q = (const bf16_t *)d.d_q_glb + (int64_t)cur * d.B * d.H * d.exc * kD + (int64_t)u * d.H * a->n * kD;
-                sc.q_sl = kD; sc.q_sh = (int64_t)a->n * kD; sc.q_sb = 0;
+                sc.d_q = cur.q_glb + (int64_t)u * cur.q_sb;
+                sc.q_sl = kD; sc.q_sh = cur.q_sh; sc.q_sb = 0;
                 sc.B = 1; sc.H = d.H; sc.Hkv = d.Hkv; sc.Lq = a->n;
                 sc.d_k = (const bf16_t *)d.d_slab + ((int64_t)u * d.max_cached + a->h_sel_slots[u * a->n_sel + i]) * slot_elems;
                 sc.k_sl = kD; sc.k_sh = (int64_t)bs * kD; sc.k_sb = 0;
@@ -1521,13 +1707,12 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     const int64_t urgent_hi = new_cursor < b1 ? new_cursor : b1;
     // While the fetches run ahead of the selection nothing waits for this block's selection at once, and the split
     // into an urgent and a bulk score launch only costs stream time: the merge and one score launch come first then.
-    const bool one_pass = L->guessing && !lse_now;
     if (one_pass) {
-        rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl, d.d_lse, stream);
+        rc = merge(a->d_out, d.d_lse);
         if (rc) return rc;
         rc = run_local_score(L, a->n, a->b0, cur, lo, b1, 0, stream);
     } else
-        rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, lse_now ? 0 : parts, stream);
+        rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, lse_early ? 0 : parts, stream);
     if (rc) return rc;
     int64_t cursor = a->cursor;
     if (a->init_take > 0) {
@@ -1584,7 +1769,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
                    : 1;
         if (rc < 0) return rc;
         if (rc == 1) {                  // the two steps on their own
-            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->slot,
+            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->fresh.qbar,
                                  stream);
             if (rc) return rc;
             if (merge)
@@ -1630,8 +1815,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     }
     // ---- 5b. the block's output rows
     if (!one_pass) {
-        rc = infllm_attn_merge(d.d_o_part, d.d_lse_part, parts, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh, a->o_sl,
-                               lse_now ? nullptr : d.d_lse, stream);
+        rc = merge(a->d_out, lse_early ? nullptr : d.d_lse);
         if (rc) return rc;
         // ---- 6. off the critical path: the rest of the local score, new units to pinned host memory
         rc = run_local_score(L, a->n, a->b0, cur, urgent_hi > lo ? urgent_hi : lo, b1, 0, stream);
@@ -1668,6 +1852,7 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
         const int wrc = dma_wait_slot(L, (int)s, "layer_flush");
         if (wrc) return wrc;
     }
+    L->batch_live = false;
     if (L->main_stream_known) {
         HIP_OK(hipEventRecord(L->idle_main, L->main_stream), "layer_flush: event");
         HIP_OK(hipEventRecord(L->idle_copy, (hipStream_t)copy_stream), "layer_flush: event");

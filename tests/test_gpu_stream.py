@@ -184,30 +184,40 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
     assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
 
 
-def test_stage_timers_sample_the_launches_they_are_asked_for():
+def test_stage_timers_sample_the_launches_they_are_asked_for(monkeypatch):
     """infllm_layer_timing / infllm_layer_read_timing (what bench.py's roofline figure is made of): every stride-th
     launch of the local stage, of the global stage and of the stream's wait for the fetch is bracketed by events; the
-    records carry the launch's sizes and a positive duration, and timing changes no result."""
+    records carry the launch's sizes and a positive duration, and timing changes no result.  With every block running
+    its own local stage there is a launch per block; with the call prepared in one go, one per group of blocks."""
     from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
     T = 1600
     q, k, v = make_stream(T, 8, 2, 23)
     kw = dict(SMALL, max_cached_block=5, async_global_stream=True)
-    plain, _ = run_gpu(q, k, v, [T], 1e4, **kw)
-    rope = RotaryEmbeddingESM(D, base=1e4, device="cuda")
-    cm = ContextManager(rope, kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"], kw["topk"],
-                        kw["exc_block_size"], None, False, kw["repr_topk"], "lru", None, True, False, False, False)
-    cm.enable_timing(64, 2)
-    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
-    out = cm.append(qd, kd, vd, qd, kd, vd)
-    torch.cuda.synchronize()
-    assert torch.equal(out.cpu(), plain)
-    n_blocks = T // kw["exc_block_size"]
-    local, glob, wait = cm.read_timing(0), cm.read_timing(1), cm.read_timing(2)
-    assert len(local) == (n_blocks + 1) // 2                       # every second launch of n_blocks
-    assert 0 < len(glob) <= len(local) and 0 < len(wait) <= len(glob)
-    for ms, nq, nk in local + glob + wait:
-        assert 0.0 < ms < 50.0 and nq == kw["exc_block_size"]
-    assert max(nk for _, _, nk in local) == kw["n_local"] + kw["exc_block_size"]
+    exc = kw["exc_block_size"]
+    for call_tokens in (0, 16 * exc):
+        monkeypatch.setattr(ContextManager, "call_tokens", call_tokens)
+        plain, _ = run_gpu(q, k, v, [T], 1e4, **kw)
+        rope = RotaryEmbeddingESM(D, base=1e4, device="cuda")
+        cm = ContextManager(rope, kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"], kw["topk"],
+                            exc, None, False, kw["repr_topk"], "lru", None, True, False, False, False)
+        cm.enable_timing(64, 2)
+        qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+        out = cm.append(qd, kd, vd, qd, kd, vd)
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), plain)
+        n_blocks = T // exc
+        local, glob, wait = cm.read_timing(0), cm.read_timing(1), cm.read_timing(2)
+        if call_tokens == 0:
+            assert len(local) == (n_blocks + 1) // 2                   # every second launch of n_blocks
+            assert 0 < len(glob) <= len(local) and 0 < len(wait) <= len(glob)
+            assert max(nk for _, _, nk in local) == kw["n_local"] + exc
+        else:
+            # 16 + 9 blocks in groups of two: 8 + 5 launches, every second one timed, the last over the odd block alone
+            assert [nq for _, nq, _ in local] == [2 * exc] * 6 + [exc]
+            assert max(nk for _, _, nk in local) == kw["n_local"] + 2 * exc
+            assert 0 < len(glob) <= (n_blocks + 1) // 2 and 0 < len(wait) <= len(glob)
+        for ms, nq, nk in local + glob + wait:
+            assert 0.0 < ms < 50.0 and (nq == exc or call_tokens)
     import ctypes
     from infllm_amd._lib import InfLLMHipError, check
     with pytest.raises(InfLLMHipError):                            # there is no fourth timer
