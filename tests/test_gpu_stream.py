@@ -16,10 +16,31 @@ from stream_parity import (D, REFERENCE, REPR_TIE_REL, SMALL, TIE_REL, Follower,
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["call in one go", "block by block"])
+def call_mode(request, monkeypatch):
+    """How an append() call is prepared: prologue and mean queries of the whole call at once and the local stage for
+    two blocks per launch (infllm_call_front, the default), or every block on its own (call_tokens = 0)."""
+    from infllm_amd.attention import ContextManager
+    if request.param == "block by block":
+        monkeypatch.setattr(ContextManager, "call_tokens", 0)
+    return request.param
+
+
 @pytest.mark.parametrize("calls", [[1500], [64] * 20 + [100, 17, 3], [1] * 40 + [700] + [1] * 30])
-def test_small_geometry_follows_oracle(calls):
+def test_small_geometry_follows_oracle(calls, call_mode):
     cm, ora, fol = compare(sum(calls), calls, H=8, Hkv=2, base=1e4, seed=len(calls), **SMALL)
     assert cm.num_global_block > SMALL["topk"]            # retrieval was exercised
+    assert bool(cm._call_tokens) == (call_mode == "call in one go")
+
+
+def test_local_stage_groups_of_other_sizes_follow_the_oracle(monkeypatch):
+    """One, three and sixteen blocks per launch of the local stage (INFLLM_LOCAL_GROUP; two is the default): the
+    blocks' partial rows lie in regions that are used in turn, whatever the group size, and a call that is not a
+    whole number of groups ends with a shorter launch."""
+    for group in ("1", "3", "16"):
+        monkeypatch.setenv("INFLLM_LOCAL_GROUP", group)
+        cm, _, _ = compare(1500, [700, 1, 1, 798], H=8, Hkv=2, base=1e4, seed=51, B=2, **SMALL)
+        assert cm.num_global_block > SMALL["topk"]
 
 
 def test_both_stages_in_one_launch_follow_the_oracle(monkeypatch):
@@ -112,7 +133,7 @@ def test_no_gqa_and_perhead():
     compare(800, [800], H=2, Hkv=2, base=1e4, seed=9, **SMALL)
 
 
-def test_reference_geometry_9k_tokens_in_two_calls():
+def test_reference_geometry_9k_tokens_in_two_calls(call_mode):
     """Mistral-7B geometry and the reference's default knobs (config/mistral-inf-llm.yaml), 9,216 tokens, mixture keys."""
     T = 8192 + 1024
     cm, ora, fol = compare(T, [8192, 1024], H=32, Hkv=8, base=1e6, seed=11, **REFERENCE)
