@@ -614,11 +614,12 @@ class ContextManager:
                 # the next stretch of the call in one go: prologue, mean queries, first retrieval, local stage
                 call_end = min(st + self._call_tokens, input_length)
                 assert self.length + call_end - self.cursor <= self.ring_cap
-                fa.d_q, fa.d_k, fa.d_v = (self._q_ptr + st * self._q_step, self._k_ptr + st * self._k_step,
-                                          self._v_ptr + st * self._v_step)
-                fa.n, fa.n_units, fa.b0 = call_end - st, self.num_global_block, self.length + st
-                fa.flags = _lib.NO_RETRIEVAL if use_chunks else 0
-                check(self._lib.infllm_call_front(self._layer, self._fa_ref, self._main_raw), "infllm_call_front")
+                if call_end - st > exc:          # a single block (a decode step) gains nothing from being prepared apart
+                    fa.d_q, fa.d_k, fa.d_v = (self._q_ptr + st * self._q_step, self._k_ptr + st * self._k_step,
+                                              self._v_ptr + st * self._v_step)
+                    fa.n, fa.n_units, fa.b0 = call_end - st, self.num_global_block, self.length + st
+                    fa.flags = _lib.NO_RETRIEVAL if use_chunks else 0
+                    check(self._lib.infllm_call_front(self._layer, self._fa_ref, self._main_raw), "infllm_call_front")
             elif not self._call_tokens:
                 call_end = input_length
             chosen = None
