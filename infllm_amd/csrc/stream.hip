@@ -96,6 +96,11 @@ struct Layer {
     int64_t ahead_issued = 0, ahead_confirmed = 0;
     bool ahead_any_path = false;                       // guess also when the fetch kernel has to move the units
     int page_cur = 0, carve_cur = 0;
+    // which units each staging slot of the carve holds (the launch that fills it is in the main stream's queue or done):
+    // a missed unit that is still there is copied from there, device to device, instead of coming back over PCIe
+    std::vector<int> stage_first, stage_count;
+    hipEvent_t stage_copied = nullptr;                 // behind the last such copy
+    std::vector<int64_t> stage_copy_dst;               // slots (row * max_cached + slot) such copies may still be on their way to
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
     int32_t topk_seq = 0;
@@ -573,8 +578,69 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
     const infllm_layer_desc &d = L->d;
     const bool side = cs != st;
     const int64_t slot_elems = 2 * (int64_t)d.Hkv * d.block_size * kD;
+    // A unit carved a few blocks ago is still in the staging slot it was gathered into (the launch that filled it is
+    // ahead of this point in the main stream): it is copied from there.  A unit that makes a selection right after it
+    // was carved - which is when a guessed selection turns out wrong - would otherwise have to wait for its own way
+    // to the host to end before it could come back.
+    std::vector<int32_t> rows_k, slots_k, units_k;
+    std::vector<const void *> srcs_k;
     if (n_miss > 0) {
         INFLLM_REQUIRE(rows && slots && units && srcs, "fetch: null miss list");
+        // slots that an earlier copy out of staging may still be on its way to: a fetch that is not ordered by the
+        // main stream (engines, copy stream) lets it land before it writes one of them again
+        if (!L->stage_copy_dst.empty()) {
+            const hipError_t q = hipEventQuery(L->stage_copied);
+            if (q == hipSuccess)
+                L->stage_copy_dst.clear();
+            else {
+                (void)hipGetLastError();
+                bool hit = false;
+                for (int i = 0; i < n_miss && !hit; ++i)
+                    for (int64_t dst : L->stage_copy_dst) hit = hit || dst == (int64_t)rows[i] * d.max_cached + slots[i];
+                if (hit) {
+                    HIP_OK(hipEventSynchronize(L->stage_copied), "fetch: wait staging copy");
+                    L->stage_copy_dst.clear();
+                }
+            }
+        }
+        hipStream_t ms = L->main_stream_known ? L->main_stream : st;       // the stream the staging slots are filled on
+        std::vector<char> staged(n_miss, 0);
+        int n_staged = 0;
+        const int64_t unit_all = (int64_t)d.B * slot_elems;
+        for (int i = 0; i < n_miss; ++i) {
+            int at = -1;
+            for (size_t sl = 0; sl < L->stage_count.size() && at < 0; ++sl)
+                if (units[i] >= L->stage_first[sl] && units[i] < L->stage_first[sl] + L->stage_count[sl]) at = (int)sl;
+            if (at < 0) continue;
+            INFLLM_REQUIRE(rows[i] >= 0 && rows[i] < d.B && slots[i] >= 0 && slots[i] < d.max_cached, "fetch: bad miss entry");
+            if (n_staged == 0) {
+                // an earlier fetch may still be on its way to the same slot (a guess that turned out wrong put another
+                // unit there; a repair put back one that is evicted again): it lands first
+                if (L->efetch_ok) {
+                    const int wrc = efetch_wait_signal(L->efetch_flag_sig, "fetch");
+                    if (wrc) return wrc;
+                }
+                if (L->fetch_wait && ms != cs) HIP_OK(hipStreamWaitEvent(ms, L->fetch_done, 0), "fetch: wait fetch");
+            }
+            const bf16_t *src = (const bf16_t *)d.d_carve_stage + ((int64_t)at * d.max_carve + (units[i] - L->stage_first[at])) * unit_all +
+                                (int64_t)rows[i] * slot_elems;
+            bf16_t *dst = (bf16_t *)d.d_slab + ((int64_t)rows[i] * d.max_cached + slots[i]) * slot_elems;
+            HIP_OK(hipMemcpyAsync(dst, src, slot_elems * sizeof(bf16_t), hipMemcpyDeviceToDevice, ms), "fetch: copy from staging");
+            L->stage_copy_dst.push_back((int64_t)rows[i] * d.max_cached + slots[i]);
+            staged[i] = 1;
+            ++n_staged;
+        }
+        if (n_staged > 0) {
+            HIP_OK(hipEventRecord(L->stage_copied, ms), "fetch: event");
+            for (int i = 0; i < n_miss; ++i) {
+                if (staged[i]) continue;
+                rows_k.push_back(rows[i]); slots_k.push_back(slots[i]); units_k.push_back(units[i]); srcs_k.push_back(srcs[i]);
+            }
+            rows = rows_k.data(); slots = slots_k.data(); units = units_k.data(); srcs = srcs_k.data();
+            n_miss = (int)rows_k.size();
+        }
+    }
+    if (n_miss > 0) {
         if (L->off.pending) {
             bool hit = false;
             for (int i = 0; i < n_miss && !hit; ++i) hit = units[i] >= L->off.first_unit && units[i] < L->off.first_unit + L->off.count;
@@ -680,11 +746,14 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
               hipEventCreateWithFlags(&L->carve_ready, hipEventDisableTiming) == hipSuccess &&
               hipEventCreateWithFlags(&L->mass_done, hipEventDisableTiming) == hipSuccess &&
               hipEventCreateWithFlags(&L->idle_main, hipEventDisableTiming) == hipSuccess &&
-              hipEventCreateWithFlags(&L->idle_copy, hipEventDisableTiming) == hipSuccess;
+              hipEventCreateWithFlags(&L->idle_copy, hipEventDisableTiming) == hipSuccess &&
+              hipEventCreateWithFlags(&L->stage_copied, hipEventDisableTiming) == hipSuccess;
     L->page_evt.resize(d.page_slots, nullptr);
     L->carve_evt.resize(d.carve_slots, nullptr);
     L->page_busy.assign(d.page_slots, 0);
     L->carve_busy.assign(d.carve_slots, 0);
+    L->stage_first.assign(d.carve_slots, 0);
+    L->stage_count.assign(d.carve_slots, 0);
 
     for (auto &e : L->page_evt) ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
     for (auto &e : L->carve_evt) ok = ok && hipEventCreateWithFlags(&e, hipEventDisableTiming) == hipSuccess;
@@ -731,7 +800,7 @@ extern "C" int infllm_layer_destroy(void *layer) {
         (void)hipEventSynchronize(L->idle_main);
         (void)hipEventSynchronize(L->idle_copy);
     }
-    for (hipEvent_t e : {L->topk_done, L->global_done, L->fetch_done, L->carve_ready, L->mass_done, L->idle_main, L->idle_copy})
+    for (hipEvent_t e : {L->topk_done, L->global_done, L->fetch_done, L->carve_ready, L->mass_done, L->idle_main, L->idle_copy, L->stage_copied})
         if (e) (void)hipEventDestroy(e);
     for (hipEvent_t e : L->page_evt)
         if (e) (void)hipEventDestroy(e);
@@ -1755,6 +1824,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
                                     a->d_rep_out, a->rep_sb, a->rep_su, a->d_repr_idx, d.d_ring_v, stage, stage + unit_elems, slot_elems,
                                     unit_all, (int64_t)bs * kD, stream);
         if (rc) return rc;
+        L->stage_first[slot] = a->n_units;
+        L->stage_count[slot] = a->n_carve;
         carved = true;
         carved_slot = slot;
     }
