@@ -68,6 +68,7 @@ struct Layer {
     hsa_signal_t efetch_sig{}, efetch_flag_sig{};
     uint32_t *d_efetch_flag = nullptr, *h_efetch_val = nullptr;
     int efetch_dev = 0;
+    uint32_t off_engine = 0;                           // the engine that takes carved units to the host (0: the runtime's choice)
     uint32_t efetch_seq = 0;
     bool efetch_wait = false;
     int cur_n = 0;                                     // queries of the block in flight
@@ -389,8 +390,13 @@ int issue_offload_dma(Layer *L) {
     for (int i = 0; i < n;) {                    // one copy per run of units that are contiguous on the host
         int j = i + 1;
         while (j < n && (char *)L->off.dst[j] == (char *)L->off.dst[j - 1] + unit_all * sizeof(bf16_t)) ++j;
-        const hsa_status_t hs = hsa_amd_memory_async_copy(L->off.dst[i], L->dma_cpu, stage + (int64_t)i * unit_all, L->dma_gpu,
-                                                          (size_t)(j - i) * unit_all * sizeof(bf16_t), 0, nullptr, L->dma_sig[slot]);
+        // on the engine kept for this direction where there is one (see efetch_setup), else wherever the runtime puts it
+        const size_t bytes = (size_t)(j - i) * unit_all * sizeof(bf16_t);
+        const hsa_status_t hs = L->off_engine ? hsa_amd_memory_async_copy_on_engine(L->off.dst[i], L->dma_cpu, stage + (int64_t)i * unit_all, L->dma_gpu,
+                                                                                    bytes, 0, nullptr, L->dma_sig[slot],
+                                                                                    (hsa_amd_sdma_engine_id_t)L->off_engine, false)
+                                              : hsa_amd_memory_async_copy(L->off.dst[i], L->dma_cpu, stage + (int64_t)i * unit_all, L->dma_gpu, bytes, 0,
+                                                                          nullptr, L->dma_sig[slot]);
         if (hs != HSA_STATUS_SUCCESS) {
             // give the engine path up for this layer: let what was issued finish, the stream path copies the units again
             hsa_signal_subtract_relaxed(L->dma_sig[slot], runs - issued);
@@ -497,8 +503,25 @@ void efetch_setup(Layer *L) {
     }
     uint32_t mask = 0;
     if (hsa_amd_memory_copy_engine_status(L->dma_gpu, L->dma_cpu, &mask) != HSA_STATUS_SUCCESS) return;
-    for (int b = 0; b < 32 && (int)L->efetch_engines.size() < kEfetchEngines; ++b)
-        if (mask & (1u << b)) L->efetch_engines.push_back(1u << b);
+    // The engines of the low eight bits of the status mask are the ones that move data without getting in the way of
+    // kernels (with a ninth or a tenth the block's own kernels ran 10-40 % longer, measured).  One of them is kept for
+    // the carved units' way to the host: while that copy (2 MiB per block) shared an engine with the fetch, the units
+    // queued behind it on that engine landed last and the whole fetch waited for them - 47.6 ms per 128K stream
+    // against 44.2 with the engines apart.  INFLLM_SHARED_ENGINES=1 keeps the old assignment (the runtime picks the
+    // offload's engine, the fetch takes all eight), INFLLM_FETCH_ENGINES=n limits the fetch to n engines.
+    const char *ne = getenv("INFLLM_FETCH_ENGINES");
+    const char *sh = getenv("INFLLM_SHARED_ENGINES");
+    const bool shared = sh && sh[0] && sh[0] != '0';
+    const int want_engines = ne && atoi(ne) > 0 ? atoi(ne) : kEfetchEngines;
+    uint32_t d2h = 0;
+    if (shared || hsa_amd_memory_copy_engine_status(L->dma_cpu, L->dma_gpu, &d2h) != HSA_STATUS_SUCCESS) d2h = 0;
+    std::vector<uint32_t> low;
+    for (int b = 0; b < 8; ++b)
+        if (mask & (1u << b)) low.push_back(1u << b);
+    L->off_engine = 0;
+    if (low.size() >= 4 && (d2h & low[1])) L->off_engine = low[1];      // the second one: the first is the fetch's flag engine
+    for (uint32_t e : low)
+        if (e != L->off_engine && (int)L->efetch_engines.size() < want_engines) L->efetch_engines.push_back(e);
     if (L->efetch_engines.size() < 2) return;
     L->efetch_dev = dev;
     if (!(L->d_efetch_flag = flag_take(dev)) || hipHostMalloc((void **)&L->h_efetch_val, kEfetchVals * sizeof(uint32_t)) != hipSuccess ||
@@ -519,6 +542,16 @@ void efetch_setup(Layer *L) {
     }
     hsa_signal_subtract_relaxed(L->efetch_sig, (hsa_signal_value_t)(L->efetch_engines.size() - issued));
     if (efetch_wait_signal(L->efetch_sig, "layer_create") != 0 || issued != (int)L->efetch_engines.size()) return;
+    if (L->off_engine) {                 // the same for the engine of the other direction; if it refuses, the runtime chooses
+        hsa_signal_store_relaxed(L->efetch_sig, 1);
+        if (hsa_amd_memory_async_copy_on_engine(L->h_efetch_val + (kEfetchVals - 1), L->dma_cpu, L->d_efetch_flag, L->dma_gpu, 4, 0, nullptr,
+                                                L->efetch_sig, (hsa_amd_sdma_engine_id_t)L->off_engine, false) != HSA_STATUS_SUCCESS) {
+            hsa_signal_store_relaxed(L->efetch_sig, 0);
+            L->off_engine = 0;
+        } else if (efetch_wait_signal(L->efetch_sig, "layer_create") != 0)
+            return;
+        L->h_efetch_val[kEfetchVals - 1] = 0;
+    }
     L->efetch_ok = true;
 }
 
@@ -1070,6 +1103,24 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
     const int C = d.H * kD;
     const int n_blocks = (a->n + d.exc - 1) / d.exc;
 
+    // ---- the first block's retrieval first: the host waits for its ids before it can fetch anything for this call,
+    //      and the prologue of the whole call would put 50-60 us in front of them.  The first block's rows go through
+    //      the prologue twice (the second time with the rest of the call, to the same effect).
+    int rc;
+    L->topk_pending = false;
+    L->batch_retrieved = false;
+    const bool retrieve = a->n_units > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL);
+    if (retrieve) {
+        INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "call_front: null representative / score buffer");
+        L->slot ^= 1;
+        rc = run_ingest(L, a, a->d_q, a->d_k, a->d_v, a->n < d.exc ? a->n : d.exc, a->b0, L->slot, true, stream);
+        if (rc) return rc;
+        rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
+        if (rc) return rc;
+        rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, stream);
+        if (rc) return rc;
+    }
+
     // ---- prologue of every token, mean query of every block
     infllm_ingest_args in{};
     in.d_q = a->d_q; in.d_k = a->d_k; in.d_v = a->d_v;
@@ -1083,7 +1134,7 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
     in.d_ring_score = d.d_ring_score; in.ring_cap = d.ring_cap;
     in.d_q_loc = L->bd.d_q_loc; in.d_q_glb = L->bd.d_q_glb;
     in.d_qpart = L->bd.d_qpart;
-    int rc = infllm_ingest(&in, stream);
+    rc = infllm_ingest(&in, stream);
     if (rc) return rc;
     rc = infllm_reduce_partials_blocks(L->bd.d_qpart, d.B, a->n, d.exc, C, L->bd.d_qbar, stream);
     if (rc) return rc;
@@ -1112,17 +1163,7 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
     L->batch_block_rows = (int64_t)nsplit * d.B * d.H * (n_blocks > 1 ? d.exc : a->n);
     L->fresh = batch_view(L, a->b0);
 
-    // ---- the first block's retrieval
-    L->topk_pending = false;
-    L->batch_retrieved = false;
-    if (a->n_units > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL)) {
-        INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "call_front: null representative / score buffer");
-        rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
-        if (rc) return rc;
-        rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, stream);
-        if (rc) return rc;
-        L->batch_retrieved = true;
-    }
+    L->batch_retrieved = retrieve;
     return 0;
 }
 
