@@ -386,7 +386,8 @@ def main():
     unit_bytes = 2 * HKV * KNOBS["block_size"] * D * 2
     res["host_link"] = {"missed_units_per_step": cm_stats["misses"], "bytes_per_step": cm_stats["misses"] * unit_bytes,
                         "avg_GBps": cm_stats["misses"] * unit_bytes / (dt / args.steps) / 1e9,
-                        "note": "PCIe 5.0 x16: 64 GB/s raw; 8 DMA engines move 13 x 512 KiB units at 54 GB/s on an idle GPU, 44 GB/s beside the stream's kernels"}
+                        "note": "PCIe 5.0 x16: 64 GB/s raw; 8 DMA engines move 13 x 512 KiB units at 54 GB/s on an idle GPU; in the stream 7 engines fetch "
+                                "(a block's ~14 units in 140-165 us beside its kernels) and the 8th takes the carved units to the host"}
     if not args.no_hbm_leg:
         res["roofline_hbm"] = hbm_leg(dev)
     if args.cpu_tokens > 0:

@@ -303,7 +303,7 @@ void *infllm_host_device_pointer(void *h_pinned);
  *                        before the representatives, since nothing waits for the selection at once);
  *   infllm_block_prefetch  (optional, further down) starts the NEXT block's fetch from its candidates.
  *
- * The fetch of missed units goes through 8 DMA engines (ROCr copies) for blocks of 64 queries or more, and the
+ * The fetch of missed units goes through 7 DMA engines (ROCr copies) for blocks of 64 queries or more, and the
  * main stream waits with hipStreamWaitValue32 for a sequence number the engines write behind the units; shorter
  * blocks, and processes without usable engines (or with INFLLM_NO_DMA_FETCH=1), use the zero-copy kernel
  * of infllm_fetch_units on the copy stream.  Either way the fetch is ordered behind the last reader of the slots
