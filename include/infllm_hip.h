@@ -521,6 +521,10 @@ int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, 
 int infllm_block_prefetch(void *layer, const infllm_select_args *a, void *stream, void *copy_stream);
 /* how many guesses were made / turned out to be the selection */
 int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed);
+/* Missed units that were served from a carve staging slot so far (a device-to-device copy on the main stream instead
+ * of a transfer from pinned host memory; MemoryUnit.load, context_manager.py:76-91, for a unit whose gather into
+ * staging is at most four carving blocks old).  INFLLM_NO_STAGING_COPY=1 (read by infllm_layer_create) turns it off. */
+int64_t infllm_layer_staged_units(void *layer);
 
 /* Event timing of the two attention stages (for benchmarks): enable with a record
  * capacity and a stride (every stride-th launch of each stage is bracketed by two events; an event pair

@@ -378,6 +378,10 @@ class ContextManager:
                   "infllm_layer_prefetch_stats")
         return issued.value, confirmed.value
 
+    def staged_units(self):
+        """Missed units that were copied from a carve staging slot instead of coming from pinned host memory."""
+        return int(self._lib.infllm_layer_staged_units(self._layer)) if self._layer else 0
+
     def read_timing(self, which):
         """[(ms, n_queries, n_keys)] of the timed launches; which = 0 local stage, 1 global stage."""
         cap = self._timing_cap

@@ -102,6 +102,8 @@ struct Layer {
     std::vector<int> stage_first, stage_count;
     hipEvent_t stage_copied = nullptr;                 // behind the last such copy
     std::vector<int64_t> stage_copy_dst;               // slots (row * max_cached + slot) such copies may still be on their way to
+    bool stage_copy_ok = true;                         // INFLLM_NO_STAGING_COPY=1: every missed unit comes from the host
+    int64_t staged_units = 0;                          // missed units served from a staging slot so far
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
     int32_t topk_seq = 0;
@@ -642,7 +644,7 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
         const int64_t unit_all = (int64_t)d.B * slot_elems;
         for (int i = 0; i < n_miss; ++i) {
             int at = -1;
-            for (size_t sl = 0; sl < L->stage_count.size() && at < 0; ++sl)
+            for (size_t sl = 0; L->stage_copy_ok && sl < L->stage_count.size() && at < 0; ++sl)
                 if (units[i] >= L->stage_first[sl] && units[i] < L->stage_first[sl] + L->stage_count[sl]) at = (int)sl;
             if (at < 0) continue;
             INFLLM_REQUIRE(rows[i] >= 0 && rows[i] < d.B && slots[i] >= 0 && slots[i] < d.max_cached, "fetch: bad miss entry");
@@ -662,6 +664,7 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
             L->stage_copy_dst.push_back((int64_t)rows[i] * d.max_cached + slots[i]);
             staged[i] = 1;
             ++n_staged;
+            ++L->staged_units;
         }
         if (n_staged > 0) {
             HIP_OK(hipEventRecord(L->stage_copied, ms), "fetch: event");
@@ -815,6 +818,8 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         L->ahead_any_path = any && any[0] && any[0] != '0';
         const char *fs = getenv("INFLLM_FUSED_STAGES");
         L->local_in_front = !(fs && fs[0] && fs[0] != '0');
+        const char *ns = getenv("INFLLM_NO_STAGING_COPY");
+        L->stage_copy_ok = !(ns && ns[0] && ns[0] != '0');
     }
     if (hipHostMalloc((void **)&L->h_cand, ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
         (void)hipGetLastError();
@@ -1426,6 +1431,11 @@ extern "C" int infllm_block_prefetch(void *layer, const infllm_select_args *a, v
     g.active = true;
     ++L->ahead_issued;
     return g.n_miss_all;
+}
+
+extern "C" int64_t infllm_layer_staged_units(void *layer) {
+    if (!layer) return infllm_fail(-1, "layer_staged_units: null layer");
+    return ((Layer *)layer)->staged_units;
 }
 
 extern "C" int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed) {

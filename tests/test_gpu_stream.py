@@ -205,6 +205,37 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
     assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
 
 
+def test_units_still_in_a_staging_slot_are_copied_from_there(monkeypatch):
+    """A missed unit whose rows are still in the staging slot they were gathered into when the unit was carved (the
+    last four carving blocks) is copied from there on the main stream instead of being read back from pinned host
+    memory.  Same bytes either way: outputs bit for bit, same residency events - with the fetch ahead of the selection
+    (whose wrong guesses are the blocks in which a just-carved unit is selected), without it, through the engines and
+    through the fetch kernel, on one stream and with the side stream."""
+    from infllm_amd.attention import ContextManager
+    T = 2600
+    q, k, v = make_stream(T, 8, 2, 27, B=2)
+    served = 0
+    for extra in (dict(max_cached_block=5, async_global_stream=True), dict(max_cached_block=9), dict(max_cached_block=6, cache_strategy="fifo")):
+        kw = dict(SMALL, **extra)
+        for ahead in (True, False):
+            monkeypatch.setattr(ContextManager, "fetch_ahead", ahead)
+            for no_dma in ("0", "1"):
+                monkeypatch.setenv("INFLLM_NO_DMA_FETCH", no_dma)
+                monkeypatch.setenv("INFLLM_FETCH_AHEAD_ALWAYS", "1")
+                monkeypatch.setenv("INFLLM_NO_STAGING_COPY", "1")
+                host, cm0 = run_gpu(q, k, v, [1300, 1300], 1e4, **kw)
+                assert cm0.staged_units() == 0
+                monkeypatch.delenv("INFLLM_NO_STAGING_COPY")
+                staged, cm1 = run_gpu(q, k, v, [1300, 1300], 1e4, **kw)
+                served += cm1.staged_units()
+                assert torch.equal(host, staged) and cm0.stats == cm1.stats
+                for u in range(2):
+                    assert cm0.policy[u].evicted_log == cm1.policy[u].evicted_log and cm0.policy[u].cached == cm1.policy[u].cached
+    monkeypatch.delenv("INFLLM_NO_DMA_FETCH")
+    monkeypatch.delenv("INFLLM_FETCH_AHEAD_ALWAYS")
+    assert served > 20                  # fresh units do get selected in this stream
+
+
 def test_stage_timers_sample_the_launches_they_are_asked_for(monkeypatch):
     """infllm_layer_timing / infllm_layer_read_timing (what bench.py's roofline figure is made of): every stride-th
     launch of the local stage, of the global stage and of the stream's wait for the fetch is bracketed by events; the
