@@ -1101,6 +1101,7 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
     INFLLM_REQUIRE(a->n >= 1 && a->n <= L->bd.max_tokens, "call_front: %d tokens do not fit the buffers (%d)", a->n, L->bd.max_tokens);
     INFLLM_REQUIRE(a->n <= d.ring_cap, "call_front: %d tokens do not fit a ring of %lld rows", a->n, (long long)d.ring_cap);
     INFLLM_REQUIRE(a->n_units >= 0 && a->b0 >= 0, "call_front: negative state");
+    INFLLM_REQUIRE(a->d_q && a->d_k && a->d_v, "call_front: null q / k / v");
     L->main_stream = st;
     L->main_stream_known = true;
     L->batch_live = false;
