@@ -65,7 +65,9 @@ struct Layer {
     // its pinned source values, and the sequence number of the fetch in flight.
     bool efetch_ok = false;
     std::vector<uint32_t> efetch_engines;
-    hsa_signal_t efetch_sig{}, efetch_flag_sig{};
+    hsa_signal_t efetch_sig[2]{}, efetch_flag_sig[2]{};   // two sets, used in turn: a fetch may be issued while the one before is in flight
+    bool efetch_prev_in_use = false;                   // the last fetch wrote only slots of the selection in use
+    bool efetch_overlap = true;                        // INFLLM_FETCH_OVERLAP=0: one fetch at a time
     uint32_t *d_efetch_flag = nullptr, *h_efetch_val = nullptr;
     int efetch_dev = 0;
     uint32_t off_engine = 0;                           // the engine that takes carved units to the host (0: the runtime's choice)
@@ -460,6 +462,16 @@ int efetch_wait_signal(hsa_signal_t sig, const char *what) {
     return 0;
 }
 
+// every fetch issued so far has landed (flag copies included)
+int efetch_wait_all(Layer *L, const char *what) {
+    for (int i = 0; i < 2; ++i) {
+        if (!L->efetch_flag_sig[i].handle) continue;
+        const int rc = efetch_wait_signal(L->efetch_flag_sig[i], what);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
 // Flag words in signal memory are never given back to the runtime: memory of that kind that a kernel has read (the
 // stream's wait is a kernel) is best not freed while the process lives, so a layer that goes away leaves its word
 // to the next one on the same device.
@@ -527,33 +539,36 @@ void efetch_setup(Layer *L) {
     if (L->efetch_engines.size() < 2) return;
     L->efetch_dev = dev;
     if (!(L->d_efetch_flag = flag_take(dev)) || hipHostMalloc((void **)&L->h_efetch_val, kEfetchVals * sizeof(uint32_t)) != hipSuccess ||
-        hsa_signal_create(0, 0, nullptr, &L->efetch_sig) != HSA_STATUS_SUCCESS ||
-        hsa_signal_create(0, 0, nullptr, &L->efetch_flag_sig) != HSA_STATUS_SUCCESS) {
+        hsa_signal_create(0, 0, nullptr, &L->efetch_sig[0]) != HSA_STATUS_SUCCESS ||
+        hsa_signal_create(0, 0, nullptr, &L->efetch_flag_sig[0]) != HSA_STATUS_SUCCESS ||
+        hsa_signal_create(0, 0, nullptr, &L->efetch_sig[1]) != HSA_STATUS_SUCCESS ||
+        hsa_signal_create(0, 0, nullptr, &L->efetch_flag_sig[1]) != HSA_STATUS_SUCCESS) {
         (void)hipGetLastError();
         return;
     }
     // the first copy on an engine creates its queue (milliseconds): do that here, once per process and engine
     for (int i = 0; i < kEfetchVals; ++i) L->h_efetch_val[i] = 0;
-    hsa_signal_store_relaxed(L->efetch_sig, (hsa_signal_value_t)L->efetch_engines.size());
+    hsa_signal_store_relaxed(L->efetch_sig[0], (hsa_signal_value_t)L->efetch_engines.size());
     int issued = 0;
     for (uint32_t e : L->efetch_engines) {
-        if (hsa_amd_memory_async_copy_on_engine(L->d_efetch_flag, L->dma_gpu, L->h_efetch_val, L->dma_cpu, 4, 0, nullptr, L->efetch_sig,
+        if (hsa_amd_memory_async_copy_on_engine(L->d_efetch_flag, L->dma_gpu, L->h_efetch_val, L->dma_cpu, 4, 0, nullptr, L->efetch_sig[0],
                                                 (hsa_amd_sdma_engine_id_t)e, false) != HSA_STATUS_SUCCESS)
             break;
         ++issued;
     }
-    hsa_signal_subtract_relaxed(L->efetch_sig, (hsa_signal_value_t)(L->efetch_engines.size() - issued));
-    if (efetch_wait_signal(L->efetch_sig, "layer_create") != 0 || issued != (int)L->efetch_engines.size()) return;
+    hsa_signal_subtract_relaxed(L->efetch_sig[0], (hsa_signal_value_t)(L->efetch_engines.size() - issued));
+    if (efetch_wait_signal(L->efetch_sig[0], "layer_create") != 0 || issued != (int)L->efetch_engines.size()) return;
     if (L->off_engine) {                 // the same for the engine of the other direction; if it refuses, the runtime chooses
-        hsa_signal_store_relaxed(L->efetch_sig, 1);
+        hsa_signal_store_relaxed(L->efetch_sig[0], 1);
         if (hsa_amd_memory_async_copy_on_engine(L->h_efetch_val + (kEfetchVals - 1), L->dma_cpu, L->d_efetch_flag, L->dma_gpu, 4, 0, nullptr,
-                                                L->efetch_sig, (hsa_amd_sdma_engine_id_t)L->off_engine, false) != HSA_STATUS_SUCCESS) {
-            hsa_signal_store_relaxed(L->efetch_sig, 0);
+                                                L->efetch_sig[0], (hsa_amd_sdma_engine_id_t)L->off_engine, false) != HSA_STATUS_SUCCESS) {
+            hsa_signal_store_relaxed(L->efetch_sig[0], 0);
             L->off_engine = 0;
-        } else if (efetch_wait_signal(L->efetch_sig, "layer_create") != 0)
+        } else if (efetch_wait_signal(L->efetch_sig[0], "layer_create") != 0)
             return;
         L->h_efetch_val[kEfetchVals - 1] = 0;
     }
+    { const char *ov = getenv("INFLLM_FETCH_OVERLAP"); L->efetch_overlap = !(ov && ov[0] == '0'); }
     L->efetch_ok = true;
 }
 
@@ -571,38 +586,47 @@ int fetch_by_engines(Layer *L, int n_miss, const void *const *srcs, int64_t nbyt
         (void)hipGetLastError();
         HIP_OK(hipEventSynchronize(L->global_done), "fetch: wait global");
     }
-    // One fetch at a time: the host waits here until the previous one has landed (in a long prefill that is some 40 us
-    // of every block - the link is busy three quarters of the time).  Letting the next fetch start while this one is
-    // in flight (a second set of signals) was measured: its copies take bandwidth from the stragglers of the fetch the
-    // stream is waiting for, the waits grow and the stream is no faster.
-    int rc = efetch_wait_signal(L->efetch_flag_sig, "fetch");
+    // A fetch ahead writes no slot of the selection in use, and those are all that the fetch before it writes (unless
+    // that one also put back what a wrong guess had overwritten): the two may be in flight together, each engine
+    // taking its copies in the order they were issued, so the link does not idle between one fetch's landing and the
+    // host's issue of the next; the host only makes sure that the fetch before the last has landed (whose signals this
+    // one takes over).  Any other fetch lets everything land first.  Measured with the engines told apart (see
+    // efetch_setup): 43.1-43.6 ms per 128K stream against 43.7-43.8 with one fetch at a time (INFLLM_FETCH_OVERLAP=0);
+    // while the carved units' copy to the host still shared an engine with the fetch the overlap lost (the next
+    // fetch's copies took bandwidth from the stragglers the stream was waiting for).
+    const int set = (int)((L->efetch_seq + 1) & 1u);
+    int rc = L->efetch_overlap && ahead && L->efetch_prev_in_use ? efetch_wait_signal(L->efetch_flag_sig[set], "fetch") : efetch_wait_all(L, "fetch");
     if (rc) return rc;
     const uint32_t seq = ++L->efetch_seq;
-    uint32_t *val = L->h_efetch_val + (seq % kEfetchVals);
+    uint32_t *val = L->h_efetch_val + (seq % (kEfetchVals - 1));
     *val = seq;
-    hsa_signal_store_relaxed(L->efetch_sig, n_miss);
-    hsa_signal_store_relaxed(L->efetch_flag_sig, 1);
+    hsa_signal_t sig = L->efetch_sig[set], flag_sig = L->efetch_flag_sig[set];
+    hsa_signal_store_relaxed(sig, n_miss);
+    hsa_signal_store_relaxed(flag_sig, 1);
     int issued = 0;
     bool ok = true;
     for (int i = 0; i < n_miss && ok; ++i) {
-        ok = hsa_amd_memory_async_copy_on_engine(L->fetch_dst[i], L->dma_gpu, srcs[i], L->dma_cpu, (size_t)nbytes, 0, nullptr, L->efetch_sig,
+        ok = hsa_amd_memory_async_copy_on_engine(L->fetch_dst[i], L->dma_gpu, srcs[i], L->dma_cpu, (size_t)nbytes, 0, nullptr, sig,
                                                  (hsa_amd_sdma_engine_id_t)L->efetch_engines[i % L->efetch_engines.size()], false) ==
              HSA_STATUS_SUCCESS;
         issued += ok ? 1 : 0;
     }
+    // the sequence number goes out behind the units, on the engine that wrote the one before: the flag never steps back
     if (ok)
-        ok = hsa_amd_memory_async_copy_on_engine(L->d_efetch_flag, L->dma_gpu, val, L->dma_cpu, 4, 1, &L->efetch_sig, L->efetch_flag_sig,
+        ok = hsa_amd_memory_async_copy_on_engine(L->d_efetch_flag, L->dma_gpu, val, L->dma_cpu, 4, 1, &sig, flag_sig,
                                                  (hsa_amd_sdma_engine_id_t)L->efetch_engines[0], false) == HSA_STATUS_SUCCESS;
     if (!ok) {
         // give the engine path up: let what was issued land, then the kernel copies everything again
-        hsa_signal_subtract_relaxed(L->efetch_sig, n_miss - issued);
-        hsa_signal_store_relaxed(L->efetch_flag_sig, 0);
-        rc = efetch_wait_signal(L->efetch_sig, "fetch");
+        hsa_signal_subtract_relaxed(sig, n_miss - issued);
+        hsa_signal_store_relaxed(flag_sig, 0);
+        rc = efetch_wait_signal(sig, "fetch");
+        if (!rc) rc = efetch_wait_all(L, "fetch");
         L->efetch_ok = false;
         --L->efetch_seq;
         return rc;
     }
     L->efetch_wait = true;
+    L->efetch_prev_in_use = true;
     return 1;
 }
 
@@ -652,7 +676,7 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
                 // an earlier fetch may still be on its way to the same slot (a guess that turned out wrong put another
                 // unit there; a repair put back one that is evicted again): it lands first
                 if (L->efetch_ok) {
-                    const int wrc = efetch_wait_signal(L->efetch_flag_sig, "fetch");
+                    const int wrc = efetch_wait_all(L, "fetch");
                     if (wrc) return wrc;
                 }
                 if (L->fetch_wait && ms != cs) HIP_OK(hipStreamWaitEvent(ms, L->fetch_done, 0), "fetch: wait fetch");
@@ -717,7 +741,7 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
         if (erc < 0) return erc;
         if (erc == 0) {
             if (L->efetch_ok) {                   // engine copies of an earlier fetch may aim at the same slots
-                const int wrc = efetch_wait_signal(L->efetch_flag_sig, "fetch");
+                const int wrc = efetch_wait_all(L, "fetch");
                 if (wrc) return wrc;
             }
             if (side && L->has_global && !ahead) HIP_OK(hipStreamWaitEvent(cs, L->global_done, 0), "fetch: wait global");
@@ -855,13 +879,15 @@ extern "C" int infllm_layer_destroy(void *layer) {
     if (L->h_cand) (void)hipHostFree(L->h_cand);
     for (void *c : L->ahead.shadow)
         if (c) (void)infllm_cache_destroy(c);
-    if (L->efetch_sig.handle) {
-        (void)efetch_wait_signal(L->efetch_sig, "layer_destroy");
-        (void)hsa_signal_destroy(L->efetch_sig);
-    }
-    if (L->efetch_flag_sig.handle) {
-        (void)efetch_wait_signal(L->efetch_flag_sig, "layer_destroy");
-        (void)hsa_signal_destroy(L->efetch_flag_sig);
+    for (int i = 0; i < 2; ++i) {
+        if (L->efetch_sig[i].handle) {
+            (void)efetch_wait_signal(L->efetch_sig[i], "layer_destroy");
+            (void)hsa_signal_destroy(L->efetch_sig[i]);
+        }
+        if (L->efetch_flag_sig[i].handle) {
+            (void)efetch_wait_signal(L->efetch_flag_sig[i], "layer_destroy");
+            (void)hsa_signal_destroy(L->efetch_flag_sig[i]);
+        }
     }
     if (L->d_efetch_flag) flag_give(L->efetch_dev, L->d_efetch_flag);
     if (L->h_efetch_val) (void)hipHostFree(L->h_efetch_val);
@@ -1353,7 +1379,9 @@ int ahead_repair(Layer *L, void *const *caches, int n_extra, const int32_t *rows
         sr.push_back(g.victim_src[i]);
     }
     g.victim_unit.clear();
-    return do_fetch(L, (int)r.size(), r.data(), sl.data(), un.data(), sr.data(), st, cs);
+    const int rc = do_fetch(L, (int)r.size(), r.data(), sl.data(), un.data(), sr.data(), st, cs);
+    L->efetch_prev_in_use = false;            // it also wrote slots of units that are not selected: the next guess may evict those
+    return rc;
 }
 
 }  // namespace
@@ -1957,7 +1985,7 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
         if (rrc) return rrc;
         // nothing later is ordered behind this repair by itself: finish it here (it is not a path a stream takes)
         if (L->efetch_ok) {
-            rrc = efetch_wait_signal(L->efetch_flag_sig, "layer_flush");
+            rrc = efetch_wait_all(L, "layer_flush");
             if (rrc) return rrc;
         }
         HIP_OK(hipStreamSynchronize(cs), "layer_flush: repair");

@@ -188,8 +188,9 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
         assert cm0.prefetch_stats() == (0, 0) and cm0.stats["misses"] > 0
         monkeypatch.setattr(ContextManager, "fetch_ahead", True)
         monkeypatch.setenv("INFLLM_FETCH_AHEAD_ALWAYS", "1")       # by default only the engines fetch ahead
-        for no_dma in ("0", "1"):
+        for no_dma, overlap in (("0", "1"), ("0", "0"), ("1", "1")):
             monkeypatch.setenv("INFLLM_NO_DMA_FETCH", no_dma)
+            monkeypatch.setenv("INFLLM_FETCH_OVERLAP", overlap)     # the next fetch issued while the previous one is in flight, or not
             ahead, cm1 = run_gpu(q, k, v, [1300, 1300], 1e4, **kw)
             issued, confirmed = cm1.prefetch_stats()
             assert issued > 0 and 0 <= confirmed <= issued
@@ -201,6 +202,7 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
                 assert cm0.policy[u].cached == cm1.policy[u].cached            # which slot a unit sits in may differ
                 assert sorted(cm1.policy[u].slot_of.values()) == sorted(set(cm1.policy[u].slot_of.values()))
         monkeypatch.delenv("INFLLM_NO_DMA_FETCH")
+        monkeypatch.delenv("INFLLM_FETCH_OVERLAP")
         monkeypatch.delenv("INFLLM_FETCH_AHEAD_ALWAYS")
     assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
 
