@@ -33,6 +33,8 @@ def test_argument_errors_are_reported_not_raised_across_the_abi():
     assert b"null" in lib.infllm_last_error()
     assert lib.infllm_copy_async(None, None, 4, 1, None) < 0
     assert lib.infllm_score_topk(None, 0, 0, 0, None, 0, None, None, None) < 0
+    assert lib.infllm_layer_set_batch(None, None) < 0 and lib.infllm_call_front(None, None, None) < 0
+    assert lib.infllm_layer_staged_units(None) < 0
     with pytest.raises(_lib.InfLLMHipError):
         _lib.check(-1, "probe")
 
@@ -44,6 +46,7 @@ def test_struct_layouts_match_header_sizes():
     assert ctypes.sizeof(_lib.IngestArgs) == 3 * 8 + 9 * 8 + 4 * 4 + 2 * 8 + 8 + 8 + 4 * 8 + 8 + 3 * 8
     assert ctypes.sizeof(_lib.AttnArgs) == 8 + 24 + 16 + 16 + 48 + 24 + 8 + 16 + 8 + 8 + 8 + 16
     assert ctypes.sizeof(_lib.ScoreArgs) == 8 + 24 + 16 + 8 + 24 + 24 + 8 + 16 + 8 + 8 + 8 + 24
+    assert ctypes.sizeof(_lib.BatchDesc) == 6 * 8 + 8 + 2 * 4
 
 
 @pytest.mark.parametrize("strategy", ["lru", "fifo"])
