@@ -335,10 +335,10 @@ def main():
         for _ in range(n):
             cm, out = run_stream(q, k, v, args.chunk, timing=True)
             if prev is not None:
-                records.append((prev.read_timing(0), prev.read_timing(1), prev.read_timing(2), prev.prefetch_stats(), dict(prev.stats)))
+                records.append((prev.read_timing(0), prev.read_timing(1), prev.read_timing(2), prev.prefetch_stats(), dict(prev.stats), (prev.fetched_units(), prev.staged_units())))
             prev = cm
         torch.cuda.synchronize()
-        records.append((prev.read_timing(0), prev.read_timing(1), prev.read_timing(2), prev.prefetch_stats(), dict(prev.stats)))
+        records.append((prev.read_timing(0), prev.read_timing(1), prev.read_timing(2), prev.prefetch_stats(), dict(prev.stats), (prev.fetched_units(), prev.staged_units())))
         return records, out
 
     run_steps(args.warmup) if args.warmup > 0 else None
@@ -384,10 +384,14 @@ def main():
     # what the stream as a whole is bound by: the missed units' way from pinned host memory over PCIe (repairs of wrong
     # guesses come on top of the misses counted here)
     unit_bytes = 2 * HKV * KNOBS["block_size"] * D * 2
-    res["host_link"] = {"missed_units_per_step": cm_stats["misses"], "bytes_per_step": cm_stats["misses"] * unit_bytes,
-                        "avg_GBps": cm_stats["misses"] * unit_bytes / (dt / args.steps) / 1e9,
-                        "note": "PCIe 5.0 x16: 64 GB/s raw; 8 DMA engines move 13 x 512 KiB units at 54 GB/s on an idle GPU; in the stream 7 engines fetch "
-                                "(a block's ~14 units in 140-165 us beside its kernels) and the 8th takes the carved units to the host"}
+    moved, staged = runs[-1][5]
+    res["host_link"] = {"missed_units_per_step": cm_stats["misses"], "units_from_host_per_step": moved,
+                        "units_from_staging_per_step": staged, "bytes_per_step": moved * unit_bytes,
+                        "avg_GBps": moved * unit_bytes / (dt / args.steps) / 1e9,
+                        "note": "units_from_host counts every 512 KiB unit that crossed PCIe towards the device: the selections' misses, "
+                                "candidates a guess fetched in vain and what its repair brought back; units still in a carve staging slot "
+                                "are copied on the device.  PCIe 5.0 x16: 64 GB/s raw; 8 DMA engines move 13 units at 54 GB/s on an idle "
+                                "GPU; in the stream 7 engines fetch and the 8th takes the carved units to the host"}
     if not args.no_hbm_leg:
         res["roofline_hbm"] = hbm_leg(dev)
     if args.cpu_tokens > 0:

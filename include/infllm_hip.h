@@ -525,6 +525,10 @@ int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed
  * of a transfer from pinned host memory; MemoryUnit.load, context_manager.py:76-91, for a unit whose gather into
  * staging is at most four carving blocks old).  INFLLM_NO_STAGING_COPY=1 (read by infllm_layer_create) turns it off. */
 int64_t infllm_layer_staged_units(void *layer);
+/* Units moved from pinned host memory to the slab so far, whichever way (DMA engines or the fetch kernel): the misses
+ * of the selections, the candidates a guess fetched that were not selected after all, and what a wrong guess's
+ * repair brought back - the host-to-device traffic of MemoryUnit.load (context_manager.py:76-91) in units. */
+int64_t infllm_layer_fetched_units(void *layer);
 
 /* Event timing of the two attention stages (for benchmarks): enable with a record
  * capacity and a stride (every stride-th launch of each stage is bracketed by two events; an event pair

@@ -45,7 +45,8 @@ _HOST_CHUNK_UNITS = 64       # units per pinned host allocation
 _MAX_SPLITS = 16             # key splits of one attention stage
 _NUM_CUS = 256               # MI355X
 _PAGE_SLOTS = 4
-_CARVE_SLOTS = 4
+_CARVE_SLOTS = 4             # staging slots of the carve, used in turn (more of them serve more misses on the device - 16: 18 %,
+                             # 64: 57 % of the benchmark stream's - but the stream is no faster for it, measured)
 
 
 class CachePolicy:
@@ -381,6 +382,10 @@ class ContextManager:
     def staged_units(self):
         """Missed units that were copied from a carve staging slot instead of coming from pinned host memory."""
         return int(self._lib.infllm_layer_staged_units(self._layer)) if self._layer else 0
+
+    def fetched_units(self):
+        """Units moved from pinned host memory to the device cache so far (wrongly guessed ones and repairs included)."""
+        return int(self._lib.infllm_layer_fetched_units(self._layer)) if self._layer else 0
 
     def read_timing(self, which):
         """[(ms, n_queries, n_keys)] of the timed launches; which = 0 local stage, 1 global stage."""

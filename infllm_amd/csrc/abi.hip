@@ -113,6 +113,29 @@ extern "C" int infllm_fetch_units(const void *const *h_src, void *const *d_dst, 
     return 0;
 }
 
+// library-internal: the same for sources in device memory (units that are still in a carve staging slot): one launch
+// for all of them, shaped for HBM rather than for PCIe (16 KiB per workgroup, as many workgroups as there are pieces)
+int infllm_copy_units(const void *const *d_src, void *const *d_dst, int32_t n, int64_t nbytes, void *stream) {
+    INFLLM_REQUIRE(n >= 0 && nbytes > 0 && nbytes % 16 == 0, "copy_units: bad sizes n=%d nbytes=%lld", n, (long long)nbytes);
+    INFLLM_REQUIRE(n == 0 || (d_src && d_dst), "copy_units: null list");
+    for (int first = 0; first < n; first += kFetchMax) {
+        const int m = n - first < kFetchMax ? n - first : kFetchMax;
+        FetchList list;
+        for (int i = 0; i < m; ++i) {
+            INFLLM_REQUIRE(d_src[first + i] && d_dst[first + i], "copy_units: null entry %d", first + i);
+            INFLLM_REQUIRE(((uintptr_t)d_src[first + i] | (uintptr_t)d_dst[first + i]) % 16 == 0, "copy_units: entry %d is not 16-byte aligned",
+                           first + i);
+            list.src[i] = (const uint4 *)d_src[first + i];
+            list.dst[i] = (uint4 *)d_dst[first + i];
+        }
+        const int64_t piece = 256 * 4 * 16;
+        const int64_t work = (int64_t)m * ((nbytes + piece - 1) / piece);
+        hipLaunchKernelGGL(unit_fetch_kernel<4>, dim3((unsigned)(work < 2048 ? work : 2048)), dim3(256), 0, (hipStream_t)stream, list, m, nbytes);
+        INFLLM_CHECK_LAUNCH("copy_units");
+    }
+    return 0;
+}
+
 extern "C" void *infllm_host_device_pointer(void *h_pinned) {
     void *d = nullptr;
     if (!h_pinned || hipHostGetDevicePointer(&d, h_pinned, 0) != hipSuccess) {

@@ -106,6 +106,7 @@ struct Layer {
     std::vector<int64_t> stage_copy_dst;               // slots (row * max_cached + slot) such copies may still be on their way to
     bool stage_copy_ok = true;                         // INFLLM_NO_STAGING_COPY=1: every missed unit comes from the host
     int64_t staged_units = 0;                          // missed units served from a staging slot so far
+    int64_t fetched_units = 0;                         // units moved from pinned host memory so far (guessed ones and repairs included)
     hipEvent_t mass_done = nullptr;
     bool mass_pending = false;
     int32_t topk_seq = 0;
@@ -173,6 +174,7 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
 int infllm_inline_page_limit();
+int infllm_copy_units(const void *const *d_src, void *const *d_dst, int32_t n, int64_t nbytes, void *stream);
 int infllm_attn_stage_blocked(const infllm_attn_args *a, int32_t exc, int64_t block_rows, void *stream);
 int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2, const float *d_lse_part2,
                        int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
@@ -664,6 +666,8 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
         }
         hipStream_t ms = L->main_stream_known ? L->main_stream : st;       // the stream the staging slots are filled on
         std::vector<char> staged(n_miss, 0);
+        std::vector<const void *> st_src;
+        std::vector<void *> st_dst;
         int n_staged = 0;
         const int64_t unit_all = (int64_t)d.B * slot_elems;
         for (int i = 0; i < n_miss; ++i) {
@@ -684,13 +688,16 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
             const bf16_t *src = (const bf16_t *)d.d_carve_stage + ((int64_t)at * d.max_carve + (units[i] - L->stage_first[at])) * unit_all +
                                 (int64_t)rows[i] * slot_elems;
             bf16_t *dst = (bf16_t *)d.d_slab + ((int64_t)rows[i] * d.max_cached + slots[i]) * slot_elems;
-            HIP_OK(hipMemcpyAsync(dst, src, slot_elems * sizeof(bf16_t), hipMemcpyDeviceToDevice, ms), "fetch: copy from staging");
+            st_src.push_back(src);
+            st_dst.push_back(dst);
             L->stage_copy_dst.push_back((int64_t)rows[i] * d.max_cached + slots[i]);
             staged[i] = 1;
             ++n_staged;
             ++L->staged_units;
         }
         if (n_staged > 0) {
+            const int crc = infllm_copy_units(st_src.data(), st_dst.data(), n_staged, slot_elems * (int64_t)sizeof(bf16_t), ms);      // one launch for all
+            if (crc) return crc;
             HIP_OK(hipEventRecord(L->stage_copied, ms), "fetch: event");
             for (int i = 0; i < n_miss; ++i) {
                 if (staged[i]) continue;
@@ -730,6 +737,7 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
                 if (wrc) return wrc;
             }
         }
+        L->fetched_units += n_miss;
         L->fetch_dst.resize(n_miss);
         for (int i = 0; i < n_miss; ++i) {
             INFLLM_REQUIRE(rows[i] >= 0 && rows[i] < d.B && slots[i] >= 0 && slots[i] < d.max_cached && srcs[i], "fetch: bad miss entry");
@@ -1465,6 +1473,11 @@ extern "C" int infllm_block_prefetch(void *layer, const infllm_select_args *a, v
 extern "C" int64_t infllm_layer_staged_units(void *layer) {
     if (!layer) return infllm_fail(-1, "layer_staged_units: null layer");
     return ((Layer *)layer)->staged_units;
+}
+
+extern "C" int64_t infllm_layer_fetched_units(void *layer) {
+    if (!layer) return infllm_fail(-1, "layer_fetched_units: null layer");
+    return ((Layer *)layer)->fetched_units;
 }
 
 extern "C" int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed) {

@@ -34,7 +34,7 @@ def test_argument_errors_are_reported_not_raised_across_the_abi():
     assert lib.infllm_copy_async(None, None, 4, 1, None) < 0
     assert lib.infllm_score_topk(None, 0, 0, 0, None, 0, None, None, None) < 0
     assert lib.infllm_layer_set_batch(None, None) < 0 and lib.infllm_call_front(None, None, None) < 0
-    assert lib.infllm_layer_staged_units(None) < 0
+    assert lib.infllm_layer_staged_units(None) < 0 and lib.infllm_layer_fetched_units(None) < 0
     with pytest.raises(_lib.InfLLMHipError):
         _lib.check(-1, "probe")
 
