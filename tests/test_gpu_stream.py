@@ -21,6 +21,7 @@ def call_mode(request, monkeypatch):
     """How an append() call is prepared: prologue and mean queries of the whole call at once and the local stage for
     two blocks per launch (infllm_call_front, the default), or every block on its own (call_tokens = 0)."""
     from infllm_amd.attention import ContextManager
+    monkeypatch.delenv("INFLLM_CALL_TOKENS", raising=False)
     if request.param == "block by block":
         monkeypatch.setattr(ContextManager, "call_tokens", 0)
     return request.param
@@ -248,6 +249,8 @@ def test_stage_timers_sample_the_launches_they_are_asked_for(monkeypatch):
     q, k, v = make_stream(T, 8, 2, 23)
     kw = dict(SMALL, max_cached_block=5, async_global_stream=True)
     exc = kw["exc_block_size"]
+    monkeypatch.delenv("INFLLM_CALL_TOKENS", raising=False)
+    monkeypatch.delenv("INFLLM_LOCAL_GROUP", raising=False)
     for call_tokens in (0, 16 * exc):
         monkeypatch.setattr(ContextManager, "call_tokens", call_tokens)
         plain, _ = run_gpu(q, k, v, [T], 1e4, **kw)
