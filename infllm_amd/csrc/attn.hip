@@ -557,65 +557,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
     if (grp == 0) a.d_lse_part[row] = l_tot > 0.f ? m_run * scale + log2f(l_tot) : -INFINITY;
 }
 
-// The partials of a merge may lie in two places: the first n_first of them behind the pointers the kernel is given,
-// the rest wherever the second stage wrote them.  skip_l / skip_o are what has to be added to an index into the first
-// buffers (log-sum-exps; fp16 elements beyond the row term) to land in the second.
-struct PartSets {
-    int32_t n_first;
-    int64_t skip_l, skip_o;
-    __device__ __forceinline__ int64_t l(int p, int64_t rows) const { return (int64_t)p * rows + (p >= n_first ? skip_l : 0); }
-    __device__ __forceinline__ int64_t o(int p) const { return p >= n_first ? skip_o : 0; }
-};
-
-// one thread per (row, 8 dims): P fp16 partials -> bf16 output row + final lse
-__global__ __launch_bounds__(256) void attn_merge_kernel(const _Float16 *o_part, const float *lse_part, int P, int B, int H,
-                                                         int Lq, bf16_t *out, int64_t o_sb, int64_t o_sh, int64_t o_sl,
-                                                         float *lse_out, PartSets ps) {
-    const int64_t rows = (int64_t)B * H * Lq;
-    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t row = e >> 4;
-    const int c = (int)(e & 15);
-    if (row >= rows) return;
-    // partials in batches of 8 so that the loads of a batch are in flight together (decode-sized blocks merge
-    // dozens of partials of very few rows: a chain of dependent loads would be all latency)
-    float m = -INFINITY;
-    for (int p0 = 0; p0 < P; p0 += 8) {
-        float l8[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) l8[i] = p0 + i < P ? lse_part[ps.l(p0 + i, rows) + row] : -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) m = fmaxf(m, l8[i]);
-    }
-    float acc[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
-    float den = 0.f;
-    if (m > -INFINITY) {
-        for (int p0 = 0; p0 < P; p0 += 8) {
-            float l8[8];
-            f16x8 o8[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const bool on = p0 + i < P;
-                l8[i] = on ? lse_part[ps.l(p0 + i, rows) + row] : -INFINITY;
-                o8[i] = on ? *(const f16x8 *)(o_part + (ps.l(p0 + i, rows) + row) * kD + ps.o(p0 + i) + c * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            }
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float w = __builtin_amdgcn_exp2f(l8[i] - m);       // exp2(-inf) = 0: empty partials hold zeros
-#pragma unroll
-                for (int j = 0; j < 8; ++j) acc[j] += (float)o8[i][j] * w;
-                den += w;
-            }
-        }
-    }
-    const float inv = den > 0.f ? 1.f / den : 0.f;
-    const int i = (int)(row % Lq), h = (int)((row / Lq) % H), b = (int)(row / ((int64_t)Lq * H));
-    u32x4 packed{pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv),
-                 pack_bf16x2(acc[4] * inv, acc[5] * inv), pack_bf16x2(acc[6] * inv, acc[7] * inv)};
-    *(u32x4 *)(out + (int64_t)b * o_sb + (int64_t)h * o_sh + (int64_t)i * o_sl + c * 8) = packed;
-    if (c == 0 && lse_out) lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
-}
+// one thread per (row, 8 dims): P fp16 partials -> bf16 output row + final lse (merge_piece, common.h)
+__global__ __launch_bounds__(256) void attn_merge_kernel(MergeJob job) { merge_piece(job, (int64_t)blockIdx.x * 256 + threadIdx.x); }
 
 // the log-sum-exp half of the merge alone: one thread per row
 __global__ __launch_bounds__(256) void attn_merge_lse_kernel(const float *lse_part, int P, int64_t rows, float *lse_out, PartSets ps) {
@@ -941,15 +884,16 @@ extern "C" int infllm_attn_fwd_noalloc(const infllm_attn_args *local, const infl
     return infllm_attn_fwd(local ? &l : nullptr, global ? &g : nullptr, d_out, o_sb, o_sh, o_sl, d_lse, stream);
 }
 
-// library-internal: the merge over two sets of partials, P1 behind (d_o_part, d_lse_part) and P2 behind
-// (d_o_part2, d_lse_part2), in that order; P2 == 0 is the plain merge
-int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2,
-                       const float *d_lse_part2, int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb,
-                       int64_t o_sh, int64_t o_sl, float *d_lse, void *stream) {
-    INFLLM_REQUIRE(d_o_part && d_lse_part, "attn_merge: null pointer");
+// library-internal: the description of a merge over two sets of partials, P1 behind (d_o_part, d_lse_part) and P2
+// behind (d_o_part2, d_lse_part2), in that order; P2 == 0 is the plain merge
+int infllm_merge_job(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2, const float *d_lse_part2,
+                     int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
+                     MergeJob *job) {
+    INFLLM_REQUIRE(d_o_part && d_lse_part && job, "attn_merge: null pointer");
     INFLLM_REQUIRE(P1 >= 1 && P2 >= 0 && (P2 == 0 || (d_o_part2 && d_lse_part2)), "attn_merge: bad partial sets %d + %d", P1, P2);
-    const int32_t P = P1 + P2;
-    PartSets ps{P, 0, 0};
+    INFLLM_REQUIRE(B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes B=%d H=%d Lq=%d", B, H, Lq);
+    INFLLM_REQUIRE((o_sl % 8 | o_sh % 8 | o_sb % 8) == 0, "attn_merge: output strides must be multiples of 8");
+    PartSets ps{P1 + P2, 0, 0};
     if (P2 > 0) {
         const int64_t rows_ = (int64_t)B * H * Lq;
         ps.n_first = P1;
@@ -957,8 +901,19 @@ int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_
         ps.skip_l = (int64_t)(((intptr_t)d_lse_part2 - (intptr_t)d_lse_part) / (intptr_t)sizeof(float)) - (int64_t)P1 * rows_;
         ps.skip_o = (int64_t)(((intptr_t)d_o_part2 - (intptr_t)d_o_part) / 2) - (int64_t)P1 * rows_ * kD - ps.skip_l * kD;
     }
-    INFLLM_REQUIRE(P >= 1 && B > 0 && H > 0 && Lq > 0, "attn_merge: bad sizes P=%d B=%d H=%d Lq=%d", P, B, H, Lq);
-    INFLLM_REQUIRE((o_sl % 8 | o_sh % 8 | o_sb % 8) == 0, "attn_merge: output strides must be multiples of 8");
+    *job = MergeJob{(const _Float16 *)d_o_part, d_lse_part, P1 + P2, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse, ps};
+    return 0;
+}
+
+// library-internal: the merge over two sets of partials
+int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2,
+                       const float *d_lse_part2, int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb,
+                       int64_t o_sh, int64_t o_sl, float *d_lse, void *stream) {
+    MergeJob job;
+    const int jrc = infllm_merge_job(d_o_part, d_lse_part, P1, d_o_part2, d_lse_part2, P2, B, H, Lq, d_out, o_sb, o_sh, o_sl, d_lse, &job);
+    if (jrc) return jrc;
+    const int32_t P = P1 + P2;
+    const PartSets ps = job.ps;
     // few rows, many partials (decode-sized blocks): 16 lanes per row piece, each taking every 16th partial
     const bool wide = P > 8 && P <= 128 && (int64_t)B * H * Lq <= 2048;
     if (!d_out) {                                     // log-sum-exp only
@@ -979,7 +934,7 @@ int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_
                            (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse, ps);
     else
         hipLaunchKernelGGL(attn_merge_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                           (const _Float16 *)d_o_part, d_lse_part, P, B, H, Lq, (bf16_t *)d_out, o_sb, o_sh, o_sl, d_lse, ps);
+                           job);
     INFLLM_CHECK_LAUNCH("attn_merge");
     return 0;
 }

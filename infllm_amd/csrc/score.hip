@@ -11,6 +11,7 @@
 // (A operand, shared by the 4 waves, double buffered).  Exactly one lane writes each
 // (head, key) cell, so results are deterministic.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -20,9 +21,31 @@ constexpr int kQPad = kD + 8;              // LDS row of Q (bf16 elements): 272 
 // bounds the short launches that sit on the critical path between two blocks.  QS = queries per LDS stage: a short
 // launch is a chain of stages that each wait for one global load (there is next to no arithmetic to hide it behind),
 // so it takes stages of 128 queries and half as many of them.
-template <int KS, int QS>
-__global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a) {
+//
+// MERGE: the launch also carries the merge of the block's partial attention outputs, as extra workgroups behind the
+// scoring ones (blockIdx.y >= score_tiles; one thread per (row, 8 dims), merge_piece of common.h).  The two kinds of
+// work do not depend on each other - the scoring workgroups join the partial log-sum-exps themselves, by the merge's
+// own arithmetic - and the merge is a stream of loads that runs beside the matrix work: one launch instead of two
+// on the chain from one block's selection to the next.
+struct ScoreMerge {
+    MergeJob job;
+    int32_t score_tiles;               // blockIdx.y below this scores, from there on merges
+};
+struct NoScoreMerge {};
+
+template <int KS, int QS, bool MERGE = false>
+__global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a, std::conditional_t<MERGE, ScoreMerge, NoScoreMerge> sm) {
     constexpr int kWaveKeys = 32 * KS, kKeysPerWg = 4 * kWaveKeys, kQStage = QS;
+    int n_tiles = gridDim.y;
+    PartSets lps{a.n_parts, 0, 0};
+    if constexpr (MERGE) {
+        n_tiles = sm.score_tiles;
+        if ((int)blockIdx.y >= n_tiles) {
+            merge_piece(sm.job, ((int64_t)((int)blockIdx.y - n_tiles) * gridDim.x + blockIdx.x) * 256 + threadIdx.x);
+            return;
+        }
+        lps = sm.job.ps;
+    }
     extern __shared__ __attribute__((aligned(16))) char score_lds[];
     bf16_t(*Qs)[kQStage][kQPad] = (bf16_t(*)[kQStage][kQPad])score_lds;                               // [2][QS][kQPad]
     float(*Ls)[kQStage] = (float(*)[kQStage])(score_lds + 2 * kQStage * kQPad * sizeof(bf16_t));      // [2][QS]
@@ -37,7 +60,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     // Workgroups are dispatched x fastest: all heads of one key tile, then the next tile.  The two tiles at either end
     // of a masked key range see only part of the queries and finish early, so they go last: when the grid is a little
     // more than what the chip holds at once, the workgroups that start late are then the short ones.
-    const int n_tiles = gridDim.y, slot = blockIdx.y;
+    const int slot = blockIdx.y;
     int tile = slot;
     if (n_tiles >= 6 && a.mask != INFLLM_MASK_NONE)
         tile = slot < n_tiles - 4 ? slot + 2 : slot == n_tiles - 4 ? 1 : slot == n_tiles - 3 ? n_tiles - 2 : slot == n_tiles - 2 ? 0 : n_tiles - 1;
@@ -105,7 +128,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
                 for (int p0 = 0; p0 < a.n_parts; p0 += 8) {
                     float l8[8], m8 = -INFINITY;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) l8[i] = p0 + i < a.n_parts ? lse[(int64_t)(p0 + i) * rows + i0 + tid] : -INFINITY;
+                    for (int i = 0; i < 8; ++i) l8[i] = p0 + i < a.n_parts ? lse[lps.l(p0 + i, rows) + i0 + tid] : -INFINITY;
 #pragma unroll
                     for (int i = 0; i < 8; ++i) m8 = fmaxf(m8, l8[i]);
                     if (m8 == -INFINITY) continue;
@@ -261,7 +284,9 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
 
 }  // namespace
 
-extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
+namespace {
+
+int check_score_args(const infllm_score_args *a) {
     INFLLM_REQUIRE(a != nullptr, "local_score: null argument block");
     INFLLM_REQUIRE(a->d_q && a->d_k && a->d_lse && a->d_score, "local_score: null pointer");
     INFLLM_REQUIRE(a->B > 0 && a->H > 0 && a->Hkv > 0 && a->H % a->Hkv == 0 && a->Lq > 0,
@@ -273,29 +298,73 @@ extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
     INFLLM_REQUIRE(a->n_parts >= 0 && a->n_parts <= 1024, "local_score: %d partial log-sum-exps", a->n_parts);
     INFLLM_REQUIRE((a->q_sl % 8 | a->q_sh % 8 | a->q_sb % 8 | a->k_sl % 8 | a->k_sh % 8 | a->k_sb % 8) == 0,
                    "local_score: strides must be multiples of 8");
-    if (a->j_hi <= a->j_lo) return 0;
     INFLLM_REQUIRE(a->j_hi - a->j_lo <= (int64_t)65000 * 256, "local_score: key range of %lld rows exceeds one launch",
                    (long long)(a->j_hi - a->j_lo));
-    auto lds_bytes = [](int qs) { return (size_t)(2 * qs * kQPad * sizeof(bf16_t) + 2 * qs * sizeof(float)); };
+    return 0;
+}
+
+size_t score_lds_bytes(int qs) { return (size_t)(2 * qs * kQPad * sizeof(bf16_t) + 2 * qs * sizeof(float)); }
+
+int score_lds_setup() {
     static bool lds_set = false;                       // dynamic LDS above 64 KiB must be enabled once per kernel
     if (!lds_set) {
         hipError_t e = hipFuncSetAttribute((const void *)local_score_kernel<1, 128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)lds_bytes(128));
+                                           (int)score_lds_bytes(128));
         if (e == hipSuccess)
             e = hipFuncSetAttribute((const void *)local_score_kernel<2, 128>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)lds_bytes(128));
+                                    (int)score_lds_bytes(128));
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute((const void *)local_score_kernel<2, 128, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)score_lds_bytes(128));
         if (e != hipSuccess) return infllm_fail(-2, "local_score: %s", hipGetErrorString(e));
         lds_set = true;
     }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" int infllm_local_score(const infllm_score_args *a, void *stream) {
+    int rc = check_score_args(a);
+    if (rc) return rc;
+    if (a->j_hi <= a->j_lo) return 0;
+    rc = score_lds_setup();
+    if (rc) return rc;
     if (a->j_hi - a->j_lo > 1024) {
         const int64_t tiles = (a->j_hi - 1) / 64 - a->j_lo / 64 + 1;
-        hipLaunchKernelGGL((local_score_kernel<2, 128>), dim3(a->B * a->H, (unsigned)((tiles + 3) / 4)), dim3(256), lds_bytes(128),
-                           (hipStream_t)stream, *a);
+        hipLaunchKernelGGL((local_score_kernel<2, 128>), dim3(a->B * a->H, (unsigned)((tiles + 3) / 4)), dim3(256), score_lds_bytes(128),
+                           (hipStream_t)stream, *a, NoScoreMerge{});
     } else {
         const int64_t tiles = (a->j_hi - 1) / 32 - a->j_lo / 32 + 1;
-        hipLaunchKernelGGL((local_score_kernel<1, 128>), dim3(a->B * a->H, (unsigned)((tiles + 3) / 4)), dim3(256), lds_bytes(128),
-                           (hipStream_t)stream, *a);
+        hipLaunchKernelGGL((local_score_kernel<1, 128>), dim3(a->B * a->H, (unsigned)((tiles + 3) / 4)), dim3(256), score_lds_bytes(128),
+                           (hipStream_t)stream, *a, NoScoreMerge{});
     }
     INFLLM_CHECK_LAUNCH("local_score");
+    return 0;
+}
+
+// library-internal: the local score of a block and the merge of its partial attention outputs in one launch.  The
+// scores are taken against the joint log-sum-exp of the job's partials (a->d_lse and a->n_parts are set from the job);
+// returns 1, with nothing launched, where the one-launch form does not apply (short key ranges).
+int infllm_local_score_merged(const infllm_score_args *a, const MergeJob *job, void *stream) {
+    INFLLM_REQUIRE(a && job, "local_score_merged: null argument");
+    INFLLM_REQUIRE(job->out && job->B == a->B && job->H == a->H && job->Lq == a->Lq && job->P >= 1 && job->P <= 8,
+                   "local_score_merged: the merge does not belong to these queries");
+    infllm_score_args sc = *a;
+    sc.d_lse = job->lse_part;
+    sc.n_parts = job->P;
+    int rc = check_score_args(&sc);
+    if (rc) return rc;
+    if (sc.j_hi - sc.j_lo <= 1024) return 1;
+    rc = score_lds_setup();
+    if (rc) return rc;
+    const int64_t tiles = (sc.j_hi - 1) / 64 - sc.j_lo / 64 + 1;
+    const int score_tiles = (int)((tiles + 3) / 4);
+    const int64_t merge_wgs = ((int64_t)job->B * job->H * job->Lq * 16 + 255) / 256;
+    const int gx = sc.B * sc.H;
+    const int merge_slots = (int)((merge_wgs + gx - 1) / gx);
+    hipLaunchKernelGGL((local_score_kernel<2, 128, true>), dim3(gx, (unsigned)(score_tiles + merge_slots)), dim3(256), score_lds_bytes(128),
+                       (hipStream_t)stream, sc, ScoreMerge{*job, score_tiles});
+    INFLLM_CHECK_LAUNCH("local_score_merged");
     return 0;
 }

@@ -175,6 +175,10 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
 int infllm_inline_page_limit();
 int infllm_copy_units(const void *const *d_src, void *const *d_dst, int32_t n, int64_t nbytes, void *stream);
+int infllm_merge_job(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2, const float *d_lse_part2,
+                     int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
+                     MergeJob *job);
+int infllm_local_score_merged(const infllm_score_args *a, const MergeJob *job, void *stream);
 int infllm_attn_stage_blocked(const infllm_attn_args *a, int32_t exc, int64_t block_rows, void *stream);
 int infllm_attn_merge2(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2, const float *d_lse_part2,
                        int32_t P2, int32_t B, int32_t H, int32_t Lq, void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse,
@@ -1071,9 +1075,8 @@ int run_score_new_rank(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_s
 }
 
 // n_parts > 0: the stages' partial log-sum-exps are joined inside the launch (d_lse is not ready yet)
-int run_local_score(Layer *L, int n, int64_t b0, const Layer::QView &qv, int64_t j_lo, int64_t j_hi, int n_parts, void *stream) {
+infllm_score_args local_score_args(Layer *L, int n, int64_t b0, const Layer::QView &qv, int64_t j_lo, int64_t j_hi, int n_parts) {
     const infllm_layer_desc &d = L->d;
-    if (j_hi <= j_lo) return 0;
     infllm_score_args sc{};
     sc.d_q = qv.q_loc;
     sc.q_sl = kD; sc.q_sh = qv.q_sh; sc.q_sb = qv.q_sb;
@@ -1084,6 +1087,12 @@ int run_local_score(Layer *L, int n, int64_t b0, const Layer::QView &qv, int64_t
     sc.mask = INFLLM_MASK_WINDOW; sc.accumulate = 1; sc.offset = b0; sc.window = d.n_local;
     sc.d_lse = n_parts > 0 ? d.d_lse_part : d.d_lse; sc.n_parts = n_parts; sc.softmax_scale = d.softmax_scale;
     sc.d_score = d.d_ring_score; sc.score_sh = d.ring_cap; sc.score_sb = (int64_t)d.H * d.ring_cap; sc.score_cap = d.ring_cap;
+    return sc;
+}
+
+int run_local_score(Layer *L, int n, int64_t b0, const Layer::QView &qv, int64_t j_lo, int64_t j_hi, int n_parts, void *stream) {
+    if (j_hi <= j_lo) return 0;
+    const infllm_score_args sc = local_score_args(L, n, b0, qv, j_lo, j_hi, n_parts);
     return infllm_local_score(&sc, stream);
 }
 
@@ -1870,9 +1879,25 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     // While the fetches run ahead of the selection nothing waits for this block's selection at once, and the split
     // into an urgent and a bulk score launch only costs stream time: the merge and one score launch come first then.
     if (one_pass) {
-        rc = merge(a->d_out, d.d_lse);
+        // ... in ONE launch where the key range is long enough for the scoring kernel to have workgroups to spare
+        MergeJob job;
+        rc = batched ? infllm_merge_job(cur.o_loc, cur.lse_loc, sl, d.d_o_part, d.d_lse_part, parts - sl, d.B, d.H, a->n, a->d_out, a->o_sb,
+                                        a->o_sh, a->o_sl, d.d_lse, &job)
+                     : infllm_merge_job(d.d_o_part, d.d_lse_part, parts, nullptr, nullptr, 0, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh,
+                                        a->o_sl, d.d_lse, &job);
         if (rc) return rc;
-        rc = run_local_score(L, a->n, a->b0, cur, lo, b1, 0, stream);
+        static const bool apart = getenv("INFLLM_SCORE_MERGE_APART") && getenv("INFLLM_SCORE_MERGE_APART")[0] != '0';
+        rc = 1;
+        if (!apart && parts <= 8 && b1 > lo) {
+            const infllm_score_args sc = local_score_args(L, a->n, a->b0, cur, lo, b1, 0);
+            rc = infllm_local_score_merged(&sc, &job, stream);
+            if (rc < 0) return rc;
+        }
+        if (rc == 1) {
+            rc = merge(a->d_out, d.d_lse);
+            if (rc) return rc;
+            rc = run_local_score(L, a->n, a->b0, cur, lo, b1, 0, stream);
+        }
     } else
         rc = run_local_score(L, a->n, a->b0, cur, lo, urgent_hi, lse_early ? 0 : parts, stream);
     if (rc) return rc;

@@ -208,6 +208,29 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
     assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
 
 
+def test_merge_carried_by_the_score_launch_gives_the_bits_of_the_two_launches(monkeypatch):
+    """While fetches run ahead of the selection, a block's merge (output rows, joint log-sum-exp) rides in the launch of
+    its local score as extra workgroups; INFLLM_SCORE_MERGE_APART=1 keeps the two launches.  Same arithmetic either way:
+    outputs, selections and representatives bit for bit, at the small geometry with two batch rows and at the
+    reference geometry, block by block and with the call prepared in one go."""
+    from infllm_amd.attention import ContextManager
+    for call_tokens in (8192, 0):
+        monkeypatch.setattr(ContextManager, "call_tokens", call_tokens)
+        for args in ((2600, [1300, 1300], 8, 2, 1e4, 61, 2, dict(SMALL, max_cached_block=6)), (4096 + 8192, [4096, 8192], 32, 8, 1e6, 62, 1, REFERENCE)):
+            T, calls, H, Hkv, base, seed, B, kw = args
+            q, k, v = make_stream(T, H, Hkv, seed, B=B)
+            runs = []
+            for apart in ("1", "0"):
+                monkeypatch.setenv("INFLLM_SCORE_MERGE_APART", apart)
+                out, cm = run_gpu(q, k, v, calls, base, **kw)
+                issued, _ = cm.prefetch_stats()
+                runs.append((out, [b["order"] for b in cm.trace_blocks], cm.trace_repr_indices(), cm.stats, issued))
+            monkeypatch.delenv("INFLLM_SCORE_MERGE_APART")
+            (o0, s0, r0, st0, g0), (o1, s1, r1, st1, g1) = runs
+            assert torch.equal(o0, o1) and s0 == s1 and st0 == st1 and g1 > 0           # guesses ran: the one-launch form was used
+            assert r0.keys() == r1.keys() and all(torch.equal(r0[u], r1[u]) for u in r0)
+
+
 def test_units_still_in_a_staging_slot_are_copied_from_there(monkeypatch):
     """A missed unit whose rows are still in the staging slot they were gathered into when the unit was carved (the
     last four carving blocks) is copied from there on the main stream instead of being read back from pinned host
