@@ -286,9 +286,11 @@ void *infllm_host_device_pointer(void *h_pinned);
  *
  *   infllm_block_front   the block's prologue (RoPE + rings) and retrieval (mean query, unit
  *                        scores, top-k, asynchronous copy of the ids to pinned memory) unless
- *                        the previous block already did them ahead; the local stage; then,
- *                        when the caller passes the NEXT block's rows, that block's prologue
- *                        and the scores of the units that already exist;
+ *                        the previous block already did them ahead; when the caller passes the NEXT
+ *                        block's rows, that block's prologue, the scores of the units that already
+ *                        exist and their k best (the candidates of the next selection); then the local
+ *                        stage (inside a call prepared by infllm_call_front: no prologue, and the
+ *                        local stage of two blocks per launch);
  *   infllm_block_select  waits until the ids of this block are readable on the host, runs the cache
  *                        policy and issues the fetch of the missed units (copy stream); the same in
  *                        separate steps: infllm_layer_wait_topk, the caller's own policy,
@@ -299,15 +301,18 @@ void *infllm_host_device_pointer(void *h_pinned);
  *                        prepared - the scores of the new units, the next block's top-k and
  *                        the copy of its ids; only then the block's output rows, the rest of the
  *                        local score and the gather of the new units into a staging slot
- *                        (while fetches run ahead of the selection: merge and ONE local-score launch
- *                        before the representatives, since nothing waits for the selection at once);
+ *                        (while fetches run ahead of the selection: ONE local-score launch over the whole
+ *                        window before the representatives, with the merge riding in it as extra
+ *                        workgroups, since nothing waits for the selection at once);
  *   infllm_block_prefetch  (optional, further down) starts the NEXT block's fetch from its candidates.
  *
  * The fetch of missed units goes through 7 DMA engines (ROCr copies) for blocks of 64 queries or more, and the
  * main stream waits with hipStreamWaitValue32 for a sequence number the engines write behind the units; shorter
  * blocks, and processes without usable engines (or with INFLLM_NO_DMA_FETCH=1), use the zero-copy kernel
  * of infllm_fetch_units on the copy stream.  Either way the fetch is ordered behind the last reader of the slots
- * and behind the offload of units that are still on their way to the host.
+ * and behind the offload of units that are still on their way to the host.  A missed unit whose rows are still in
+ * the staging slot they were gathered into when it was carved is copied from there on the main stream instead.
+ * An eighth engine is kept for the carved units' way to the host.
  *
  * The chain from one block's ids to the next block's ids is therefore: fetch, global stage,
  * a small local-score launch (which joins the stages' log-sum-exps itself), representatives, a
