@@ -454,6 +454,7 @@ int infllm_layer_wait_mass(void *layer);
 int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_miss_row, const int32_t *h_miss_slot,
                        const int32_t *h_miss_unit, const void *const *h_miss_src, void *stream, void *copy_stream);
 int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream);
+
 int infllm_layer_flush(void *layer, void *copy_stream);
 
 /* ---- residency policy of the device unit cache, one object per batch row (context_manager.py:246-265 for the
@@ -504,7 +505,6 @@ typedef struct {
     int32_t *h_n_evicted, *h_n_miss;                  /* out, optional: [B] */
 } infllm_select_args;
 int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, void *copy_stream);
-
 /* The fetch ahead of the selection.  infllm_block_front ranks the units that exist before its block for the NEXT
  * block already (the selection proper, late in infllm_block_back, only weighs these candidates against the units
  * carved in between) and publishes them to the host.  Called after infllm_block_back, this runs the residency

@@ -426,36 +426,8 @@ class ContextManager:
             for u in range(B):
                 self.policy[u].add_scores(self._mass_units[u], masses[u][:len(self._mass_units[u])])
             self._mass_units = None
-        if self.select_in_steps:
-            n_sel, n_miss, selected = self._select_stepwise(preselected, N)
-        else:
-            if preselected is not None or N <= topk:
-                # chosen for the whole chunk (context_manager.py:381-382), or every unit there is
-                selected = preselected if preselected is not None else [list(range(N))] * B
-                n_sel = len(selected[0])
-                for u in range(B):
-                    self._sel_ids[u * n_sel:(u + 1) * n_sel] = selected[u]
-                sa.h_selected, sa.n_sel, sa.wait_topk = ctypes.addressof(self._sel_ids), n_sel, 0
-                n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
-            else:
-                n_sel = topk
-                sa.h_selected, sa.n_sel, sa.wait_topk = self.topk_idx_host.data_ptr(), n_sel, 1   # the one host wait of a block
-                n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
-                selected = None                                   # read back below, off the chain
-            if n_miss < 0:
-                check(n_miss, "infllm_block_select")
-            # the transfer has started; everything from here on overlaps it
-            if selected is None:
-                selected = self.topk_idx_host.tolist()
-            stats["evictions"] += sum(self._n_evicted[:B])
-            for u in range(B):
-                if self.policy[u].evicted_log is not None:
-                    self.policy[u].evicted_log.append(list(self._evicted[u * n_sel:u * n_sel + self._n_evicted[u]]))
-        stats["hits"] += B * n_sel - n_miss
-        stats["misses"] += n_miss
-        if self.cache_strategy == "lru":
-            self.load_count += 1
-        # ---- state machine after the block (context_manager.py:614-679)
+        # ---- state machine after the block (context_manager.py:614-679): it does not depend on the selection, so the
+        #      arguments of the block's second half are ready before the host waits for the ids
         cursor, init_len = self.cursor, self.init_len
         live = b1 - cursor
         take = 0
@@ -463,8 +435,8 @@ class ContextManager:
             take = min(self.n_init - init_len, live - self.n_local)
             live -= take
         c = max((live - self.n_local) // bs, 0)
-        ba.n, ba.n_sel, ba.b0 = n, n_sel, b0
-        ba.n_miss, ba.init_len, ba.cursor = n_miss, init_len, cursor
+        ba.n, ba.b0 = n, b0
+        ba.init_len, ba.cursor = init_len, cursor
         ba.d_out = out_ptr
         ba.init_take, ba.n_carve, ba.n_units = take, c, N
         idx_out = None
@@ -477,9 +449,44 @@ class ContextManager:
             if self.record_trace:
                 idx_out = torch.empty((B, c, self.unit_size, self.repr_topk), dtype=torch.int32, device=self.device)
             ba.d_repr_idx = idx_out.data_ptr() if idx_out is not None else None
-        rc = lib.infllm_block_back(layer, self._ba_ref, self._main_raw, self._copy_raw)
-        if rc:
-            check(rc, "infllm_block_back")
+        if self.select_in_steps:
+            n_sel, n_miss, selected = self._select_stepwise(preselected, N)
+            ba.n_sel, ba.n_miss = n_sel, n_miss
+            rc = lib.infllm_block_back(layer, self._ba_ref, self._main_raw, self._copy_raw)
+            if rc:
+                check(rc, "infllm_block_back")
+        else:
+            if preselected is not None or N <= topk:
+                # chosen for the whole chunk (context_manager.py:381-382), or every unit there is
+                selected = preselected if preselected is not None else [list(range(N))] * B
+                n_sel = len(selected[0])
+                for u in range(B):
+                    self._sel_ids[u * n_sel:(u + 1) * n_sel] = selected[u]
+                sa.h_selected, sa.n_sel, sa.wait_topk = ctypes.addressof(self._sel_ids), n_sel, 0
+            else:
+                n_sel = topk
+                sa.h_selected, sa.n_sel, sa.wait_topk = self.topk_idx_host.data_ptr(), n_sel, 1   # the one host wait of a block
+                selected = None                                   # read back below, off the chain
+            ba.n_sel = n_sel
+            # selection -> policy -> fetch, then the block's second half at once: next to nothing of the interpreter sits
+            # between the arrival of the ids and the launch of the global stage (one native call for both measured no faster)
+            n_miss = lib.infllm_block_select(layer, self._sa_ref, self._main_raw, self._copy_raw)
+            if n_miss < 0:
+                check(n_miss, "infllm_block_select")
+            ba.n_miss = n_miss
+            rc = lib.infllm_block_back(layer, self._ba_ref, self._main_raw, self._copy_raw)
+            if rc:
+                check(rc, "infllm_block_back")
+            if selected is None:
+                selected = self.topk_idx_host.tolist()
+            stats["evictions"] += sum(self._n_evicted[:B])
+            for u in range(B):
+                if self.policy[u].evicted_log is not None:
+                    self.policy[u].evicted_log.append(list(self._evicted[u * n_sel:u * n_sel + self._n_evicted[u]]))
+        stats["hits"] += B * n_sel - n_miss
+        stats["misses"] += n_miss
+        if self.cache_strategy == "lru":
+            self.load_count += 1
         if n_next and preselected is None and self.fetch_ahead and not self.select_in_steps and self.cache_strategy != "lru-s":
             sa.n_sel = topk
             rc = lib.infllm_block_prefetch(layer, self._sa_ref, self._main_raw, self._copy_raw)
