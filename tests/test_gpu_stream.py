@@ -45,9 +45,12 @@ def test_local_stage_groups_of_other_sizes_follow_the_oracle(monkeypatch):
 
 
 def test_both_stages_in_one_launch_follow_the_oracle(monkeypatch):
-    """INFLLM_FUSED_STAGES=1: the local and the global stage of every block as one launch over one list of tiles
-    (infllm_attn_stages_fused) - same acceptance against the oracle, at the small and at the reference geometry, and
+    """INFLLM_FUSED_STAGES=1 (with every block running its own local stage, call_tokens = 0): the local and the global
+    stage of every block as one launch over one list of tiles (infllm_attn_stages_fused) - same acceptance against the oracle, at the small and at the reference geometry, and
     the same discrete trajectory as the two-launch order."""
+    from infllm_amd.attention import ContextManager
+    monkeypatch.delenv("INFLLM_CALL_TOKENS", raising=False)
+    monkeypatch.setattr(ContextManager, "call_tokens", 0)          # the one-launch form belongs to blocks that run on their own
     monkeypatch.setenv("INFLLM_FUSED_STAGES", "1")
     cm, _, _ = compare(1500, [700, 1, 1, 798], H=8, Hkv=2, base=1e4, seed=41, B=2, **SMALL)
     assert cm.num_global_block > SMALL["topk"]
