@@ -85,6 +85,7 @@ def test_config2_stream_is_the_same_with_and_without_the_fetch_ahead(stream_128k
     q, k, v, qd, kd, vd = stream_128k
     T = 131072
     monkeypatch.delenv("INFLLM_NO_DMA_FETCH", raising=False)      # the engines where the process can use them ...
+    monkeypatch.delenv("INFLLM_NO_STAGING_COPY", raising=False)
     monkeypatch.setenv("INFLLM_FETCH_AHEAD_ALWAYS", "1")          # ... and guesses also where it cannot
 
     def run(ahead):
