@@ -114,7 +114,7 @@ extern "C" int infllm_fetch_units(const void *const *h_src, void *const *d_dst, 
 }
 
 // library-internal: the same for sources in device memory (units that are still in a carve staging slot): one launch
-// for all of them, shaped for HBM rather than for PCIe (16 KiB per workgroup, as many workgroups as there are pieces)
+// for all of them, shaped for HBM rather than for PCIe (as many workgroups as there are 4 KiB pieces)
 int infllm_copy_units(const void *const *d_src, void *const *d_dst, int32_t n, int64_t nbytes, void *stream) {
     INFLLM_REQUIRE(n >= 0 && nbytes > 0 && nbytes % 16 == 0, "copy_units: bad sizes n=%d nbytes=%lld", n, (long long)nbytes);
     INFLLM_REQUIRE(n == 0 || (d_src && d_dst), "copy_units: null list");
@@ -128,9 +128,9 @@ int infllm_copy_units(const void *const *d_src, void *const *d_dst, int32_t n, i
             list.src[i] = (const uint4 *)d_src[first + i];
             list.dst[i] = (uint4 *)d_dst[first + i];
         }
-        const int64_t piece = 256 * 4 * 16;
+        const int64_t piece = 256 * 1 * 16;             // 4 KiB per workgroup: one round trip each, 128 workgroups per 512 KiB unit
         const int64_t work = (int64_t)m * ((nbytes + piece - 1) / piece);
-        hipLaunchKernelGGL(unit_fetch_kernel<4>, dim3((unsigned)(work < 2048 ? work : 2048)), dim3(256), 0, (hipStream_t)stream, list, m, nbytes);
+        hipLaunchKernelGGL(unit_fetch_kernel<1>, dim3((unsigned)(work < 4096 ? work : 4096)), dim3(256), 0, (hipStream_t)stream, list, m, nbytes);
         INFLLM_CHECK_LAUNCH("copy_units");
     }
     return 0;
