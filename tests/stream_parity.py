@@ -134,9 +134,14 @@ class Follower:
         return gpu
 
 
-def assert_outputs_close(got, want, what=""):
+def assert_outputs_close(got, want, what="", relative_above_one=False):
+    """max-abs / mean-abs of the acceptance rule.  relative_above_one: the max-abs bound becomes MAX_ABS * |want| for
+    outputs beyond 1 in magnitude - for inputs that are not N(0,1) (activations of a decoder reach |v| = 7 and attention
+    rows that rest on one or two keys give outputs of 2..5, where neighbouring bf16 values are 0.016 or 0.031 apart, so
+    the rounding of the bf16 result alone can use up an absolute 2e-2)."""
     err = (got.float() - want.float()).abs()
-    assert float(err.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (what, float(err.max()), float(err.mean()))
+    worst = err / want.float().abs().clamp_min(1.0) if relative_above_one else err
+    assert float(worst.max()) <= MAX_ABS and float(err.mean()) <= MEAN_ABS, (what, float(worst.max()), float(err.max()), float(err.mean()))
 
 
 def assert_reps_match(cm, ora, first_unit=0):
@@ -152,10 +157,10 @@ def assert_reps_match(cm, ora, first_unit=0):
         assert bool(((got - want).abs() <= tol).all()), (u, float((got - want).abs().max()))
 
 
-def compare(T, calls, H, Hkv, base, seed, B=1, mixture=True, **kw):
-    """One stream through the GPU ContextManager and through the oracle following it; returns (cm, oracle, follower)."""
-    q, k, v = make_stream(T, H, Hkv, seed, B=B, mixture=mixture)
-    got, cm = run_gpu(q, k, v, calls, base, **kw)
+def follow(cm, got, q, k, v, calls, base, relative_above_one=False, **kw):
+    """The oracle over the CPU bf16 tensors q, k, v in the given calls, following the choices of `cm` (a manager that
+    recorded its trace over exactly those calls and returned `got`); asserts every rule above and returns
+    (oracle, follower)."""
     fol = Follower(cm, kw["topk"], kw.get("repr_topk", 1))
     ora = new_oracle(base, fol, **kw)
     outs, pos = [], 0
@@ -166,12 +171,21 @@ def compare(T, calls, H, Hkv, base, seed, B=1, mixture=True, **kw):
     want = torch.cat(outs, dim=2)
     assert not fol.violations, fol.violations[:5]
     assert [b["order"] for b in cm.trace_blocks] == [b["order"] for b in ora.block_trace]
-    assert cm.num_global_block == ora.n_units and cm.length == ora.length == T
-    assert_outputs_close(got, want)
+    assert cm.num_global_block == ora.n_units and cm.length == ora.length == pos
+    assert_outputs_close(got, want, relative_above_one=relative_above_one)
     if not kw.get("perhead", False):
         assert_reps_match(cm, ora)
         # the cache model saw the same ordered selections, so residency events must match too
         hits = sum(len(e["selected"]) - len(e["misses"]) for c in ora.cache for e in c.events)
         assert cm.stats["hits"] == hits
         assert cm.stats["evictions"] == sum(len(e["evicted"]) for c in ora.cache for e in c.events)
+    return ora, fol
+
+
+def compare(T, calls, H, Hkv, base, seed, B=1, mixture=True, **kw):
+    """One stream through the GPU ContextManager and through the oracle following it; returns (cm, oracle, follower)."""
+    q, k, v = make_stream(T, H, Hkv, seed, B=B, mixture=mixture)
+    got, cm = run_gpu(q, k, v, calls, base, **kw)
+    assert sum(calls) == T
+    ora, fol = follow(cm, got, q, k, v, calls, base, **kw)
     return cm, ora, fol
