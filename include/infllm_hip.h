@@ -175,7 +175,9 @@ int infllm_attn_stages_fused(const infllm_attn_args *local, const infllm_attn_ar
  * allocating library routine).  Limit: (local nsplit + global nsplit) * B * H * Lq <= INFLLM_NOALLOC_MAX_PART_ROWS
  * partial rows (260 bytes each: 16.25 MiB of device memory per GPU, held until the process ends); larger calls are
  * rejected with an error.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams,
- * two threads) race - serialise them, or use infllm_attn_fwd with workspaces of your own. */
+ * two threads) race - serialise them, or use infllm_attn_fwd with workspaces of your own.  The first call on a device
+ * also looks up that device's copy of the array and sets the kernels' attributes (safe from several threads at once,
+ * but not something a graph capture records): make one call per device before capturing. */
 #define INFLLM_NOALLOC_MAX_PART_ROWS 65536
 int infllm_attn_fwd_noalloc(const infllm_attn_args *local, const infllm_attn_args *global,
                             void *d_out, int64_t o_sb, int64_t o_sh, int64_t o_sl, float *d_lse, void *stream);
@@ -530,6 +532,13 @@ int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t *confirmed
  * of a transfer from pinned host memory; MemoryUnit.load, context_manager.py:76-91, for a unit whose gather into
  * staging is at most four carving blocks old).  INFLLM_NO_STAGING_COPY=1 (read by infllm_layer_create) turns it off. */
 int64_t infllm_layer_staged_units(void *layer);
+/* Which of two interchangeable paths the blocks of this layer took so far (for tests that compare the paths): counts[0]
+ * page tables of the global stage (get_global_hidden_and_mask, context_manager.py:386-451) carried in the stage's own
+ * launch, [1] written to device memory by the table kernel, [2] uploaded from the host; [3] merges of a block's partial
+ * outputs (torch_impl.py:15-36) carried by the block's local-score launch, [4] launched on their own in a block whose
+ * order of launches allowed the carried form.  INFLLM_PAGE_TABLE_KERNEL=1 and INFLLM_SCORE_MERGE_APART=1, read by
+ * infllm_layer_create, move blocks from [0] to [1] and from [3] to [4]. */
+int infllm_layer_path_counts(void *layer, int64_t *counts /* [5] */);
 /* Units moved from pinned host memory to the slab so far, whichever way (DMA engines or the fetch kernel): the misses
  * of the selections, the candidates a guess fetched that were not selected after all, and what a wrong guess's
  * repair brought back - the host-to-device traffic of MemoryUnit.load (context_manager.py:76-91) in units. */

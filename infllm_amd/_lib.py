@@ -159,6 +159,7 @@ SYMBOLS = {
     "infllm_layer_set_batch": (c_i32, [c_vp, C.POINTER(BatchDesc)]),
     "infllm_layer_staged_units": (c_i64, [c_vp]),
     "infllm_layer_fetched_units": (c_i64, [c_vp]),
+    "infllm_layer_path_counts": (c_i32, [c_vp, c_vp]),
     "infllm_call_front": (c_i32, [c_vp, C.POINTER(FrontArgs), c_vp]),
     "infllm_layer_wait_topk": (c_i32, [c_vp]),
     "infllm_layer_wait_mass": (c_i32, [c_vp]),

@@ -383,6 +383,13 @@ class ContextManager:
         """Missed units that were copied from a carve staging slot instead of coming from pinned host memory."""
         return int(self._lib.infllm_layer_staged_units(self._layer)) if self._layer else 0
 
+    def path_counts(self):
+        """Which interchangeable paths this layer's blocks took (infllm_layer_path_counts)."""
+        counts = (ctypes.c_int64 * 5)()
+        if self._layer:
+            check(self._lib.infllm_layer_path_counts(self._layer, counts), "infllm_layer_path_counts")
+        return dict(zip(("tables_inline", "tables_kernel", "tables_upload", "score_merged", "score_apart"), (int(c) for c in counts)))
+
     def fetched_units(self):
         """Units moved from pinned host memory to the device cache so far (wrongly guessed ones and repairs included)."""
         return int(self._lib.infllm_layer_fetched_units(self._layer)) if self._layer else 0
@@ -629,7 +636,9 @@ class ContextManager:
             if self._call_tokens and st == call_end:
                 # the next stretch of the call in one go: prologue, mean queries, first retrieval, local stage
                 call_end = min(st + self._call_tokens, input_length)
-                assert self.length + call_end - self.cursor <= self.ring_cap
+                if self.length + call_end - self.cursor > self.ring_cap:
+                    raise RuntimeError(f"a call of {call_end} tokens at {self.length} does not fit the rings "
+                                       f"({self.ring_cap} rows, carving cursor {self.cursor})")
                 if call_end - st > exc:          # a single block (a decode step) gains nothing from being prepared apart
                     fa.d_q, fa.d_k, fa.d_v = (self._q_ptr + st * self._q_step, self._k_ptr + st * self._k_step,
                                               self._v_ptr + st * self._v_step)

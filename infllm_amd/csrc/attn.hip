@@ -20,6 +20,7 @@
 
 #include "common.h"
 
+#include <atomic>
 #include <cstddef>
 #include <cstring>
 #include <type_traits>
@@ -839,8 +840,9 @@ extern "C" int infllm_attn_fwd(const infllm_attn_args *local, const infllm_attn_
 constexpr int64_t kStaticPartRows = INFLLM_NOALLOC_MAX_PART_ROWS;            // (split, batch row, head, query) rows
 static __device__ __align__(256) unsigned char attn_static_scratch[kStaticPartRows * (kD * 2 + 4)];
 constexpr int kMaxDevices = 64;
-static unsigned char *static_scratch_ptr[kMaxDevices];                       // per device: where ITS copy of the array lives
-static bool static_scratch_known[kMaxDevices];
+// per device: where ITS copy of the array lives.  Atomic: two threads making their first call on a device both look the
+// address up and store the same value
+static std::atomic<unsigned char *> static_scratch_ptr[kMaxDevices];
 
 extern "C" int infllm_attn_fwd_noalloc(const infllm_attn_args *local, const infllm_attn_args *global, void *d_out, int64_t o_sb,
                                        int64_t o_sh, int64_t o_sl, float *d_lse, void *stream) {
@@ -859,16 +861,17 @@ extern "C" int infllm_attn_fwd_noalloc(const infllm_attn_args *local, const infl
     int dev = -1;
     HIP_OK_ATTN(hipGetDevice(&dev), "attn_fwd_noalloc");
     INFLLM_REQUIRE(dev >= 0 && dev < kMaxDevices, "attn_fwd_noalloc: device %d", dev);
-    if (!static_scratch_known[dev]) {          // once per device, with that device current: the symbol's address THERE
+    unsigned char *scratch = static_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!scratch) {                            // once per device, with that device current: the symbol's address THERE
         void *p = nullptr;
         HIP_OK_ATTN(hipGetSymbolAddress(&p, HIP_SYMBOL(attn_static_scratch)), "attn_fwd_noalloc: hipGetSymbolAddress");
         INFLLM_REQUIRE(p != nullptr, "attn_fwd_noalloc: no address for the scratch array");
-        static_scratch_ptr[dev] = (unsigned char *)p;
-        static_scratch_known[dev] = true;
+        scratch = (unsigned char *)p;
+        static_scratch_ptr[dev].store(scratch, std::memory_order_release);
     }
     // o partials first (fp16 rows), the log-sum-exps behind all of them; the global stage's follow the local stage's
-    uint16_t *o_part = (uint16_t *)static_scratch_ptr[dev];
-    float *lse_part = (float *)(static_scratch_ptr[dev] + kStaticPartRows * kD * 2);
+    uint16_t *o_part = (uint16_t *)scratch;
+    float *lse_part = (float *)(scratch + kStaticPartRows * kD * 2);
     infllm_attn_args l{}, g{};
     if (local) {
         l = *local;

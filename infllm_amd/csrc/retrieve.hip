@@ -5,6 +5,9 @@
 // outputs are deterministic.
 #include "common.h"
 
+#include <algorithm>
+#include <atomic>
+
 namespace {
 
 __device__ __forceinline__ float wave_sum(float x) {
@@ -406,6 +409,199 @@ __global__ __launch_bounds__(256) void score_new_rank_kernel(const bf16_t *reps,
     publish(flag, flag_value);
 }
 
+
+// ---------------------------------------------------------------- unit scores and their top-k in ONE launch
+// (context_manager.py:159-163: logits = block_k @ mean query, topk(...).indices)
+// The scoring is unit_scores_rows_kernel's, term by term (a unit's score does not depend on which kernel computed it).
+// Every workgroup then takes a ticket; the one that draws the last ticket knows that all scores are written and
+// selects.  What crosses workgroups - the scores, the ticket - moves through agent-scope atomic accesses, which are
+// performed at the level of the memory hierarchy that all XCDs share, so no workgroup has to write its L2 back.
+//
+// The selection orders the units by the 64-bit composite (order_key(score) << 32 | ~id): all distinct, larger =
+// better score, equal scores by ascending id - torch.topk's order as the residency policy sees it.  The keys are
+// dealt to G >= k groups of threads; the smallest of the groups' maxima is a threshold that at least k composites
+// reach, and with scores that do not depend on the unit number in a regular way only about G ln G do.  Those few are
+// ranked against each other by counting.  When more than kSurvivorCap reach it (scores that fall with the unit
+// number, say) the exact k-th largest composite is built bit by bit instead - slower, never wrong.
+constexpr int kRetrThreads = 512;
+constexpr int kSurvivorCap = 1024;
+constexpr int kTicketSlots = 64;
+static __device__ unsigned int retrieval_tickets[kTicketSlots];       // zero at load; the last workgroup puts its slot back to zero
+
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int o) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, o, 64), hi = __shfl_xor((uint32_t)(v >> 32), o, 64);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// the selection by one workgroup of kRetrThreads threads over N <= NB * 16 * kRetrThreads scores; a thread keeps its
+// keys (units tid, tid + kRetrThreads, ...) in registers
+template <int NB>
+__device__ __forceinline__ void select_topk_block(const float *scores, int N, int k, int32_t *idx_out, int32_t *idx_out2) {
+    __shared__ uint64_t surv[kSurvivorCap + 8];
+    __shared__ __align__(16) uint32_t gmax[64];
+    __shared__ int wave_cnt[kRetrThreads / 64];
+    __shared__ int s_count;
+    constexpr int R = NB * 16;                                   // 16 loads in flight per thread and round trip
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t key[R];
+    uint32_t best = 0;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        float sc[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int n = tid + (b * 16 + j) * kRetrThreads;
+            // an agent-scope load: it is served from where the other workgroups' agent-scope stores went
+            sc[j] = n < N ? __hip_atomic_load(scores + n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int n = tid + (b * 16 + j) * kRetrThreads;
+            key[b * 16 + j] = n < N ? order_key(sc[j]) : 0u;
+            best = key[b * 16 + j] > best ? key[b * 16 + j] : best;
+        }
+    }
+    auto composite = [&](int j) { return ((uint64_t)key[j] << 32) | (uint32_t)(0xffffffffu - (uint32_t)(tid + j * kRetrThreads)); };
+    if (tid == 0) s_count = 0;
+    if (tid < 64) gmax[tid] = 0xffffffffu;
+    __syncthreads();
+    // groups of 32, 16 or 8 lanes: 16, 32 or 64 groups; the threshold is on the score's key alone (units that tie with
+    // it all pass, and are told apart by the composites afterwards)
+    const int width = k <= 16 ? 32 : k <= 32 ? 16 : 8;
+    for (int o = 1; o < width; o <<= 1) {
+        const uint32_t other = __shfl_xor(best, o, 64);
+        best = other > best ? other : best;
+    }
+    if ((lane & (width - 1)) == 0) gmax[tid / width] = best;
+    __syncthreads();
+    uint32_t tau = 0xffffffffu;
+#pragma unroll
+    for (int g = 0; g < 64; g += 4) {
+        const u32x4 m = *(const u32x4 *)(gmax + g);
+        tau = min(min(tau, m[0]), min(m[1], min(m[2], m[3])));
+    }
+    auto collect = [&](uint64_t thr) {                           // composites >= thr into surv[]; s_count = how many there are
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            const uint64_t c = composite(j);
+            if (tid + j * kRetrThreads < N && c >= thr) {
+                const int pos = atomicAdd(&s_count, 1);
+                if (pos < kSurvivorCap) surv[pos] = c;
+            }
+        }
+        __syncthreads();
+    };
+    collect((uint64_t)tau << 32);
+    if (s_count > kSurvivorCap) {
+        // exact: the largest t with at least k composites >= t, one bit at a time from the top
+        uint64_t t = 0;
+        for (int bit = 63; bit >= 0; --bit) {
+            const uint64_t trial = t | (1ull << bit);
+            int c = 0;
+#pragma unroll
+            for (int j = 0; j < R; ++j) c += (tid + j * kRetrThreads < N && composite(j) >= trial) ? 1 : 0;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, 64);
+            __syncthreads();                                     // wave_cnt of the previous round fully read
+            if (lane == 0) wave_cnt[wave] = c;
+            __syncthreads();
+            int tot = 0;
+#pragma unroll
+            for (int w = 0; w < kRetrThreads / 64; ++w) tot += wave_cnt[w];
+            if (tot >= k) t = trial;
+        }
+        __syncthreads();
+        if (tid == 0) s_count = 0;
+        __syncthreads();
+        collect(t);                                              // exactly k of them now
+    }
+    const int S = s_count;
+    const int S8 = (S + 7) & ~7;                                 // padded with composites below every real one: the
+    for (int i = S + tid; i < S8; i += kRetrThreads) surv[i] = 0;  // ranking loop then reads eight entries per round trip
+    __syncthreads();
+    for (int i = tid; i < S; i += kRetrThreads) {
+        const uint64_t mine = surv[i];
+        int rank = 0;
+        for (int j = 0; j < S8; j += 8) {
+            uint64_t o[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = surv[j + e];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) rank += o[e] > mine ? 1 : 0;
+        }
+        if (rank < k) put_id(idx_out, idx_out2, rank, (int32_t)(0xffffffffu - (uint32_t)mine));
+    }
+}
+
+template <int CPL, int ROWS>
+__global__ __launch_bounds__(kRetrThreads) void retrieve_fused_kernel(const bf16_t *reps, int64_t rep_stride, int N, const float *qbar,
+                                                                      float *scores, int k, int32_t *idx_out, int32_t *idx_out2,
+                                                                      int32_t *flag, int32_t flag_value, int ticket_slot) {
+    extern __shared__ float qs[];                                // the mean query
+    __shared__ int is_last;
+    constexpr int C = CPL * 512;
+    const int lane = threadIdx.x & 63;
+    const int waves_per_wg = kRetrThreads / 64;
+    const int n_waves = gridDim.x * waves_per_wg;
+    int n = blockIdx.x * waves_per_wg + (threadIdx.x >> 6);     // rows n, n + n_waves, ... belong to this wave
+    u32x4 w[ROWS][CPL];
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r)
+        if (n + r * n_waves < N) {
+            const bf16_t *row = reps + (int64_t)(n + r * n_waves) * rep_stride + lane * 8;
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) w[r][j] = __builtin_nontemporal_load((const u32x4 *)(row + j * 512));
+        }
+    for (int e = threadIdx.x * 4; e < C; e += kRetrThreads * 4) *(f32x4 *)(qs + e) = *(const f32x4 *)(qbar + e);
+    __syncthreads();
+    float q[CPL][8];
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) {
+        const f32x4 lo = *(const f32x4 *)(qs + j * 512 + lane * 8), hi = *(const f32x4 *)(qs + j * 512 + lane * 8 + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) q[j][i] = lo[i], q[j][4 + i] = hi[i];
+    }
+    while (n < N) {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const int cur = n + r * n_waves;
+            if (cur >= N) break;
+            float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc0 += bf16_bits_to_f32(w[r][j][i] & 0xffffu) * q[j][2 * i];
+                    acc1 += bf16_bits_to_f32(w[r][j][i] >> 16) * q[j][2 * i + 1];
+                }
+            }
+            const int nxt = cur + ROWS * n_waves;
+            if (nxt < N) {
+                const bf16_t *row = reps + (int64_t)nxt * rep_stride + lane * 8;
+#pragma unroll
+                for (int j = 0; j < CPL; ++j) w[r][j] = __builtin_nontemporal_load((const u32x4 *)(row + j * 512));
+            }
+            const float acc = wave_sum(acc0 + acc1);
+            if (lane == 0) __hip_atomic_store(scores + cur, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        n += ROWS * n_waves;
+    }
+    // every wave's score stores have been performed before the workgroup takes its ticket
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned int drawn = __hip_atomic_fetch_add(&retrieval_tickets[ticket_slot], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = drawn == gridDim.x - 1;
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (threadIdx.x == 0) __hip_atomic_store(&retrieval_tickets[ticket_slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (N <= 16 * kRetrThreads) select_topk_block<1>(scores, N, k, idx_out, idx_out2);
+    else select_topk_block<2>(scores, N, k, idx_out, idx_out2);
+    publish(flag, flag_value);
+}
+
 // ---------------------------------------------------------------- representative keys
 constexpr int kMaxUnit = 2048;             // largest supported unit (block_size)
 
@@ -585,9 +781,51 @@ extern "C" int infllm_score_new_topk(const void *d_reps, int64_t rep_stride, int
     return rc == 1 ? infllm_fail(-1, "score_new_topk: rows of %d elements (supported: 512, 1024, 2048, 4096)", C) : rc;
 }
 
+
+// library-internal: unit scores of all N units and the k best of them in ONE launch (retrieve_fused_kernel), the ids
+// leaving as infllm_topk_publish_pair leaves them.  Returns 1, with nothing launched, where that kernel does not apply
+// (row lengths other than 512 * {1, 2, 4, 8}, more than 16384 units, k > 64): the caller then launches the two steps.
+int infllm_retrieve_fused(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbar, int32_t k, float *d_scores,
+                          int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag, int32_t flag_value, void *stream) {
+    INFLLM_REQUIRE(d_reps && d_qbar && d_scores && d_idx, "retrieve: null pointer");
+    INFLLM_REQUIRE(N > 0 && k > 0 && k <= N, "retrieve: k=%d with N=%d", k, N);
+    INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "retrieve: row stride %lld", (long long)rep_stride);
+    if (N > 16384 || k > 64 || C % 512 != 0) return 1;
+    const int cpl = C / 512;
+    if (cpl != 1 && cpl != 2 && cpl != 4 && cpl != 8) return 1;
+    static std::atomic<unsigned int> next_slot{0};
+    const int slot = (int)(next_slot.fetch_add(1, std::memory_order_relaxed) % kTicketSlots);
+    constexpr int waves_per_wg = kRetrThreads / 64;
+    const bool deep = N >= 4096;
+    const int per_wg = waves_per_wg * (deep ? 2 : 1);
+    int wgs = (N + per_wg - 1) / per_wg;
+    if (wgs > 256) wgs = 256;
+    const size_t lds = (size_t)C * sizeof(float);
+    const bf16_t *reps = (const bf16_t *)d_reps;
+    const hipStream_t st = (hipStream_t)stream;
+#define FUSED_CASE(c)                                                                                                              \
+    case c: {                                                                                                                      \
+        auto kern = deep ? retrieve_fused_kernel<c, 2> : retrieve_fused_kernel<c, 1>;                                              \
+        hipLaunchKernelGGL(kern, dim3(wgs), dim3(kRetrThreads), lds, st, reps, rep_stride, N, d_qbar, d_scores, k, d_idx, d_idx2,   \
+                           d_flag, flag_value, slot);                                                                              \
+        break;                                                                                                                     \
+    }
+    switch (cpl) {
+        FUSED_CASE(1) FUSED_CASE(2) FUSED_CASE(4) FUSED_CASE(8)
+    }
+#undef FUSED_CASE
+    INFLLM_CHECK_LAUNCH("retrieve");
+    return 0;
+}
+
 extern "C" int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbar,
                                  int32_t k, float *d_scores, int32_t *d_idx, void *stream) {
     INFLLM_REQUIRE(N > 0 && k >= 0 && k <= N, "score_topk: k=%d with N=%d", k, N);
+    if (k > 0) {
+        INFLLM_REQUIRE(d_idx, "score_topk: null index pointer");
+        const int frc = infllm_retrieve_fused(d_reps, rep_stride, N, C, d_qbar, k, d_scores, d_idx, nullptr, nullptr, 0, stream);
+        if (frc != 1) return frc;
+    }
     int rc = infllm_unit_scores(d_reps, rep_stride, 0, N, C, d_qbar, d_scores, stream);
     if (rc == 0 && k > 0) rc = infllm_topk(d_scores, N, k, d_idx, stream);
     return rc;

@@ -105,6 +105,11 @@ struct Layer {
     hipEvent_t stage_copied = nullptr;                 // behind the last such copy
     std::vector<int64_t> stage_copy_dst;               // slots (row * max_cached + slot) such copies may still be on their way to
     bool stage_copy_ok = true;                         // INFLLM_NO_STAGING_COPY=1: every missed unit comes from the host
+    bool page_table_kernel = false;                    // INFLLM_PAGE_TABLE_KERNEL=1: short page tables are written by a kernel too
+    bool score_merge_apart = false;                    // INFLLM_SCORE_MERGE_APART=1: the merge never rides in the score launch
+    // which of those paths the blocks took (infllm_layer_path_counts): page tables carried by the launch / written by
+    // the kernel / uploaded; merges carried by the score launch / launched on their own in a block that could carry one
+    int64_t n_tables_inline = 0, n_tables_kernel = 0, n_tables_upload = 0, n_score_merged = 0, n_score_apart = 0;
     int64_t staged_units = 0;                          // missed units served from a staging slot so far
     int64_t fetched_units = 0;                         // units moved from pinned host memory so far (guessed ones and repairs included)
     hipEvent_t mass_done = nullptr;
@@ -119,6 +124,12 @@ struct Layer {
     bool global_unmarked = false;         // the last global stage ran without recording global_done (see block_back)
     hipEvent_t idle_main = nullptr, idle_copy = nullptr;      // recorded by layer_flush: this layer's work up to there
     bool idle_recorded = false;
+    bool unflushed = false;               // work was enqueued since the last layer_flush (a call that ended half way)
+    hipStream_t last_copy_stream = nullptr;
+    // where the carving stood after the last block (rows from there on are still needed): infllm_call_front checks
+    // the rings' room against it
+    bool cursor_known = false;
+    int64_t cursor = 0;
     bool topk_pending = false;
     int slot = 0;                         // workspace slot written last
     // Where a block's rotated queries, mean query and (when its local stage already ran) local partials are: a slot of
@@ -173,6 +184,8 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_retrieve_fused(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbar, int32_t k, float *d_scores,
+                          int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag, int32_t flag_value, void *stream);
 int infllm_inline_page_limit();
 int infllm_copy_units(const void *const *d_src, void *const *d_dst, int32_t n, int64_t nbytes, void *stream);
 int infllm_merge_job(const uint16_t *d_o_part, const float *d_lse_part, int32_t P1, const uint16_t *d_o_part2, const float *d_lse_part2,
@@ -527,21 +540,16 @@ void efetch_setup(Layer *L) {
     // kernels (with a ninth or a tenth the block's own kernels ran 10-40 % longer, measured).  One of them is kept for
     // the carved units' way to the host: while that copy (2 MiB per block) shared an engine with the fetch, the units
     // queued behind it on that engine landed last and the whole fetch waited for them - 47.6 ms per 128K stream
-    // against 44.2 with the engines apart.  INFLLM_SHARED_ENGINES=1 keeps the old assignment (the runtime picks the
-    // offload's engine, the fetch takes all eight), INFLLM_FETCH_ENGINES=n limits the fetch to n engines.
-    const char *ne = getenv("INFLLM_FETCH_ENGINES");
-    const char *sh = getenv("INFLLM_SHARED_ENGINES");
-    const bool shared = sh && sh[0] && sh[0] != '0';
-    const int want_engines = ne && atoi(ne) > 0 ? atoi(ne) : kEfetchEngines;
+    // against 44.2 with the engines apart.
     uint32_t d2h = 0;
-    if (shared || hsa_amd_memory_copy_engine_status(L->dma_cpu, L->dma_gpu, &d2h) != HSA_STATUS_SUCCESS) d2h = 0;
+    if (hsa_amd_memory_copy_engine_status(L->dma_cpu, L->dma_gpu, &d2h) != HSA_STATUS_SUCCESS) d2h = 0;
     std::vector<uint32_t> low;
     for (int b = 0; b < 8; ++b)
         if (mask & (1u << b)) low.push_back(1u << b);
     L->off_engine = 0;
     if (low.size() >= 4 && (d2h & low[1])) L->off_engine = low[1];      // the second one: the first is the fetch's flag engine
     for (uint32_t e : low)
-        if (e != L->off_engine && (int)L->efetch_engines.size() < want_engines) L->efetch_engines.push_back(e);
+        if (e != L->off_engine && (int)L->efetch_engines.size() < kEfetchEngines) L->efetch_engines.push_back(e);
     if (L->efetch_engines.size() < 2) return;
     L->efetch_dev = dev;
     if (!(L->d_efetch_flag = flag_take(dev)) || hipHostMalloc((void **)&L->h_efetch_val, kEfetchVals * sizeof(uint32_t)) != hipSuccess ||
@@ -642,6 +650,8 @@ int do_fetch(Layer *L, int n_miss, const int32_t *rows, const int32_t *slots, co
              hipStream_t st, hipStream_t cs, bool ahead = false) {
     const infllm_layer_desc &d = L->d;
     const bool side = cs != st;
+    L->unflushed = true;
+    L->last_copy_stream = cs;
     const int64_t slot_elems = 2 * (int64_t)d.Hkv * d.block_size * kD;
     // A unit carved a few blocks ago is still in the staging slot it was gathered into (the launch that filled it is
     // ahead of this point in the main stream): it is copied from there.  A unit that makes a selection right after it
@@ -856,6 +866,10 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         L->local_in_front = !(fs && fs[0] && fs[0] != '0');
         const char *ns = getenv("INFLLM_NO_STAGING_COPY");
         L->stage_copy_ok = !(ns && ns[0] && ns[0] != '0');
+        const char *pk = getenv("INFLLM_PAGE_TABLE_KERNEL");
+        L->page_table_kernel = pk && pk[0] && pk[0] != '0';
+        const char *ma = getenv("INFLLM_SCORE_MERGE_APART");
+        L->score_merge_apart = ma && ma[0] && ma[0] != '0';
     }
     if (hipHostMalloc((void **)&L->h_cand, ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
         (void)hipGetLastError();
@@ -870,7 +884,14 @@ extern "C" int infllm_layer_destroy(void *layer) {
     Layer *L = (Layer *)layer;
     // The caller frees the layer's buffers next: wait for the work that uses them - what layer_flush marked on the two
     // streams (every append ends with it), not for the device, which may be busy with other layers.
-    if (L->idle_recorded) {
+    // A layer destroyed between a block's calls and the flush (an append() that raised, a C caller that skipped the
+    // flush) has work in flight that no such mark covers: then the two streams themselves are waited for.
+    if (L->unflushed) {
+        if (L->main_stream_known) (void)hipStreamSynchronize(L->main_stream);
+        if (L->last_copy_stream) (void)hipStreamSynchronize(L->last_copy_stream);
+        if (L->efetch_ok) (void)efetch_wait_all(L, "layer_destroy");
+        (void)hipGetLastError();
+    } else if (L->idle_recorded) {
         (void)hipEventSynchronize(L->idle_main);
         (void)hipEventSynchronize(L->idle_copy);
     }
@@ -1029,6 +1050,38 @@ int run_topk(Layer *L, const float *scores, int64_t scores_sb, int n_units, void
     return 0;
 }
 
+// scores of all units and the selection among them (run_unit_scores + run_topk), one launch per batch row where the
+// geometry has the kernel for it
+int run_retrieval(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_su, float *scores, int64_t scores_sb, int n_units,
+                  const float *qbar, void *stream) {
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream;
+    const int C = d.H * kD;
+    const bool poll = d.d_topk_flag && d.h_topk_flag && !d.h_topk_idx;
+    if (poll) ++L->topk_seq;
+    for (int u = 0; u < d.B; ++u) {
+        const bool last = poll && u == d.B - 1;
+        const bf16_t *reps_u = (const bf16_t *)reps + (int64_t)u * rep_sb;
+        float *scores_u = scores + (int64_t)u * scores_sb;
+        int rc = infllm_retrieve_fused(reps_u, rep_su, n_units, C, qbar + (int64_t)u * C, d.topk, scores_u, d.d_topk_idx + (int64_t)u * d.topk,
+                                       nullptr, last ? d.d_topk_flag : nullptr, L->topk_seq, stream);
+        if (rc < 0) return rc;
+        if (rc == 1) {
+            rc = infllm_unit_scores(reps_u, rep_su, 0, n_units, C, qbar + (int64_t)u * C, scores_u, stream);
+            if (rc) return rc;
+            rc = infllm_topk_publish(scores_u, n_units, d.topk, d.d_topk_idx + (int64_t)u * d.topk, last ? d.d_topk_flag : nullptr,
+                                     L->topk_seq, stream);
+            if (rc) return rc;
+        }
+    }
+    if (d.h_topk_idx)      // NULL: d_topk_idx is itself host-visible pinned memory, the kernel wrote there
+        HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
+    if (!poll) HIP_OK(hipEventRecord(L->topk_done, st), "event");
+    L->topk_stream = st;
+    L->topk_pending = true;
+    return 0;
+}
+
 // the selection for the next block from the candidates chosen ahead and the n_new units carved since
 int run_topk_merge(Layer *L, const float *scores, int64_t scores_sb, int n_old, int n_new, void *stream) {
     const infllm_layer_desc &d = L->d;
@@ -1145,8 +1198,14 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
     INFLLM_REQUIRE(a->n <= d.ring_cap, "call_front: %d tokens do not fit a ring of %lld rows", a->n, (long long)d.ring_cap);
     INFLLM_REQUIRE(a->n_units >= 0 && a->b0 >= 0, "call_front: negative state");
     INFLLM_REQUIRE(a->d_q && a->d_k && a->d_v, "call_front: null q / k / v");
+    // the rows from the carving cursor on are still needed (remainder, window, score track): writing a->n rows at b0
+    // must not reach around the ring to them
+    INFLLM_REQUIRE(!L->cursor_known || a->b0 - L->cursor + a->n <= d.ring_cap,
+                   "call_front: %d tokens at %lld would overwrite ring rows from %lld on (ring of %lld rows)", a->n, (long long)a->b0,
+                   (long long)L->cursor, (long long)d.ring_cap);
     L->main_stream = st;
     L->main_stream_known = true;
+    L->unflushed = true;
     L->batch_live = false;
     L->prepared = false;
     const int C = d.H * kD;
@@ -1164,9 +1223,7 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
         L->slot ^= 1;
         rc = run_ingest(L, a, a->d_q, a->d_k, a->d_v, a->n < d.exc ? a->n : d.exc, a->b0, L->slot, true, stream);
         if (rc) return rc;
-        rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
-        if (rc) return rc;
-        rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, stream);
+        rc = run_retrieval(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, L->fresh.qbar, stream);
         if (rc) return rc;
     }
 
@@ -1227,6 +1284,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     int rc;
     L->main_stream = st;
     L->main_stream_known = true;
+    L->unflushed = true;
 
     // ---- this block's prologue and retrieval, unless the previous block prepared them
     const bool batched = block_in_batch(L, a->b0, a->n);       // its prologue and local stage ran in infllm_call_front
@@ -1243,9 +1301,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
         if (!retrieved) L->topk_pending = false;
         if (retrieve && !retrieved) {
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
-            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
-            if (rc) return rc;
-            rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, a->n_units, stream);
+            rc = run_retrieval(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, L->fresh.qbar, stream);
             if (rc) return rc;
         }
     }
@@ -1272,20 +1328,34 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
         }
         if (a->n_units > 0 && !(a->flags & INFLLM_NO_RETRIEVAL)) {
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
-            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, 0, a->n_units, L->fresh.qbar, stream);
-            if (rc) return rc;
-            // their k best now, while the fetch is in flight: the selection after the block then only has to weigh these
-            // against the few units carved in between, instead of running over every unit on the chain
+            // The scores of the existing units and their k best now, while the fetch is in flight: the selection after the
+            // block then only has to weigh these against the few units carved in between, instead of running over every
+            // unit on the chain.  One launch per batch row where the geometry has the kernel for it, else two.
             L->cand_units = -1;
-            if (L->d_cand && a->n_units > d.topk) {
-                // the host gets a copy, with a sequence number behind the last row's: it may fetch them ahead
-                if (L->h_cand) ++L->cand_seq;
-                for (int u = 0; u < d.B; ++u) {
-                    rc = infllm_topk_publish_pair(a->d_unit_scores + (int64_t)u * a->unit_scores_sb, a->n_units, d.topk,
-                                                  L->d_cand + (int64_t)u * d.topk, L->h_cand ? L->h_cand + (int64_t)u * d.topk : nullptr,
-                                                  L->h_cand && u == d.B - 1 ? L->h_cand + (int64_t)d.B * d.topk : nullptr, L->cand_seq, stream);
+            const bool want_cand = L->d_cand && a->n_units > d.topk;
+            if (want_cand && L->h_cand) ++L->cand_seq;       // the host gets a copy, with a sequence number behind the last row's: it may fetch them ahead
+            const int C = d.H * kD;
+            for (int u = 0; u < d.B; ++u) {
+                const bf16_t *reps_u = (const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb;
+                float *scores_u = a->d_unit_scores + (int64_t)u * a->unit_scores_sb;
+                const float *qbar_u = L->fresh.qbar + (int64_t)u * C;
+                int32_t *cand_host = L->h_cand ? L->h_cand + (int64_t)u * d.topk : nullptr;
+                int32_t *cand_flag = L->h_cand && u == d.B - 1 ? L->h_cand + (int64_t)d.B * d.topk : nullptr;
+                rc = want_cand ? infllm_retrieve_fused(reps_u, a->rep_su, a->n_units, C, qbar_u, d.topk, scores_u, L->d_cand + (int64_t)u * d.topk,
+                                                       cand_host, cand_flag, L->cand_seq, stream)
+                               : 1;
+                if (rc < 0) return rc;
+                if (rc == 1) {
+                    rc = infllm_unit_scores(reps_u, a->rep_su, 0, a->n_units, C, qbar_u, scores_u, stream);
                     if (rc) return rc;
+                    if (want_cand) {
+                        rc = infllm_topk_publish_pair(scores_u, a->n_units, d.topk, L->d_cand + (int64_t)u * d.topk, cand_host, cand_flag,
+                                                      L->cand_seq, stream);
+                        if (rc) return rc;
+                    }
                 }
+            }
+            if (want_cand) {
                 L->cand_units = a->n_units;
                 L->cand_for_units = L->h_cand ? a->n_units : -1;
             }
@@ -1484,6 +1554,17 @@ extern "C" int64_t infllm_layer_staged_units(void *layer) {
     return ((Layer *)layer)->staged_units;
 }
 
+extern "C" int infllm_layer_path_counts(void *layer, int64_t *counts) {
+    INFLLM_REQUIRE(layer && counts, "layer_path_counts: null argument");
+    const Layer *L = (const Layer *)layer;
+    counts[0] = L->n_tables_inline;
+    counts[1] = L->n_tables_kernel;
+    counts[2] = L->n_tables_upload;
+    counts[3] = L->n_score_merged;
+    counts[4] = L->n_score_apart;
+    return 0;
+}
+
 extern "C" int64_t infllm_layer_fetched_units(void *layer) {
     if (!layer) return infllm_fail(-1, "layer_fetched_units: null layer");
     return ((Layer *)layer)->fetched_units;
@@ -1634,6 +1715,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     hipStream_t st = (hipStream_t)stream, cs = (hipStream_t)copy_stream;
     const bool side = cs != st;
     const int bs = d.block_size;
+    L->unflushed = true;
+    L->last_copy_stream = cs;
     INFLLM_REQUIRE(a->n >= 1 && a->n <= d.exc && a->n_sel >= 0 && a->n_sel <= d.topk, "block_back: bad block sizes");
     INFLLM_REQUIRE(a->n_miss >= 0 && a->n_miss <= d.B * a->n_sel && a->init_len >= 0 && a->init_len <= d.init_cap,
                    "block_back: bad miss / init counts");
@@ -1664,8 +1747,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     // kernel from the slot list, or uploaded.  INFLLM_PAGE_TABLE_KERNEL=1 keeps the kernel for short tables too.
     infllm_page inline_pages[64];
     bool pages_inline = false;
-    static const bool inline_allowed = [] { const char *e = getenv("INFLLM_PAGE_TABLE_KERNEL"); return !(e && e[0] && e[0] != '0'); }();
-    if (inline_allowed) {
+    if (!L->page_table_kernel) {
         const int room = infllm_inline_page_limit() < 64 ? infllm_inline_page_limit() : 64;
         int n0 = host_pages(d, a, 0, overflow_end, inline_pages, room);
         if (n0 > 0 && (int64_t)d.B * n0 <= room) {
@@ -1679,6 +1761,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         }
     }
     if (pages_inline) {
+        ++L->n_tables_inline;
     } else if (d.B * a->n_sel <= kPageJobSlots) {
         PageJob j{};
         j.B = d.B; j.Hkv = d.Hkv; j.bs = bs; j.max_cached = d.max_cached; j.n_sel = a->n_sel; j.init_len = a->init_len;
@@ -1704,6 +1787,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         if (n_pages > 0) {
             hipLaunchKernelGGL(build_pages_kernel, dim3((n_pages + 63) / 64, d.B), dim3(64), 0, st, j, d.d_pages);
             INFLLM_CHECK_LAUNCH("build_pages");
+            ++L->n_tables_kernel;
         }
     } else
     {
@@ -1751,6 +1835,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
                    "block_back: page upload");
             HIP_OK(hipEventRecord(L->page_evt[slot], st), "block_back: event");
             L->page_busy[slot] = 1;
+            ++L->n_tables_upload;
         }
     }
 
@@ -1875,6 +1960,8 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     int carved_slot = 0;
     L->main_stream = st;
     const int64_t new_cursor = a->cursor + a->init_take + (int64_t)a->n_carve * bs;
+    L->cursor = new_cursor;
+    L->cursor_known = true;
     const int64_t urgent_hi = new_cursor < b1 ? new_cursor : b1;
     // While the fetches run ahead of the selection nothing waits for this block's selection at once, and the split
     // into an urgent and a bulk score launch only costs stream time: the merge and one score launch come first then.
@@ -1886,14 +1973,15 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
                      : infllm_merge_job(d.d_o_part, d.d_lse_part, parts, nullptr, nullptr, 0, d.B, d.H, a->n, a->d_out, a->o_sb, a->o_sh,
                                         a->o_sl, d.d_lse, &job);
         if (rc) return rc;
-        static const bool apart = getenv("INFLLM_SCORE_MERGE_APART") && getenv("INFLLM_SCORE_MERGE_APART")[0] != '0';
         rc = 1;
-        if (!apart && parts <= 8 && b1 > lo) {
+        if (!L->score_merge_apart && parts <= 8 && b1 > lo) {
             const infllm_score_args sc = local_score_args(L, a->n, a->b0, cur, lo, b1, 0);
             rc = infllm_local_score_merged(&sc, &job, stream);
             if (rc < 0) return rc;
+            if (rc == 0) ++L->n_score_merged;
         }
         if (rc == 1) {
+            ++L->n_score_apart;
             rc = merge(a->d_out, d.d_lse);
             if (rc) return rc;
             rc = run_local_score(L, a->n, a->b0, cur, lo, b1, 0, stream);
@@ -2046,6 +2134,7 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
         HIP_OK(hipEventRecord(L->idle_main, L->main_stream), "layer_flush: event");
         HIP_OK(hipEventRecord(L->idle_copy, (hipStream_t)copy_stream), "layer_flush: event");
         L->idle_recorded = true;
+        L->unflushed = false;
     }
     return 0;
 }

@@ -435,6 +435,45 @@ def test_topk_on_heavily_tied_scores_is_the_stable_descending_prefix(N, k, level
     assert idx.cpu().tolist() == order[:k]
 
 
+@pytest.mark.parametrize("N,k,pattern", [(6000, 16, "levels"), (16384, 16, "one_group"), (16384, 64, "one_group"), (9000, 16, "falling"),
+                                         (9000, 40, "rising"), (8192, 33, "constant"), (700, 64, "levels"), (16, 16, "falling")])
+def test_scores_and_selection_in_one_launch_give_the_stable_descending_prefix(N, k, pattern):
+    """infllm_score_topk where scoring and selection are ONE launch (rows of 512 elements, k <= 64, N <= 16384), on
+    scores made to be exact in fp32 (score = 256 * column 0 + column 1 of small integers): few distinct values, scores
+    that fall or rise with the unit number, all equal, and "one_group" - the high scores sit on the units that the
+    selection deals to ONE of its thread groups, so its threshold lets more candidates through than it can rank and
+    the exact bit-by-bit search takes over.  Always: the first k of a stable descending sort, in that order."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(N + k)
+    n = torch.arange(N)
+    if pattern == "levels":
+        val = torch.randint(0, 5, (N,), generator=g) - 2
+    elif pattern == "falling":
+        val = -n
+    elif pattern == "rising":
+        val = n
+    elif pattern == "constant":
+        val = torch.full((N,), 7)
+    else:
+        val = torch.where(n % 512 < 32, 1000 + torch.randint(0, 50, (N,), generator=g), torch.randint(0, 900, (N,), generator=g))
+    reps = torch.zeros((N, 512), dtype=torch.bfloat16)
+    reps[:, 0] = torch.div(val, 256, rounding_mode="floor").float()
+    reps[:, 1] = (val % 256).float()
+    qbar = torch.zeros(512)
+    qbar[0], qbar[1] = 256.0, 1.0
+    scores = torch.full((N,), float("nan"), dtype=torch.float32, device="cuda")
+    idx = torch.full((k,), -1, dtype=torch.int32, device="cuda")
+    ops.score_topk(reps.cuda(), N, qbar.cuda(), k, scores, idx)
+    assert scores.cpu().tolist() == val.float().tolist()
+    order = sorted(range(N), key=lambda i: (-int(val[i]), i))
+    assert idx.cpu().tolist() == order[:k]
+    # the same call again (the launch leaves its ticket slot ready for the next one), and a plain selection for reference
+    idx2, idx3 = torch.full_like(idx, -1), torch.full_like(idx, -1)
+    ops.score_topk(reps.cuda(), N, qbar.cuda(), k, scores, idx2)
+    ops.topk(scores, N, k, idx3)
+    assert torch.equal(idx2, idx) and torch.equal(idx3, idx)
+
+
 @pytest.mark.parametrize("bs,r,H,Hkv", [(128, 4, 32, 8), (8, 2, 4, 2), (100, 1, 3, 3), (64, 64, 2, 1)])
 def test_repr_keys_matches_oracle(bs, r, H, Hkv):
     ops = _ops()

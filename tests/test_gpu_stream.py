@@ -73,11 +73,14 @@ def test_page_table_in_the_launch_gives_the_bits_of_the_table_in_memory(monkeypa
             monkeypatch.delenv("INFLLM_PAGE_TABLE_KERNEL", raising=False)
         q, k, v = make_stream(T, H, Hkv, seed, B=B)
         out, cm = run_gpu(q, k, v, calls, base, **kw)
-        return out, [b["order"] for b in cm.trace_blocks]
+        return out, [b["order"] for b in cm.trace_blocks], cm.path_counts()
 
     for args in ((1500, [700, 1, 1, 798], 8, 2, 1e4, 45, 2, SMALL), (4096 + 2048, [4096, 2048], 32, 8, 1e6, 46, 1, REFERENCE)):
         a, b = run(False, *args), run(True, *args)
         assert torch.equal(a[0], b[0]) and a[1] == b[1] and len(a[1]) > 10
+        # the two runs really took the two paths (the switch is read when a layer is created)
+        assert a[2]["tables_inline"] >= 4 and a[2]["tables_kernel"] == 0, a[2]          # one table per block with a global stage
+        assert b[2]["tables_inline"] == 0 and b[2]["tables_kernel"] == a[2]["tables_inline"], (a[2], b[2])
 
 
 def test_score_decay_policy_follows_oracle():
@@ -227,10 +230,14 @@ def test_merge_carried_by_the_score_launch_gives_the_bits_of_the_two_launches(mo
                 monkeypatch.setenv("INFLLM_SCORE_MERGE_APART", apart)
                 out, cm = run_gpu(q, k, v, calls, base, **kw)
                 issued, _ = cm.prefetch_stats()
-                runs.append((out, [b["order"] for b in cm.trace_blocks], cm.trace_repr_indices(), cm.stats, issued))
+                runs.append((out, [b["order"] for b in cm.trace_blocks], cm.trace_repr_indices(), cm.stats, issued, cm.path_counts()))
             monkeypatch.delenv("INFLLM_SCORE_MERGE_APART")
-            (o0, s0, r0, st0, g0), (o1, s1, r1, st1, g1) = runs
-            assert torch.equal(o0, o1) and s0 == s1 and st0 == st1 and g1 > 0           # guesses ran: the one-launch form was used
+            (o0, s0, r0, st0, g0, p0), (o1, s1, r1, st1, g1, p1) = runs
+            assert torch.equal(o0, o1) and s0 == s1 and st0 == st1 and g1 > 0           # guesses ran
+            # ... and the carried form was used by the second run only (the switch is read when a layer is created)
+            # (windows of up to 1024 keys, the small geometry's, never take it: there both runs are the two-launch order)
+            assert p0["score_merged"] == 0 and p0["score_apart"] == p1["score_merged"] + p1["score_apart"], (p0, p1)
+            assert (p1["score_merged"] > 0) == (kw["n_local"] > 1024), (p0, p1)
             assert r0.keys() == r1.keys() and all(torch.equal(r0[u], r1[u]) for u in r0)
 
 

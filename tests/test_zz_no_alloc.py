@@ -72,6 +72,18 @@ def test_noalloc_forward_equals_the_workspace_forward_twice_in_a_row():
     assert first.shape != second.shape
     again = _both_ways(ops, big)                      # and the large one once more
     assert torch.equal(again, first)
+    # the advertised property: a call on a device that has been used before allocates nothing - neither on the device
+    # (hipMemGetInfo sees every hipMalloc, torch's included) nor through torch's allocator
+    blocks, o_part, lse_part, (B, H, Lq), _ = big
+    out, lse = torch.empty((B, H, Lq, D), dtype=torch.bfloat16, device="cuda"), torch.empty((B, H, Lq), device="cuda")
+    la, ga = blocks(o_part, lse_part)
+    torch.cuda.synchronize()
+    free0, held0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+    for _ in range(3):
+        ops.attn_fwd_noalloc(la, ga, out, lse)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_reserved() == held0
+    assert torch.equal(out, first)
     # beyond the built-in scratch: rejected, nothing launched
     B, H, Lq, P = 1, 32, 512, 8
     assert P * B * H * Lq > ops.NOALLOC_MAX_PART_ROWS
