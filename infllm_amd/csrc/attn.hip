@@ -426,16 +426,16 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
         // instruction instead of two additions.
         float psum[2] = {0.f, 0.f};
         uint32_t pw[2][8];
+        auto exps = [&](int ks, int r0, int r1) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
+            for (int r = r0; r < r1; r += 2) {
                 float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r], scale, neg_ms));
                 float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[ks][r + 1], scale, neg_ms));
                 pw[ks][r >> 1] = pack_bf16x2(p0, p1);
                 psum[ks] = sum_bf16x2(pw[ks][r >> 1], psum[ks]);
             }
-        l_run += psum[0] + psum[1];
+        };
+        exps(0, 0, 16);                        // the first 32 keys now; the other 32 beside the MFMAs that consume these
         {
             // 4 steps of 16 keys, 4 MFMAs each; the V^T operands of a step are requested from LDS while the
             // MFMAs of the previous step run
@@ -459,12 +459,26 @@ __global__ __launch_bounds__(kThreads, 2) void attn_stage_kernel(infllm_attn_arg
                 const int ks = gi >> 1, mm = gi & 1;
                 u32x4 praw{pw[ks][4 * mm], pw[ks][4 * mm + 1], pw[ks][4 * mm + 2], pw[ks][4 * mm + 3]};
                 bf16x8 pb = __builtin_bit_cast(bf16x8, praw);
+                // A wave's own vector-ALU work hides under its MFMAs when the two are interleaved instruction by
+                // instruction (an MFMA holds the matrix pipe for 32 cycles and the issue port for a few): the
+                // exponentials of the tile's second half go between the MFMAs of its first half.
+                if (gi < 2) exps(1, 8 * gi, 8 * gi + 8);
 #pragma unroll
                 for (int dt = 0; dt < kD / 32; ++dt)
                     oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[gi & 1][dt]), pb, oacc[dt], 0, 0, 0);
+                if (gi < 2) {
+#pragma unroll
+                    for (int dt = 0; dt < kD / 32; ++dt) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);      // multiply-adds, rounding, row sum
+                        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);      // two exponentials
+                        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                    }
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        l_run += psum[0] + psum[1];
     };
 
     // Tiles are handled in pairs: one barrier per two tiles.  While the pair (t, t+1) is multiplied, the next
