@@ -90,33 +90,126 @@ def counted_traffic(summary, key):
         return None
 
 
-def hbm_leg(dev, n_units=8192, tables=8, launches=200):
-    """The HBM half of the metric, measured in this run: unit scoring (context_manager.py:159-163) over n_units
-    representatives of H*D bf16 each, the shape of BASELINE config 3 - N*H*D*2 algorithmic bytes per launch (64 MiB),
-    read once.  The launches rotate over `tables` distinct tables (512 MiB together, more than the 256 MB of last-level
-    cache), so every launch reads from HBM; the figure is the MEAN over all launches, timed with events on the stream
-    the kernel runs on."""
-    from infllm_amd import ops
-    C = H * D
-    reps = torch.randn((tables, n_units, C), device=dev, dtype=torch.bfloat16)
-    qbar = torch.randn((C,), device=dev)
-    scores = torch.empty((n_units,), dtype=torch.float32, device=dev)
-    for i in range(2 * tables):
-        ops.score_topk(reps[i % tables], n_units, qbar, 0, scores, None)
+def _event_time_us(fn, launches, warm):
+    """mean microseconds per call of fn(i), timed with events on the stream the kernels are launched on"""
+    for i in range(warm):
+        fn(i)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for i in range(launches):
-        ops.score_topk(reps[i % tables], n_units, qbar, 0, scores, None)
+        fn(i)
     e1.record()
     torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / launches
+    return e0.elapsed_time(e1) / launches * 1e3
+
+
+def _hbm_entry(kernel, what, nbytes, us, launches, **extra):
+    gbs = nbytes / (us * 1e-6) / 1e9
+    return dict(kernel=kernel, what=what, algorithmic_bytes=int(nbytes), avg_us=us, GBps=gbs, frac_of_8TBps=gbs / 8000.0,
+                launches_timed=launches, **extra)
+
+
+def hbm_leg(dev, n_units=8192, tables=8, launches=200):
+    """The HBM half of the metric, measured in this run: a RETRIEVAL (context_manager.py:159-163: unit scores, then
+    their top-k) over n_units representatives of H*D bf16 each, the shape of BASELINE config 3, as ONE launch -
+    N*H*D*2 algorithmic bytes (64 MiB), read once (the selection re-reads the N fp32 scores: 32 KiB).  The launches
+    rotate over `tables` distinct tables (512 MiB together, more than the 256 MB of last-level cache), so every launch
+    reads from HBM; the figure is the MEAN over all launches, timed with events on the stream the kernel runs on.
+    Returns (roofline object of the retrieval, entry of the scoring kernel alone)."""
+    from infllm_amd import ops
+    C, k = H * D, KNOBS["topk"]
+    reps = torch.randn((tables, n_units, C), device=dev, dtype=torch.bfloat16)
+    qbar = torch.randn((C,), device=dev)
+    scores = torch.empty((n_units,), dtype=torch.float32, device=dev)
+    idx = torch.empty((k,), dtype=torch.int32, device=dev)
     nbytes = n_units * C * 2
-    gbs = nbytes / (ms * 1e-3) / 1e9
-    return {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0,
-            "traffic": counted_traffic("unit_scores__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"),
-            "kernel": f"unit_scores_rows_kernel ({n_units} x {C} bf16 representatives = {nbytes / 2 ** 20:.0f} MiB per launch, "
-                      f"{tables} tables in rotation)",
-            "avg_launch_ms": ms, "launches_timed": launches}
+    us = _event_time_us(lambda i: ops.score_topk(reps[i % tables], n_units, qbar, k, scores, idx), launches, 2 * tables)
+    gbs = nbytes / (us * 1e-6) / 1e9
+    retrieval = {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0,
+                 "traffic": counted_traffic("retrieval__decode8192.hbm_bytes.txt", "retrieval_traffic_bytes"),
+                 "kernel": f"retrieve_fused_kernel<8, 2>: unit scores + top-{k} in one launch ({n_units} x {C} bf16 representatives = "
+                           f"{nbytes / 2 ** 20:.0f} MiB per launch, {tables} tables in rotation)",
+                 "avg_launch_ms": us * 1e-3, "launches_timed": launches}
+    us = _event_time_us(lambda i: ops.score_topk(reps[i % tables], n_units, qbar, 0, scores, None), launches, 2 * tables)
+    scoring = _hbm_entry("unit_scores_rows_kernel<8, 2>", f"unit scores alone, {n_units} x {C} bf16, {tables} tables in rotation", nbytes, us,
+                         launches, traffic=counted_traffic("unit_scores__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"))
+    return retrieval, scoring
+
+
+def kernels_hbm_leg(dev):
+    """The other HBM-bound kernels of the path at the shapes the benchmark configurations give them, each timed in this
+    run with events over repeated launches; algorithmic bytes as the scope table counts them.  Inputs of more than a
+    few MB rotate over enough copies to exceed the last-level cache."""
+    import ctypes
+    from infllm_amd import ops
+    out = []
+    bf = dict(dtype=torch.bfloat16, device=dev)
+    n_local, bs, n_init, topk, exc = (KNOBS[k] for k in ("n_local", "block_size", "n_init", "topk", "exc_block_size"))
+    # ---- prologue of an append() call: RoPE, rings, rotated queries (rope.py:4-112, context_manager.py:712-747)
+    n = 8192
+    cap = (n_local + exc + bs + n + 63) // 64 * 64 + 64
+    q, k, v = (torch.randn((1, h, n, D), device=dev).bfloat16() for h in (H, HKV, HKV))
+    rings = [torch.zeros((1, HKV, cap, D), **bf) for _ in range(3)]
+    ring_score = torch.zeros((1, H, cap), dtype=torch.float32, device=dev)
+    q_loc, q_glb = torch.empty((1, H, n, D), **bf), torch.empty((1, H, n, D), **bf)
+    qpart = torch.empty((1, (n + 15) // 16, H * D), dtype=torch.float32, device=dev)
+    inv_freq = (ROPE_BASE ** (-torch.arange(0, D, 2, dtype=torch.float32) / D)).to(dev)
+    us = _event_time_us(lambda i: ops.ingest(q, k, v, 100000 + i * n, n_local - 1, inv_freq, 1.0, *rings, ring_score, q_loc, q_glb, qpart), 20, 3)
+    per_token = (H + 2 * HKV) * D * 2 + 2 * H * D * 2 + 3 * HKV * D * 2
+    out.append(_hbm_entry("ingest_kernel", f"prologue of an {n}-token append() call: reads q, k, v, writes both rotated q and three ring rows "
+                                           f"({per_token} B per token)", n * per_token, us, 20))
+    del q, k, v, q_loc, q_glb, qpart
+    # ---- representatives of the units a block carves (context_manager.py:268-277) and their rows out of the rings
+    n_units = exc // bs
+    rs = torch.rand((1, H, cap), dtype=torch.float32, device=dev)
+    rep = torch.empty((1, 64, H * D), **bf)
+    us = _event_time_us(lambda i: ops.repr_keys(rs, rings[0], 5000 + 7 * i, bs, n_units, KNOBS["repr_topk"], rep, rep.stride(0), rep.stride(1)), 200, 10)
+    per_unit = H * bs * 4 + H * KNOBS["repr_topk"] * D * 2 + H * D * 2
+    out.append(_hbm_entry("repr_keys_kernel", f"representatives of the {n_units} units of a block: scores, {KNOBS['repr_topk']} gathered keys per head, "
+                                              f"one row out ({per_unit} B per unit); a chain of dependent arg-max steps, latency-bound",
+                          n_units * per_unit, us, 200))
+    stage = torch.empty((n_units, 1, 2, HKV, bs, D), **bf)
+
+    def gather(i):
+        for which, ring in ((0, rings[0]), (1, rings[2])):
+            ops.gather_rows(ring, 5000 + 7 * i, n_units * bs, stage[0, 0, which].data_ptr(), stage.stride(1), stage.stride(3),
+                            unit_rows=bs, out_su=stage.stride(0))
+    unit_bytes = 2 * HKV * bs * D * 2
+    us = _event_time_us(gather, 200, 10)
+    out.append(_hbm_entry("gather_rows_kernel x2", f"K and V rows of a block's {n_units} carved units, ring -> staging ({unit_bytes} B per unit, "
+                                                   "read and written once)", n_units * unit_bytes, us, 200))
+    # ---- decode-shaped attention (config 3): one query per head over the window and the retrieved units, both stages + merge
+    sets, n_glob = 12, topk * bs + n_init + 64
+    ns_l, ns_g = 32, (n_glob // 64) // 2
+    capd = (n_local + 64 + 63) // 64 * 64 + 64
+    qd = torch.randn((1, H, 1, D), device=dev).bfloat16()
+    ring_k, ring_v = torch.randn((sets, 1, HKV, capd, D), device=dev).bfloat16(), torch.randn((sets, 1, HKV, capd, D), device=dev).bfloat16()
+    pool = torch.randn((sets, 2, HKV, n_glob, D), device=dev).bfloat16()
+    n_pages = n_glob // 64
+    pages = []
+    for s_ in range(sets):
+        ent = [(pool[s_, 0].data_ptr() + i * 64 * D * 2, pool[s_, 1].data_ptr() + i * 64 * D * 2, n_glob * D, 64) for i in range(n_pages)]
+        arr = ops.make_pages(ent)
+        host = torch.empty((n_pages * 32,), dtype=torch.uint8)
+        ctypes.memmove(host.data_ptr(), arr, n_pages * 32)
+        pages.append(host.to(dev))
+    o_part = torch.empty((ns_l + ns_g, 1, H, 1, D), dtype=torch.float16, device=dev)
+    lse_part = torch.empty((ns_l + ns_g, 1, H, 1), dtype=torch.float32, device=dev)
+    o, lse = torch.empty((1, H, 1, D), **bf), torch.empty((1, H, 1), dtype=torch.float32, device=dev)
+    b0 = 100000
+
+    def decode_attn(i):
+        s_ = i % sets
+        la = ops.linear_stage_args(qd, ring_k[s_], ring_v[s_], o_part[:ns_l], lse_part[:ns_l], cap=capd, j_lo=b0 - n_local, j_hi=b0 + 1,
+                                   mask=ops.MASK_WINDOW, offset=b0, window=n_local, nsplit=ns_l)
+        ga = ops.paged_stage_args(qd, pages[s_], n_pages, HKV, o_part[ns_l:], lse_part[ns_l:], nsplit=ns_g)
+        ops.attn_fwd(la, ga, o, lse)
+    us = _event_time_us(decode_attn, 200, 2 * sets)
+    nbytes = (n_local + 1 + n_glob) * HKV * D * 2 * 2
+    out.append(_hbm_entry("attn_stage_kernel<0> + <1> + attn_merge_wide_kernel", f"decode-shaped attention: 1 query x {H} heads over {n_local + 1} window keys "
+                          f"({ns_l} key splits) and {n_glob} retrieved keys ({ns_g} splits), K and V read once, three launches; "
+                          f"{sets} K/V sets in rotation", nbytes, us, 200))
+    return out
 
 
 def make_decode_state(dev, n_units, seed=3):
@@ -258,6 +351,75 @@ def model_workload(args, dev):
         "layer0_cache": cm.stats, "layer0_units": cm.num_global_block}))
 
 
+def extra_legs(args, dev):
+    """The other single-layer configurations, timed in this run so that their figures come with the headline:
+    the same 131,072-token stream with every unit resident (nothing crosses PCIe: the kernels' own time), BASELINE
+    config 3 (single-token steps over 8,192 prepared units) and config 5 (one 1,048,576-token stream whose queries
+    favour two mixture components per block)."""
+    from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
+    legs = {}
+    keep = KNOBS["max_cached_block"]
+    try:
+        q, k, v = make_stream(131072, 0, dev)
+        KNOBS["max_cached_block"] = 1024
+
+        times, prev = [], None
+        for i in range(5):                  # two warm-up steps, three timed ones, each on its own clock
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            cm, _ = run_stream(q, k, v, args.chunk)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            prev = cm                       # the previous step's manager goes once this step is done
+        del prev, cm
+        legs["all_resident_ms_per_step"] = sum(times[2:]) / 3 * 1e3
+        del q, k, v
+    except Exception as e:                                    # a leg never takes the headline down
+        legs["all_resident_ms_per_step"] = {"error": repr(e)}
+    finally:
+        KNOBS["max_cached_block"] = keep
+    try:
+        n_units, steps, warm = 8192, 64, 8
+        state, tokens = make_decode_state(dev, n_units)
+        rope = RotaryEmbeddingESM(D, base=ROPE_BASE, device=dev)
+        cm = ContextManager(rope, KNOBS["n_init"], KNOBS["n_local"], KNOBS["block_size"], KNOBS["max_cached_block"], KNOBS["topk"],
+                            KNOBS["exc_block_size"], None, True, KNOBS["repr_topk"], "lru", None, True, True).load_state(state)
+        del state
+        q, k, v = tokens(steps + warm)
+        one = lambda i: cm.append(q[:, :, i:i + 1], k[:, :, i:i + 1], v[:, :, i:i + 1], q[:, :, i:i + 1], k[:, :, i:i + 1], v[:, :, i:i + 1])
+        for i in range(warm):
+            one(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(warm, warm + steps):
+            out = one(i)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert torch.isfinite(out.float()).all()
+        legs["decode_leg"] = {"workload": f"config 3: {steps} single-token steps over {n_units} prepared units ({n_units * KNOBS['block_size']} past tokens)",
+                              "ms_per_step": dt / steps * 1e3, "steps_per_s": steps / dt, "cache": dict(cm.stats)}
+        del cm, q, k, v
+    except Exception as e:
+        legs["decode_leg"] = {"error": repr(e)}
+    try:
+        T5 = 1 << 20
+        q, k, v = make_stream(T5, 5, dev, favour=2)
+        cm, out = run_stream(q, k, v, args.chunk)              # pins the units' host memory once (4 GiB)
+        torch.cuda.synchronize()
+        del cm, out
+        t0 = time.perf_counter()
+        cm, out = run_stream(q, k, v, args.chunk)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert torch.isfinite(out.float()).all() and cm.length == T5
+        legs["million_leg"] = {"workload": f"config 5: one {T5}-token stream, queries favour 2 mixture components per block, max_cached {keep}, lru",
+                               "ms_per_step": dt * 1e3, "tokens_per_s": T5 / dt, "units": cm.num_global_block, "cache": dict(cm.stats)}
+        del cm, q, k, v
+    except Exception as e:
+        legs["million_leg"] = {"error": repr(e)}
+    return legs
+
+
 def cpu_baseline(tokens, threads, seed=1):
     """BASELINE config 1: the reference's torch path restated (the fp32 oracle; the reference's own files hard-code
     "cuda") on the host cores - q, k, v i.i.d. N(0,1) from `seed`, fp32, the first `tokens` tokens of the
@@ -287,7 +449,8 @@ def main():
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--chunk", type=int, default=8192, help="tokens per append() call")
     ap.add_argument("--cpu-tokens", type=int, default=16384, help="tokens of config 1 the CPU baseline runs (0 disables it)")
-    ap.add_argument("--no-hbm-leg", action="store_true", help="skip the unit-scoring (HBM roofline) measurement")
+    ap.add_argument("--no-hbm-leg", action="store_true", help="skip the HBM-bound kernels' measurements (roofline_hbm, kernels_hbm)")
+    ap.add_argument("--no-extra-legs", action="store_true", help="skip the all-resident, decode (config 3) and 1M-token (config 5) legs")
     ap.add_argument("--workload", choices=["prefill", "decode", "model"], default="prefill",
                     help="prefill = the headline 128K-token stream (config 2); decode = config 3, model = config 4 "
                          "(each with its own JSON line)")
@@ -392,8 +555,12 @@ def main():
                                 "candidates a guess fetched in vain and what its repair brought back; units still in a carve staging slot "
                                 "are copied on the device.  PCIe 5.0 x16: 64 GB/s raw; 8 DMA engines move 13 units at 54 GB/s on an idle "
                                 "GPU; in the stream 7 engines fetch and the 8th takes the carved units to the host"}
+    del q, k, v, out, runs
+    if not args.no_extra_legs and not args.favour and T == 131072 and args.max_cached_block == 32:
+        res.update(extra_legs(args, dev))
     if not args.no_hbm_leg:
-        res["roofline_hbm"] = hbm_leg(dev)
+        res["roofline_hbm"], scoring = hbm_leg(dev)
+        res["kernels_hbm"] = [scoring] + kernels_hbm_leg(dev)
     if args.cpu_tokens > 0:
         res["cpu_baseline"] = cpu_baseline(min(args.cpu_tokens, 16384), min(os.cpu_count() or 1, 16))
     print(json.dumps(res))
