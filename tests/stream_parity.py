@@ -10,10 +10,16 @@ Acceptance rules (written here once, used by every stream test):
 * representative keys (the repr_topk best tokens of a unit per query head): a pick may differ from the oracle's only
   if the oracle's scores of the swapped tokens lie within REPR_TIE_REL = 1e-2 relative of the repr_topk-th score.  The
   token scores are sums of bf16-MFMA probabilities (rotated q and k are rounded to bf16 once, 2^-9 relative each, as
-  the reference's bf16 runs round them): a logit moves by about 1.6e-3 (one sigma), and so does the score of a token
-  whose mass comes from few queries, which is the case with clustered keys.  1e-2 is six sigma of that; how often a
-  pick differs at all, and by more than 1e-3, is counted (Follower.stats) and bounded by the sweep in
-  test_gpu_stream.py.
+  the reference's bf16 runs round them), so the score of a token whose mass comes from few queries moves by a few
+  1e-3.  Measured: over 18,560 picks of unfavoured streams (20 of the small geometry, 10 of the reference geometry,
+  N(0,1) and mixture keys) plus the 2,880 picks of the two-layer Llama-3-8B-shaped model 1.5 % of the picks differ at
+  all, 15 of them by more than 1e-3, the largest gaps being 1.19e-3 (mixture keys), 1.40e-3 (N(0,1) keys), 2.05e-3
+  (small geometry) and 2.09e-3 (model activations); such streams are held to UNFAVOURED_GAP = 4e-3, twice the
+  largest.  BASELINE config 5 is the wide one: its queries lean towards two mixture components per block, so a token's
+  mass comes from a handful of near-one probabilities - 19 of 2,560 picks differ, 14 by more than 1e-3, five beyond
+  4e-3, the largest 6.29e-3 (the same with the score kernel of either form, bit for bit); it is held to the full 1e-2.
+  How often a pick differs at all, and by more than 1e-3, is counted (Follower.stats), bounded for every stream by
+  assert_tie_stats() and in total by the sweep in test_gpu_stream.py.
 
 Where a choice differs within its rule the oracle adopts the GPU's (topk_hook / repr_hook), so that the two
 trajectories stay comparable: every later decision is then judged on the same history.  The oracle keeps its
@@ -26,6 +32,7 @@ from oracle.stream import StreamOracle
 
 MAX_ABS, MEAN_ABS = 2e-2, 2e-3
 TIE_REL, REPR_TIE_REL = 1e-3, 1e-2
+UNFAVOURED_GAP = 4e-3
 D = 128
 
 SMALL = dict(n_init=16, n_local=256, block_size=32, max_cached_block=8, topk=4, exc_block_size=64, repr_topk=2)
@@ -90,6 +97,7 @@ class Follower:
         self.topk, self.repr_topk = topk, repr_topk
         self.violations = []
         self.stats = dict(selections=0, tie_topk=0, order_swaps=0, picks=0, tie_repr=0, repr_beyond_1e3=0, repr_max_gap=0.0)
+        self.repr_gaps = []           # relative gap of every pick that differs from the oracle's
 
     def topk_hook(self, block, row, scores):
         st = self.stats
@@ -129,9 +137,22 @@ class Follower:
                 if max(gaps) > REPR_TIE_REL:
                     self.violations.append(("repr", unit, row, h, sorted(a ^ b), max(gaps)))
                 st["tie_repr"] += 1
+                self.repr_gaps.append(max(gaps))
                 st["repr_beyond_1e3"] += max(gaps) > TIE_REL
                 st["repr_max_gap"] = max(st["repr_max_gap"], max(gaps))
         return gpu
+
+
+def assert_tie_stats(fol, what, max_gap=UNFAVOURED_GAP):
+    """Print how often the tie rules were used on one stream and bound it: picks that differ at all <= 4 %, by more
+    than 1e-3 <= 1 %, none beyond max_gap (REPR_TIE_REL itself is a violation); selections that differ in set or order
+    <= 10 % (at least two are allowed: streams of twenty selections)."""
+    st = fol.stats
+    print(f"{what}: {st}")
+    assert not fol.violations, fol.violations[:5]
+    assert st["repr_max_gap"] <= max_gap, (what, st)
+    assert st["tie_repr"] <= max(2, 0.04 * st["picks"]) and st["repr_beyond_1e3"] <= max(2, 0.01 * st["picks"]), (what, st)
+    assert st["tie_topk"] + st["order_swaps"] <= max(2, 0.10 * st["selections"]), (what, st)
 
 
 def assert_outputs_close(got, want, what="", relative_above_one=False):

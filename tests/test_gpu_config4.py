@@ -14,7 +14,7 @@ through the closed forms of the state machine, GreedySearch's call schedule and 
 import pytest
 import torch
 
-from stream_parity import REFERENCE, follow
+from stream_parity import REFERENCE, assert_tie_stats, follow
 
 pytestmark = pytest.mark.gpu
 transformers = pytest.importorskip("transformers")
@@ -115,7 +115,7 @@ def test_config4_two_layers_at_llama3_geometry_follow_the_oracle_layer_by_layer(
         assert fol.stats["selections"] == len(full) == sum(1 for p, n in _blocks_of(calls) if _units_after(p) > TOPK)
         assert fol.stats["picks"] == H * cm.num_global_block
         assert cm.stats["misses"] > 0 and cm.stats["evictions"] > 0
-        print(f"config 4, layer {i}: {fol.stats}")
+        assert_tie_stats(fol, f"config 4, layer {i}")
 
 
 def test_config4_full_size_thirty_two_layers_prefill_and_greedy_steps(monkeypatch):

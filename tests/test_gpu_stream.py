@@ -11,7 +11,8 @@ import pytest
 import torch
 
 from oracle.rope import RopeOracle
-from stream_parity import (D, REFERENCE, REPR_TIE_REL, SMALL, TIE_REL, Follower, compare, make_stream, new_manager, run_gpu)
+from stream_parity import (D, REFERENCE, REPR_TIE_REL, SMALL, TIE_REL, UNFAVOURED_GAP, Follower, compare, make_stream, new_manager,
+                           run_gpu)
 
 pytestmark = pytest.mark.gpu
 
@@ -359,13 +360,14 @@ def test_state_export_and_injection_resume_the_stream_exactly():
     assert cm_b.length == T0 + T1 == cm1.length and cm_b.num_global_block == cm1.num_global_block
 
 
-def test_pick_and_selection_ties_are_rare_and_within_their_rules():
+def test_pick_and_selection_ties_are_rare_and_within_their_rules(tmp_path):
     """How often the GPU's discrete choices differ from the fp32 oracle's, over 20 seeded streams of the small geometry
     and 3 of the reference geometry, with N(0,1) keys and with mixture keys.  Every difference must lie within its
-    rule (stream_parity.py: 1e-3 for unit selections, 1e-2 for representative keys - compare() asserts that); here
+    rule (stream_parity.py: 1e-3 for unit selections, 1e-2 for representative keys - compare() asserts that - and 4e-3
+    for the unfavoured streams used here); here
     the FREQUENCIES are bounded: at most 2 % of the representative picks differ at all, at most 0.5 % by more than
-    1e-3, at most 2 % of the selections differ in their set.  The counts are printed and left in a JSON file in the
-    folder for run outputs (INFLLM_TEST_OUT, else the one this build's GPU runs bring back)."""
+    1e-3, at most 2 % of the selections differ in their set.  The counts are printed and left in a JSON file in
+    pytest's temporary folder, or in the folder INFLLM_TEST_OUT names."""
     rows = []
     for seed in range(20):
         mixture = seed % 2 == 0
@@ -378,7 +380,7 @@ def test_pick_and_selection_ties_are_rare_and_within_their_rules():
     tot = {k: sum(r[k] for r in rows) for k in ("selections", "tie_topk", "order_swaps", "picks", "tie_repr", "repr_beyond_1e3")}
     tot["repr_max_gap"] = max(r["repr_max_gap"] for r in rows)
     try:
-        out_dir = os.environ.get("INFLLM_TEST_OUT", "gpurun_out")
+        out_dir = os.environ.get("INFLLM_TEST_OUT") or str(tmp_path)
         os.makedirs(out_dir, exist_ok=True)
         with open(os.path.join(out_dir, "tie_sweep.json"), "w") as f:
             json.dump(dict(total=tot, runs=rows), f, indent=1)
@@ -386,7 +388,7 @@ def test_pick_and_selection_ties_are_rare_and_within_their_rules():
         pass
     print("tie sweep:", json.dumps(tot))
     assert tot["picks"] > 5000 and tot["selections"] > 300
-    assert tot["repr_max_gap"] <= REPR_TIE_REL
+    assert tot["repr_max_gap"] <= UNFAVOURED_GAP
     assert tot["tie_repr"] <= 0.02 * tot["picks"], tot
     assert tot["repr_beyond_1e3"] <= 0.005 * tot["picks"], tot
     assert tot["tie_topk"] <= 0.02 * tot["selections"], tot
