@@ -39,6 +39,27 @@ from .. import _lib
 from .._lib import BackArgs, FrontArgs, LayerDesc, check
 from ..ops import HEAD_DIM, KEY_TILE
 
+
+# Heads narrower than the kernels' 128 dimensions (MiniCPM's 64, config/minicpm-inf-llm.yaml) run on the same kernels:
+# the two halves of a row go to dimensions [0, D/2) and [64, 64 + D/2) of a 128-wide row and the rest is zero.  RoPE
+# pairs dimension d with d + D/2 (rope.py:31-33), which are d and d + 64 in the wide row - the pairing the prologue
+# kernel uses - with zero frequencies in the unused slots; zeros add nothing to q.k, to the representatives' scores or
+# to the outputs, whose real dimensions are picked out again on the way back.  Twice the bytes and flops a kernel
+# built for 64 would need: a way to run such models, not a fast path.
+def _widen(t, d):
+    if d == HEAD_DIM:
+        return t
+    out = t.new_zeros(t.shape[:-1] + (HEAD_DIM,))
+    out[..., :d // 2] = t[..., :d // 2]
+    out[..., HEAD_DIM // 2:HEAD_DIM // 2 + d // 2] = t[..., d // 2:]
+    return out
+
+
+def _narrow(t, d):
+    if d == HEAD_DIM:
+        return t
+    return torch.cat((t[..., :d // 2], t[..., HEAD_DIM // 2:HEAD_DIM // 2 + d // 2]), dim=-1)
+
 _SIDE_STREAM = None          # one process-wide side stream, like GLOBAL_STREAM (context_manager.py:193)
 _CALL_BUFFERS = {}           # (device, stream, geometry) -> the buffers of a call prepared in one go, see _bind_call_buffers
 _HOST_CHUNK_UNITS = 64       # units per pinned host allocation
@@ -172,8 +193,7 @@ class ContextManager:
         B, H, _, D = q.shape
         Hkv = k.shape[1]
         dev = q.device
-        if D != HEAD_DIM:
-            raise ValueError(f"the HIP kernels are built for head_dim {HEAD_DIM}, got {D}")
+        assert D == HEAD_DIM                                    # rows arrive widened (see _widen)
         if self.topk > self.max_cached_block:
             raise ValueError("topk must not exceed max_cached_block")
         if self.topk > 64:
@@ -183,7 +203,7 @@ class ContextManager:
         self.batch_size = self.num_units = B
         self.num_heads = self.unit_size = H
         self.num_heads_kv = self.unit_size_kv = Hkv
-        self.dim_head = D
+        self.head_width = D                                     # of the rows the kernels see; self.dim_head is the caller's
         self.dtype = q.dtype
         self.device = dev
         bs, exc, topk = self.block_size, self.exc_block_size, self.topk
@@ -230,7 +250,11 @@ class ContextManager:
         self.pages_host = torch.empty((_PAGE_SLOTS * B * self.max_pages * page_bytes,), dtype=torch.uint8, pin_memory=True)
         self.max_carve = (exc + self.n_init) // bs + 2
         self.carve_stage = torch.empty((_CARVE_SLOTS, self.max_carve, B, 2, Hkv, bs, D), **bf)
-        self.inv_freq = self.position_embedding.inv_freq.to(device=dev, dtype=torch.float32).contiguous()
+        inv_freq = self.position_embedding.inv_freq.to(device=dev, dtype=torch.float32)
+        if inv_freq.numel() != self.dim_head // 2:
+            raise ValueError(f"the rotary embedding is built for head_dim {2 * inv_freq.numel()}, the heads have {self.dim_head}")
+        self.inv_freq = torch.zeros((HEAD_DIM // 2,), dtype=torch.float32, device=dev)
+        self.inv_freq[:inv_freq.numel()] = inv_freq                # the slots of a narrow head's padding rotate by nothing
         self.slot_bytes = 2 * Hkv * bs * D * 2              # one unit of one batch row
         self.unit_bytes = B * self.slot_bytes               # one unit, all batch rows
 
@@ -260,7 +284,7 @@ class ContextManager:
         d.d_carve_stage, d.max_carve, d.carve_slots = self.carve_stage.data_ptr(), self.max_carve, _CARVE_SLOTS
         d.d_inv_freq = self.inv_freq.data_ptr()
         d.distance_scale = float(self.position_embedding.distance_scale)
-        d.softmax_scale = 1.0 / (D ** 0.5)
+        d.softmax_scale = 1.0 / (self.dim_head ** 0.5)
         self._lib = _lib.load()
         self._layer = self._lib.infllm_layer_create(ctypes.byref(d))
         if not self._layer:
@@ -311,7 +335,7 @@ class ContextManager:
         """Buffers of a call prepared in one go: the rotated queries of up to call_tokens tokens, the blocks' mean
         queries and the local stage's partial rows.  They are dead between append() calls, so the layers that work on
         one stream (one after the other, as the layers of a model do) share one set."""
-        B, H, D, exc, T = self.num_units, self.unit_size, self.dim_head, self.exc_block_size, self._call_tokens
+        B, H, D, exc, T = self.num_units, self.unit_size, self.head_width, self.exc_block_size, self._call_tokens
         group = int(os.environ.get("INFLLM_LOCAL_GROUP", self.local_group_blocks))
         blocks = max(8, 4 * group)            # partial rows: two groups of blocks, up to two key splits each
         dev = self.device.index if self.device.index is not None else torch.cuda.current_device()
@@ -342,7 +366,7 @@ class ContextManager:
         """Address of the pinned host copy [B, 2, Hkv, bs, D] of a unit."""
         chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
         while chunk >= len(self.host_chunks):
-            t = torch.empty((_HOST_CHUNK_UNITS, self.num_units, 2, self.unit_size_kv, self.block_size, self.dim_head),
+            t = torch.empty((_HOST_CHUNK_UNITS, self.num_units, 2, self.unit_size_kv, self.block_size, self.head_width),
                             dtype=torch.bfloat16, pin_memory=True)
             self.host_chunks.append(t)
             self._host_base.append(t.data_ptr())
@@ -359,10 +383,19 @@ class ContextManager:
             self._sa.n_chunks = len(self._host_dev_base)
         return self._host_base[chunk] + idx * self.unit_bytes
 
-    def host_unit(self, unit):
-        """Pinned host tensor [B, 2, Hkv, bs, D] of a carved unit (K at index 0, V at 1)."""
+    def _host_unit_rows(self, unit):
         chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
         return self.host_chunks[chunk][idx]
+
+    def host_unit(self, unit):
+        """Pinned host tensor [B, 2, Hkv, bs, D] of a carved unit (K at index 0, V at 1); for heads narrower than 128 a
+        copy with the real dimensions picked out."""
+        return _narrow(self._host_unit_rows(unit), self.dim_head)
+
+    def rep_rows(self, row, lo, hi):
+        """Representatives of units [lo, hi) of batch row `row` as a CPU fp32 tensor [hi - lo, H * D]."""
+        r = self.reps[row, lo:hi].view(hi - lo, self.unit_size, self.head_width)
+        return _narrow(r, self.dim_head).reshape(hi - lo, -1).float().cpu()
 
     # ----------------------------------------------------------------- timing
     def enable_timing(self, capacity, stride=1):
@@ -546,7 +579,7 @@ class ContextManager:
         n_blocks = -(-(c1 - c0) // exc)
         if N <= topk:
             return [[list(range(N))] * B for _ in range(n_blocks)]
-        C = self.unit_size * self.dim_head
+        C = self.unit_size * self.head_width
         qbar = torch.empty((B, n_blocks, C), dtype=torch.float32, device=self.device)
         check(self._lib.infllm_chunk_qbar(q.data_ptr() + c0 * q.stride(2) * 2, q.stride(0), q.stride(1), q.stride(2), B,
                                           self.unit_size, c1 - c0, exc, self.inv_freq.data_ptr(),
@@ -600,6 +633,13 @@ class ContextManager:
                               .reshape(batch_size * heads, 1, input_length, -1))
             q, k, v = q.reshape(batch_size * heads, 1, input_length, -1), rep(k), rep(v)
         if not self.initialized:
+            self.dim_head = q.size(3)
+            if self.dim_head > HEAD_DIM or self.dim_head % 2:
+                raise ValueError(f"head_dim must be even and at most {HEAD_DIM}, got {self.dim_head}")
+        if q.size(3) != self.dim_head:
+            raise ValueError(f"head_dim changed from {self.dim_head} to {q.size(3)}")
+        q, k, v = _widen(q, self.dim_head), _widen(k, self.dim_head), _widen(v, self.dim_head)
+        if not self.initialized:
             self._init(q, k)
             self._bind_reps()
         assert q.shape[:2] == (self.num_units, self.unit_size) and k.shape[1] == self.unit_size_kv
@@ -608,7 +648,7 @@ class ContextManager:
             ok = t.stride(-1) == 1 and not any(s % 8 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
             return t if ok else t.contiguous()
         q, k, v = rows16(q), rows16(k), rows16(v)
-        out = torch.empty((self.num_units, self.unit_size, input_length, self.dim_head), dtype=torch.bfloat16, device=q.device)
+        out = torch.empty((self.num_units, self.unit_size, input_length, self.head_width), dtype=torch.bfloat16, device=q.device)
         fa, ba = self._fa, self._ba
         fa.q_sb, fa.q_sh, fa.q_sl = q.stride(0), q.stride(1), q.stride(2)
         fa.k_sb, fa.k_sh, fa.k_sl = k.stride(0), k.stride(1), k.stride(2)
@@ -657,6 +697,7 @@ class ContextManager:
             self._block(st, n, out_ptr + st * out_step, min(exc, call_end - st - n), chosen)
         self.length += input_length
         check(self._lib.infllm_layer_flush(self._layer, self._copy_raw), "infllm_layer_flush")
+        out = _narrow(out, self.dim_head)
         if self.perhead:
             out = out.view(batch_size, heads, input_length, -1)
         return out
@@ -671,12 +712,14 @@ class ContextManager:
         T, cur, cap = self.length, self.cursor, self.ring_cap
         rows = torch.arange(cur, T, device=self.device) % cap
         units = [self.host_unit(u).clone() for u in range(self.num_global_block)] if with_units else []
-        return dict(length=T, n_units=self.num_global_block, init_len=self.init_len,
-                    tail_k=self.ring_k_raw[:, :, rows].clone(), tail_v=self.ring_v[:, :, rows].clone(),
+        d, n = self.dim_head, self.num_global_block
+        reps = _narrow(self.reps[:, :n].view(self.num_units, n, self.unit_size, self.head_width), d).reshape(self.num_units, n, -1)
+        return dict(length=T, n_units=n, init_len=self.init_len,
+                    tail_k=_narrow(self.ring_k_raw[:, :, rows], d).clone(), tail_v=_narrow(self.ring_v[:, :, rows], d).clone(),
                     tail_score=self.ring_score[:, :, rows].clone(),
-                    init_k=self.init_kv[:, 0, :, :self.init_len].clone(), init_v=self.init_kv[:, 1, :, :self.init_len].clone(),
-                    units=torch.stack(units) if units else None,
-                    reps=self.reps[:, :self.num_global_block].clone())
+                    init_k=_narrow(self.init_kv[:, 0, :, :self.init_len], d).clone(),
+                    init_v=_narrow(self.init_kv[:, 1, :, :self.init_len], d).clone(),
+                    units=torch.stack(units) if units else None, reps=reps.clone())
 
     def load_state(self, state):
         """Start from a prepared memory.  ``state``: length T; tail_k/tail_v [B,Hkv,T-cursor,D] (un-rotated,
@@ -696,21 +739,26 @@ class ContextManager:
         cursor = init_len + n_units * self.block_size
         assert n_tail == T - cursor, f"tail holds {n_tail} tokens, the stream state needs {T - cursor}"
         assert state["init_k"].shape[2] == init_len and (n_units == 0 or state["units"].shape[0] == n_units)
-        q_like = torch.empty((B, H, 1, D), dtype=torch.bfloat16, device=tail_k.device)
+        if D > HEAD_DIM or D % 2:
+            raise ValueError(f"head_dim must be even and at most {HEAD_DIM}, got {D}")
+        self.dim_head = D
+        tail_k, tail_v = _widen(tail_k, D), _widen(tail_v, D)
+        q_like = torch.empty((B, H, 1, HEAD_DIM), dtype=torch.bfloat16, device=tail_k.device)
         self._init(q_like, tail_k[:, :, :1])
         self._bind_reps()
         self.length, self.cursor, self.init_len = T, cursor, init_len
         if init_len:
-            self.init_kv[:, 0, :, :init_len] = state["init_k"]
-            self.init_kv[:, 1, :, :init_len] = state["init_v"]
+            self.init_kv[:, 0, :, :init_len] = _widen(state["init_k"], D)
+            self.init_kv[:, 1, :, :init_len] = _widen(state["init_v"], D)
         if n_units:
             self._grow_reps(n_units) if n_units > self.reps.shape[1] else None
-            self.reps[:, :n_units] = reps
+            self.reps[:, :n_units] = _widen(reps.view(B, n_units, H, D), D).reshape(B, n_units, -1)
             for u in range(n_units):
                 self._host_unit_addr(u)                        # allocates the pinned chunk
-                self.host_unit(u).copy_(state["units"][u])
+                self._host_unit_rows(u).copy_(_widen(state["units"][u], D))
             self.num_global_block = n_units
         # tail -> rings (RoPE at the absolute positions) in pieces of one execution block
+        D = HEAD_DIM
         zq = torch.zeros((B, H, self.exc_block_size, D), dtype=torch.bfloat16, device=self.device)
         for st in range(0, n_tail, self.exc_block_size):
             n = min(self.exc_block_size, n_tail - st)

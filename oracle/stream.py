@@ -37,6 +37,12 @@ breaks ties between equal stamps at later evictions (:253-265).
 reference keeps them in a VectorTensor of the model dtype (:321-328, 675), so
 torch.bfloat16 restates its bf16 runs; None keeps the compute dtype.
 
+``q_dtype`` restates the roundings the reference's low-precision runs apply on the way
+to the mean query of a block: the one-angle-rotated queries are a tensor of the model
+dtype and so is their mean (context_manager.py:373-375), i.e. every rotated query is
+rounded before the sum and the mean after it.  None keeps the compute dtype throughout
+(the HIP path sums the unrounded fp32 rotations and keeps the mean in fp32).
+
 ``StreamOracle.from_state`` starts from a snapshot (window, un-carved tail with
 its score track, init tokens, units, representatives - the fields of
 context_manager.py:309-363 restated in absolute terms) instead of an empty
@@ -106,7 +112,7 @@ class UnitCacheModel:
 class StreamOracle:
     def __init__(self, rope, n_init, n_local, block_size, max_cached_block, topk,
                  exc_block_size, score_decay=None, repr_topk=1, cache_strategy="lru",
-                 perhead=False, topk_hook=None, repr_hook=None, chunk_topk_calc=None, rep_dtype=None):
+                 perhead=False, topk_hook=None, repr_hook=None, chunk_topk_calc=None, rep_dtype=None, q_dtype=None):
         assert exc_block_size <= n_local                      # context_manager.py:219
         self.chunk_topk_calc = chunk_topk_calc
         self.rope = rope
@@ -120,6 +126,7 @@ class StreamOracle:
         self.perhead = perhead
         self.topk_hook, self.repr_hook = topk_hook, repr_hook
         self.rep_dtype = rep_dtype
+        self.q_dtype = q_dtype
         self.length = 0
         self.ready = False
         self._chunk_plan = None
@@ -221,7 +228,11 @@ class StreamOracle:
             chosen = [list(range(self.n_units)) for _ in range(self.B)]
             scores = [None] * self.B
         else:
-            mean_q = gq_block.mean(dim=2).reshape(self.B, self.H * self.D)
+            if self.q_dtype is not None:                                       # :373-375 in the model dtype
+                mean_q = gq_block.to(self.q_dtype).float().mean(dim=2).to(self.q_dtype).to(gq_block.dtype)
+            else:
+                mean_q = gq_block.mean(dim=2)
+            mean_q = mean_q.reshape(self.B, self.H * self.D)
             chosen, scores = [], []
             for u in range(self.B):
                 reps = torch.stack(self.reps[u])                       # [N, H*D]

@@ -39,7 +39,7 @@ SMALL = dict(n_init=16, n_local=256, block_size=32, max_cached_block=8, topk=4, 
 REFERENCE = dict(n_init=128, n_local=4096, block_size=128, max_cached_block=32, topk=16, exc_block_size=512, repr_topk=4)
 
 
-def make_stream(T, H, Hkv, seed, B=1, mixture=True):
+def make_stream(T, H, Hkv, seed, B=1, mixture=True, D=D):
     """q, v ~ N(0,1); keys from a 64-component Gaussian mixture (std 0.3 around N(0,1) means), or N(0,1)."""
     g = torch.Generator().manual_seed(seed)
     q = torch.randn(B, H, T, D, generator=g)
@@ -55,7 +55,7 @@ def make_stream(T, H, Hkv, seed, B=1, mixture=True):
 
 def new_manager(base, **kw):
     from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
-    rope = RotaryEmbeddingESM(D, base=base, device="cuda")
+    rope = RotaryEmbeddingESM(kw.get("dim", D), base=base, device="cuda")
     return ContextManager(rope, kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"], kw["topk"],
                           kw["exc_block_size"], kw.get("score_decay"), False, kw.get("repr_topk", 1),
                           kw.get("cache_strategy", "lru"), kw.get("chunk_topk_calc"), kw.get("async_global_stream", False), False, False,
@@ -81,7 +81,7 @@ def run_gpu(q, k, v, calls, base, **kw):
 
 
 def new_oracle(base, follower=None, **kw):
-    return StreamOracle(RopeOracle(D, base=base), kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"],
+    return StreamOracle(RopeOracle(kw.get("dim", D), base=base), kw["n_init"], kw["n_local"], kw["block_size"], kw["max_cached_block"],
                         kw["topk"], kw["exc_block_size"], repr_topk=kw.get("repr_topk", 1), perhead=kw.get("perhead", False),
                         topk_hook=follower.topk_hook if follower else None, repr_hook=follower.repr_hook if follower else None,
                         cache_strategy=kw.get("cache_strategy", "lru"), score_decay=kw.get("score_decay"),
@@ -173,7 +173,7 @@ def assert_reps_match(cm, ora, first_unit=0):
         return
     for u in range(len(ora.reps)):
         want = torch.stack(ora.reps[u][first_unit:n]).float()
-        got = cm.reps[u, first_unit:n].float().cpu()
+        got = cm.rep_rows(u, first_unit, n)
         tol = 2.0 ** -7 * torch.maximum(want.abs(), got.abs()) + 1e-30
         assert bool(((got - want).abs() <= tol).all()), (u, float((got - want).abs().max()))
 
@@ -205,7 +205,7 @@ def follow(cm, got, q, k, v, calls, base, relative_above_one=False, **kw):
 
 def compare(T, calls, H, Hkv, base, seed, B=1, mixture=True, **kw):
     """One stream through the GPU ContextManager and through the oracle following it; returns (cm, oracle, follower)."""
-    q, k, v = make_stream(T, H, Hkv, seed, B=B, mixture=mixture)
+    q, k, v = make_stream(T, H, Hkv, seed, B=B, mixture=mixture, D=kw.get("dim", D))
     got, cm = run_gpu(q, k, v, calls, base, **kw)
     assert sum(calls) == T
     ora, fol = follow(cm, got, q, k, v, calls, base, **kw)

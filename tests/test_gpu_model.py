@@ -21,12 +21,12 @@ KNOBS = dict(n_local=128, n_init=8, topk=16, block_size=16, max_cached_block=16,
 LOGIT_TOL = 6e-2
 
 
-def _models():
+def _models(head_dim=128):
     from infllm_amd import attention
     from infllm_amd.utils import patch_hf
     torch.manual_seed(1)
-    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
-                                   num_key_value_heads=1, head_dim=128, vocab_size=300, rope_theta=500000.0)
+    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=256 // head_dim,
+                                   num_key_value_heads=128 // head_dim, head_dim=head_dim, vocab_size=300, rope_theta=500000.0)
     base = transformers.LlamaForCausalLM(cfg).bfloat16().eval()
     attention.ATTN_FORWRAD["oracle-inf-llm"] = oracle_inf_llm_forward
     cpu = patch_hf(copy.deepcopy(base).float(), "oracle-inf-llm", dict(KNOBS))
@@ -41,10 +41,11 @@ class _Tok:
         return " ".join(str(int(i)) for i in ids)
 
 
-def test_chunked_prefill_logits_and_greedy_tokens_follow_the_cpu_model():
+@pytest.mark.parametrize("head_dim", [128, 64])
+def test_chunked_prefill_logits_and_greedy_tokens_follow_the_cpu_model(head_dim):
     from infllm_amd.attention import ContextManager
     from infllm_amd.utils import GreedySearch
-    gpu, cpu = _models()
+    gpu, cpu = _models(head_dim)
     ids = torch.randint(0, 300, (1, 333), generator=torch.Generator().manual_seed(2))
     with torch.inference_mode():
         past_g = past_c = None
@@ -58,14 +59,14 @@ def test_chunked_prefill_logits_and_greedy_tokens_follow_the_cpu_model():
     assert past_g[0].num_global_block == past_c[0].n_units == 12                # units were carved and attended
     assert past_g[0].stats["misses"] > 0
 
-    gpu, cpu = _models()
+    gpu, cpu = _models(head_dim)
     text_g = GreedySearch(gpu, _Tok()).generate(input_ids=ids[0], max_length=8, chunk_size=64)[0].split()
     gs_c = GreedySearch(cpu, _Tok())
     text_c = gs_c.generate(input_ids=ids[0], max_length=8, chunk_size=64)[0].split()
     assert len(text_g) == len(text_c) == 8
     if text_g != text_c:                      # allowed only at a near-tie of the CPU model's logits
         first = next(i for i in range(8) if text_g[i] != text_c[i])
-        cpu2 = _models()[1]
+        cpu2 = _models(head_dim)[1]
         seq = torch.cat((ids, torch.tensor([[int(t) for t in text_c[:first]]], dtype=ids.dtype)), dim=1)
         with torch.inference_mode():
             logits = cpu2(input_ids=seq, use_cache=True, return_dict=True).logits[0, -1]

@@ -394,6 +394,38 @@ def test_pick_and_selection_ties_are_rare_and_within_their_rules(tmp_path):
     assert tot["tie_topk"] <= 0.02 * tot["selections"], tot
 
 
+@pytest.mark.parametrize("dim", [64, 32, 96])
+def test_heads_narrower_than_128_follow_the_oracle(dim):
+    """head_dim 64 (the reference's config/minicpm-inf-llm.yaml: 36 heads without GQA, n_local 2048), 32 and 96: the rows
+    travel through the 128-wide kernels with their two rotary halves at dimensions [0, D/2) and [64, 64 + D/2) and zeros
+    elsewhere.  Same acceptance as every stream: outputs, ordered selections, picks, representatives, residency
+    events, and the state that leaves through export_state / host_unit in the caller's width."""
+    if dim == 64:
+        kw = dict(n_init=128, n_local=2048, block_size=128, max_cached_block=32, topk=16, exc_block_size=512, repr_topk=4, dim=64)
+        T, calls, H, Hkv = 2048 + 128 + 24 * 128, [4096, 1024, 128], 36, 36
+        cm, ora, fol = compare(T, calls, H=H, Hkv=Hkv, base=1e4, seed=71, **kw)
+    else:
+        kw = dict(SMALL, dim=dim)
+        T, calls, H, Hkv = 1500, [700, 1, 1, 798], 8, 2
+        cm, ora, fol = compare(T, calls, H=H, Hkv=Hkv, base=1e4, seed=72 + dim, B=2, **kw)
+    assert cm.num_global_block > kw["topk"] and cm.dim_head == dim
+    q, k, v = make_stream(T, H, Hkv, 71 if dim == 64 else 72 + dim, B=1 if dim == 64 else 2, D=dim)
+    state = cm.export_state()
+    bs, n_init = kw["block_size"], kw["n_init"]
+    assert state["tail_k"].shape[-1] == dim and state["reps"].shape[-1] == H * dim
+    assert torch.equal(state["init_k"].cpu(), k[:, :, :n_init]) and torch.equal(state["tail_v"].cpu(), v[:, :, T - state["tail_v"].shape[2]:])
+    u = cm.num_global_block - 1
+    lo = n_init + u * bs
+    assert torch.equal(cm.host_unit(u)[:, 0], k[:, :, lo:lo + bs]) and torch.equal(cm.host_unit(u)[:, 1], v[:, :, lo:lo + bs])
+    # a fresh manager resumes from that state and continues bit for bit
+    q2, k2, v2 = make_stream(200, H, Hkv, 99, B=q.shape[0], D=dim)
+    qd, kd, vd = q2.cuda(), k2.cuda(), v2.cuda()
+    a = cm.append(qd, kd, vd, qd, kd, vd).cpu()
+    cm_b = new_manager(1e4, **kw).load_state(state)
+    b = cm_b.append(qd, kd, vd, qd, kd, vd).cpu()
+    assert a.shape[-1] == dim and torch.equal(a, b)
+
+
 def test_decode_steps_follow_oracle():
     """Single-token appends over a prepared memory (the decode shape): retrieval, fetch and attention per step."""
     calls = [1200] + [1] * 48

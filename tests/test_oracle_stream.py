@@ -358,3 +358,39 @@ def test_representatives_can_be_kept_in_the_model_dtype():
             assert torch.equal(rb, ra.bfloat16().float())
             same += 1
     assert same >= a.n_units // 2
+
+
+def test_mean_query_in_the_model_dtype_rarely_changes_a_selection():
+    """q_dtype=bfloat16 restates the reference's bf16 runs on the way to the mean query (context_manager.py:373-375:
+    rotated queries rounded to the model dtype, their mean rounded again); the HIP path keeps both in fp32, a
+    deliberate deviation towards the fp32 reference the acceptance is stated against.  How much it matters: unit scores
+    move by a few 1e-3 relative, so only selections with a near-tie at the k-th place can differ - bounded here at the
+    test geometry with mixture keys (clear gaps) and N(0,1) keys (crowded scores)."""
+    for seed, mixture, most in ((7, True, 0.05), (8, False, 0.25)):
+        g = torch.Generator().manual_seed(seed)
+        T = 1200
+        q, v = torch.randn(1, 4, T, 32, generator=g), torch.randn(1, 2, T, 32, generator=g)
+        if mixture:
+            means = torch.randn(2, 16, 32, generator=g)
+            comp = torch.randint(0, 16, (1, 2, T), generator=g)
+            k = torch.stack([means[h][comp[:, h]] for h in range(2)], dim=1) + 0.3 * torch.randn(1, 2, T, 32, generator=g)
+        else:
+            k = torch.randn(1, 2, T, 32, generator=g)
+        _, a = _run(q, k, v, [T])
+        seen = dict(blocks=0, differ=0)
+
+        def follow_a(block, row, scores):          # count, then adopt the fp32 run's selection: every block is judged on one history
+            mine, theirs = scores.topk(GEOM["topk"]), a.block_trace[block]
+            seen["blocks"] += 1
+            sa = theirs["unit_scores"][row]
+            assert float((sa - scores).abs().max()) <= 2e-2 * float(sa.abs().max())      # two bf16 roundings of the mean query
+            if set(mine.indices.tolist()) != set(theirs["selected"][row]):
+                seen["differ"] += 1
+                kth = float(sa.topk(GEOM["topk"]).values[-1])
+                for i in set(mine.indices.tolist()) ^ set(theirs["selected"][row]):
+                    assert abs(float(sa[i]) - kth) <= 2e-2 * float(sa.abs().max())         # only near the k-th place
+            return theirs["order"][row]
+
+        out_b, b = _run(q, k, v, [T], q_dtype=torch.bfloat16, topk_hook=follow_a)
+        assert seen["blocks"] >= 20 and [x["order"] for x in a.block_trace] == [x["order"] for x in b.block_trace]
+        assert seen["differ"] <= most * seen["blocks"], seen
