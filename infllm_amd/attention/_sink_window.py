@@ -17,6 +17,7 @@ fields (keys, values, tokens seen); a fourth holds the un-rotated sink keys when
 import torch
 
 from .. import ops
+from ._rows import check_head_dim, narrow, wide_inv_freq, widen
 from .dot_production_attention import get_multi_stage_dot_production_attention
 
 
@@ -25,10 +26,16 @@ def _heads(x, batch, length, heads, dim):
 
 
 def _rope_args(position_bias, device):
-    inv_freq = position_bias.inv_freq
-    if inv_freq.device != device or inv_freq.dtype != torch.float32:
-        inv_freq = inv_freq.to(device=device, dtype=torch.float32)
-    return inv_freq.contiguous(), float(position_bias.distance_scale)
+    return wide_inv_freq(position_bias.inv_freq, device), float(position_bias.distance_scale)
+
+
+def _rope(x, inv_freq, scale, pos0, consecutive=True):
+    """rows rotated at pos0 + r (or all at pos0); narrower heads take the way through a 128-wide row"""
+    d = x.shape[-1]
+    if d == ops.HEAD_DIM:
+        return ops.rope_rows(x, inv_freq, scale, pos0, consecutive)
+    check_head_dim(d)
+    return narrow(ops.rope_rows(widen(x, d), inv_freq, scale, pos0, consecutive), d).contiguous()
 
 
 def sink_window_forward(kind, n_local, n_init, fattn=False):
@@ -49,8 +56,8 @@ def sink_window_forward(kind, n_local, n_init, fattn=False):
 
         seen = past_key_value[2] if past_key_value is not None else 0
         len_k = seen + len_new
-        q_loc = ops.rope_rows(q, inv_freq, scale, len_k - len_q)
-        k_rot = ops.rope_rows(k, inv_freq, scale, seen)
+        q_loc = _rope(q, inv_freq, scale, len_k - len_q)
+        k_rot = _rope(k, inv_freq, scale, seen)
         v_all = v
         sinks = None
         if past_key_value is not None:
@@ -78,7 +85,7 @@ def sink_window_forward(kind, n_local, n_init, fattn=False):
         attn = Attn(q_loc.shape, q_loc.dtype, q_loc.device)
         attn.append(q_loc, k_rot[:, :, first:], v_all[:, :, first:], sliding_window=n_local)
         if len_k > n_local:
-            q_sink = ops.rope_rows(q, inv_freq, scale, sink_query_pos, consecutive=False)
+            q_sink = _rope(q, inv_freq, scale, sink_query_pos, consecutive=False)
             k_sink = sinks if raw_sinks and sinks is not None else k_rot[:, :, :n_init]
             v_sink = v_all[:, :, :n_init]
         else:
@@ -111,8 +118,8 @@ def causal_forward(fattn=False):
         inv_freq, scale = _rope_args(position_bias, q.device)
         seen = past_key_value[0].size(2) if past_key_value is not None else 0
         len_k = seen + len_new
-        q_rot = ops.rope_rows(q, inv_freq, scale, len_k - len_q)
-        k_rot = ops.rope_rows(k, inv_freq, scale, seen)
+        q_rot = _rope(q, inv_freq, scale, len_k - len_q)
+        k_rot = _rope(k, inv_freq, scale, seen)
         v_all = v.contiguous()
         if past_key_value is not None:
             k_rot = torch.cat((past_key_value[0], k_rot), dim=2)

@@ -39,26 +39,7 @@ from .. import _lib
 from .._lib import BackArgs, FrontArgs, LayerDesc, check
 from ..ops import HEAD_DIM, KEY_TILE
 
-
-# Heads narrower than the kernels' 128 dimensions (MiniCPM's 64, config/minicpm-inf-llm.yaml) run on the same kernels:
-# the two halves of a row go to dimensions [0, D/2) and [64, 64 + D/2) of a 128-wide row and the rest is zero.  RoPE
-# pairs dimension d with d + D/2 (rope.py:31-33), which are d and d + 64 in the wide row - the pairing the prologue
-# kernel uses - with zero frequencies in the unused slots; zeros add nothing to q.k, to the representatives' scores or
-# to the outputs, whose real dimensions are picked out again on the way back.  Twice the bytes and flops a kernel
-# built for 64 would need: a way to run such models, not a fast path.
-def _widen(t, d):
-    if d == HEAD_DIM:
-        return t
-    out = t.new_zeros(t.shape[:-1] + (HEAD_DIM,))
-    out[..., :d // 2] = t[..., :d // 2]
-    out[..., HEAD_DIM // 2:HEAD_DIM // 2 + d // 2] = t[..., d // 2:]
-    return out
-
-
-def _narrow(t, d):
-    if d == HEAD_DIM:
-        return t
-    return torch.cat((t[..., :d // 2], t[..., HEAD_DIM // 2:HEAD_DIM // 2 + d // 2]), dim=-1)
+from ._rows import check_head_dim, narrow as _narrow, wide_inv_freq, widen as _widen
 
 _SIDE_STREAM = None          # one process-wide side stream, like GLOBAL_STREAM (context_manager.py:193)
 _CALL_BUFFERS = {}           # (device, stream, geometry) -> the buffers of a call prepared in one go, see _bind_call_buffers
@@ -250,11 +231,10 @@ class ContextManager:
         self.pages_host = torch.empty((_PAGE_SLOTS * B * self.max_pages * page_bytes,), dtype=torch.uint8, pin_memory=True)
         self.max_carve = (exc + self.n_init) // bs + 2
         self.carve_stage = torch.empty((_CARVE_SLOTS, self.max_carve, B, 2, Hkv, bs, D), **bf)
-        inv_freq = self.position_embedding.inv_freq.to(device=dev, dtype=torch.float32)
-        if inv_freq.numel() != self.dim_head // 2:
-            raise ValueError(f"the rotary embedding is built for head_dim {2 * inv_freq.numel()}, the heads have {self.dim_head}")
-        self.inv_freq = torch.zeros((HEAD_DIM // 2,), dtype=torch.float32, device=dev)
-        self.inv_freq[:inv_freq.numel()] = inv_freq                # the slots of a narrow head's padding rotate by nothing
+        if self.position_embedding.inv_freq.numel() != self.dim_head // 2:
+            raise ValueError(f"the rotary embedding is built for head_dim {2 * self.position_embedding.inv_freq.numel()}, "
+                             f"the heads have {self.dim_head}")
+        self.inv_freq = wide_inv_freq(self.position_embedding.inv_freq, dev)
         self.slot_bytes = 2 * Hkv * bs * D * 2              # one unit of one batch row
         self.unit_bytes = B * self.slot_bytes               # one unit, all batch rows
 
@@ -634,8 +614,7 @@ class ContextManager:
             q, k, v = q.reshape(batch_size * heads, 1, input_length, -1), rep(k), rep(v)
         if not self.initialized:
             self.dim_head = q.size(3)
-            if self.dim_head > HEAD_DIM or self.dim_head % 2:
-                raise ValueError(f"head_dim must be even and at most {HEAD_DIM}, got {self.dim_head}")
+            check_head_dim(self.dim_head)
         if q.size(3) != self.dim_head:
             raise ValueError(f"head_dim changed from {self.dim_head} to {q.size(3)}")
         q, k, v = _widen(q, self.dim_head), _widen(k, self.dim_head), _widen(v, self.dim_head)
@@ -739,8 +718,7 @@ class ContextManager:
         cursor = init_len + n_units * self.block_size
         assert n_tail == T - cursor, f"tail holds {n_tail} tokens, the stream state needs {T - cursor}"
         assert state["init_k"].shape[2] == init_len and (n_units == 0 or state["units"].shape[0] == n_units)
-        if D > HEAD_DIM or D % 2:
-            raise ValueError(f"head_dim must be even and at most {HEAD_DIM}, got {D}")
+        check_head_dim(D)
         self.dim_head = D
         tail_k, tail_v = _widen(tail_k, D), _widen(tail_v, D)
         q_like = torch.empty((B, H, 1, HEAD_DIM), dtype=torch.bfloat16, device=tail_k.device)

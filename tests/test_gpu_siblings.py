@@ -63,6 +63,27 @@ def test_sink_window_types_follow_oracle(kind, calls, n_local, n_init):
     assert past[2] == T and past[0].shape[2] == min(T, n_local + n_init) == past[1].shape[2]     # stream_llm.py:43-52
 
 
+@pytest.mark.parametrize("kind", ["stream-llm", "infinite-lm", "origin"])
+def test_sibling_types_with_heads_of_64(kind, monkeypatch):
+    """head_dim 64 through the same three types: rows are widened for the kernels and cut back (attention/_rows.py)."""
+    import sys
+    from infllm_amd.attention import ATTN_FORWRAD
+    monkeypatch.setattr(sys.modules[__name__], "D", 64)
+    H, Hkv, calls, n_local, n_init = 4, 2, [300, 1, 1, 250], 128, 8
+    T = sum(calls)
+    xq, xk, xv = _stream(T, H, Hkv, seed=17, B=2)
+    fwd = ATTN_FORWRAD[kind](False) if kind == "origin" else ATTN_FORWRAD[kind](n_local, n_init, fattn=False)
+    got, past = _drive(fwd, xq, xk, xv, calls, H, Hkv, 1e4)
+    ora = CausalOracle(RopeOracle(64, base=1e4)) if kind == "origin" else SinkWindowOracle(RopeOracle(64, base=1e4), n_local, n_init, kind)
+    want, pos = [], 0
+    for L in calls:
+        sl = slice(pos, pos + L)
+        want.append(ora.append(_heads(xq[:, sl], H), _heads(xk[:, sl], Hkv), _heads(xv[:, sl], Hkv)))
+        pos += L
+    _check(got, torch.cat(want, dim=2))
+    assert past[0].shape[-1] == 64
+
+
 def test_origin_type_is_causal_attention():
     from infllm_amd.attention import ATTN_FORWRAD
     H, Hkv, calls = 4, 4, [200, 1, 1, 130]
