@@ -445,7 +445,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--tokens", type=int, default=131072)
     ap.add_argument("--chunk", type=int, default=8192, help="tokens per append() call")
     ap.add_argument("--cpu-tokens", type=int, default=16384, help="tokens of config 1 the CPU baseline runs (0 disables it)")

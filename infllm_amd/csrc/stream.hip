@@ -67,16 +67,12 @@ struct Layer {
     std::vector<uint32_t> efetch_engines;
     hsa_signal_t efetch_sig[2]{}, efetch_flag_sig[2]{};   // two sets, used in turn: a fetch may be issued while the one before is in flight
     bool efetch_prev_in_use = false;                   // the last fetch wrote only slots of the selection in use
-    bool efetch_overlap = true;                        // INFLLM_FETCH_OVERLAP=0: one fetch at a time
     uint32_t *d_efetch_flag = nullptr, *h_efetch_val = nullptr;
     int efetch_dev = 0;
     uint32_t off_engine = 0;                           // the engine that takes carved units to the host (0: the runtime's choice)
     uint32_t efetch_seq = 0;
     bool efetch_wait = false;
     int cur_n = 0;                                     // queries of the block in flight
-    bool local_pending = false;                        // the block's local stage has not been launched yet (block_back does it)
-    bool local_in_front = true;                        // the local stage is launched by block_front; INFLLM_FUSED_STAGES=1:
-                                                       // by block_back, in one launch with the global stage
     bool guessing = false;                             // the last selection settled a fetch made ahead of it
     // The fetch ahead of the selection (see infllm_block_prefetch): the candidates' host copy with the sequence number
     // the kernel publishes behind them, the selection whose global stage may still be running, and the guess in flight.
@@ -582,7 +578,6 @@ void efetch_setup(Layer *L) {
             return;
         L->h_efetch_val[kEfetchVals - 1] = 0;
     }
-    { const char *ov = getenv("INFLLM_FETCH_OVERLAP"); L->efetch_overlap = !(ov && ov[0] == '0'); }
     L->efetch_ok = true;
 }
 
@@ -605,11 +600,11 @@ int fetch_by_engines(Layer *L, int n_miss, const void *const *srcs, int64_t nbyt
     // taking its copies in the order they were issued, so the link does not idle between one fetch's landing and the
     // host's issue of the next; the host only makes sure that the fetch before the last has landed (whose signals this
     // one takes over).  Any other fetch lets everything land first.  Measured with the engines told apart (see
-    // efetch_setup): 43.1-43.6 ms per 128K stream against 43.7-43.8 with one fetch at a time (INFLLM_FETCH_OVERLAP=0);
+    // efetch_setup): 43.1-43.6 ms per 128K stream against 43.7-43.8 with one fetch at a time;
     // while the carved units' copy to the host still shared an engine with the fetch the overlap lost (the next
     // fetch's copies took bandwidth from the stragglers the stream was waiting for).
     const int set = (int)((L->efetch_seq + 1) & 1u);
-    int rc = L->efetch_overlap && ahead && L->efetch_prev_in_use ? efetch_wait_signal(L->efetch_flag_sig[set], "fetch") : efetch_wait_all(L, "fetch");
+    int rc = ahead && L->efetch_prev_in_use ? efetch_wait_signal(L->efetch_flag_sig[set], "fetch") : efetch_wait_all(L, "fetch");
     if (rc) return rc;
     const uint32_t seq = ++L->efetch_seq;
     uint32_t *val = L->h_efetch_val + (seq % (kEfetchVals - 1));
@@ -862,8 +857,6 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
     {
         const char *any = getenv("INFLLM_FETCH_AHEAD_ALWAYS");
         L->ahead_any_path = any && any[0] && any[0] != '0';
-        const char *fs = getenv("INFLLM_FUSED_STAGES");
-        L->local_in_front = !(fs && fs[0] && fs[0] != '0');
         const char *ns = getenv("INFLLM_NO_STAGING_COPY");
         L->stage_copy_ok = !(ns && ns[0] && ns[0] != '0');
         const char *pk = getenv("INFLLM_PAGE_TABLE_KERNEL");
@@ -1366,11 +1359,10 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     }
 
     // ---- local stage: causal sliding window over the ring.  Launched here, ahead of the host's wait for the selection
-    //      and of the stream's wait for the fetched units, both of which it covers.  With INFLLM_FUSED_STAGES=1
-    //      block_back launches it instead, in ONE launch with the global stage (measured: the launch is 6 us shorter than
-    //      the two and the merge reads half the partials, but the stream then reaches its wait for the fetch a local
-    //      stage earlier and idles longer than it saved - the missed units' way over PCIe takes 135 us of a 190 us block).
-    L->local_pending = !batched && !L->local_in_front;
+    //      and of the stream's wait for the fetched units, both of which it covers.  (Both stages of a block as ONE
+    //      launch behind that wait was measured: the launch is 6 us shorter than the two and the merge reads half the
+    //      partials, but the stream then reaches its wait for the fetch a local stage earlier and idles longer than it
+    //      saved.  infllm_attn_stages_fused remains an entry point of the library.)
     if (batched && ((a->b0 - L->batch_b0) / d.exc) % L->batch_group == 0) {
         // the local stage of this block and the next ones of its group in one launch (more queries per launch: fewer
         // key splits, fewer partial rows, the launch's fixed cost once); each block's partials go where its merge
@@ -1384,7 +1376,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
         timer_end(L, 0, ti, st);
         if (rc) return rc;
     }
-    if (!batched && L->local_in_front) {
+    if (!batched) {
         infllm_attn_args at = local_stage_args(L, a->n, a->b0, L->cur, splits_for(d, a->n, (int)((b1 - lo + kTile - 1) / kTile)));
         const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
         rc = infllm_attn_stage(&at, stream);
@@ -1839,27 +1831,12 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         }
     }
 
-    // ---- 3. the global stage and merge.  When block_front left the local stage to this call (INFLLM_FUSED_STAGES=1)
-    //         both stages are ONE launch over one list of tiles (ring tiles, then pages) behind the wait for the fetch -
-    //         for every block, not only those whose units are known to be in place: how the keys are cut into partials
-    //         then depends on the block alone, and with it every bit of the result.
+    // ---- 3. the global stage and merge (the local stage was launched by block_front or infllm_call_front)
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
     const int lin_tiles = (int)((b1 - lo + kTile - 1) / kTile);
     const int64_t part_o = (int64_t)d.B * d.H * a->n * kD, part_l = (int64_t)d.B * d.H * a->n;
-    const bool fuse = L->local_pending && n_pages > 0;
     int rc;
-    int sl = 0;
-    if (L->local_pending && !fuse) {
-        sl = splits_for(d, a->n, lin_tiles);
-        infllm_attn_args at = local_stage_args(L, a->n, a->b0, cur, sl);
-        const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo), st);
-        rc = infllm_attn_stage(&at, stream);
-        timer_end(L, 0, ti, st);
-        if (rc) return rc;
-    } else if (batched)
-        sl = cur.nsplit;                                  // launched by infllm_call_front, for the whole call
-    else if (!L->local_pending)
-        sl = splits_for(d, a->n, lin_tiles);              // launched by block_front
+    const int sl = batched ? cur.nsplit : splits_for(d, a->n, lin_tiles);       // key splits of the local stage's partials
     const int tw = L->fetch_wait || L->efetch_wait ? timer_begin(L, 2, a->n, a->n_miss, st) : -1;
     if (L->fetch_wait) {
         HIP_OK(hipStreamWaitEvent(st, L->fetch_done, 0), "block_back: wait fetch");
@@ -1879,28 +1856,15 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         at.cap = kTile;
         at.d_pages = d.d_pages; at.n_pages = n_pages;
         at.softmax_scale = d.softmax_scale;
-        if (fuse) {
-            const int ns = splits_for(d, a->n, lin_tiles + n_pages);
-            infllm_attn_args lt = local_stage_args(L, a->n, a->b0, cur, ns);
-            at.nsplit = ns;
-            at.d_o_part = d.d_o_part; at.d_lse_part = d.d_lse_part;
-            // timed as the block's dominant launch: its key count is the window plus the pages
-            const int ti = timer_begin(L, 0, a->n, (int)(b1 - lo) + n_pages * kTile, st);
-            rc = pages_inline ? infllm_attn_paged_inline(&lt, &at, inline_pages, stream) : infllm_attn_stages_fused(&lt, &at, stream);
-            timer_end(L, 0, ti, st);
-            if (rc) return rc;
-            parts = ns;
-        } else {
-            at.nsplit = splits_for(d, a->n, n_pages);
-            // behind the local stage's partials - unless those lie with the call's (then the merge takes two sets)
-            at.d_o_part = d.d_o_part + (batched ? 0 : sl * part_o);
-            at.d_lse_part = d.d_lse_part + (batched ? 0 : sl * part_l);
-            const int ti = timer_begin(L, 1, a->n, n_pages * kTile, st);
-            rc = pages_inline ? infllm_attn_paged_inline(nullptr, &at, inline_pages, stream) : infllm_attn_stage(&at, stream);
-            timer_end(L, 1, ti, st);
-            if (rc) return rc;
-            parts += at.nsplit;
-        }
+        at.nsplit = splits_for(d, a->n, n_pages);
+        // behind the local stage's partials - unless those lie with the call's (then the merge takes two sets)
+        at.d_o_part = d.d_o_part + (batched ? 0 : sl * part_o);
+        at.d_lse_part = d.d_lse_part + (batched ? 0 : sl * part_l);
+        const int ti = timer_begin(L, 1, a->n, n_pages * kTile, st);
+        rc = pages_inline ? infllm_attn_paged_inline(nullptr, &at, inline_pages, stream) : infllm_attn_stage(&at, stream);
+        timer_end(L, 1, ti, st);
+        if (rc) return rc;
+        parts += at.nsplit;
         // The next fetch (copy stream or DMA engines) must not overtake these reads.  While guesses are being settled
         // no event is needed for that: a fetch ahead never writes a slot of the selection in use, and a fetch behind
         // a selection is issued by a host that has read that selection, which the stream produced after this stage.
@@ -1911,7 +1875,6 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         } else
             L->global_unmarked = side || L->efetch_ok;
     }
-    L->local_pending = false;
     // Only the joint log-sum-exp is needed on the way to the next selection, and only by the small score launch of
     // step 4, which joins the partial values itself; the merge (output rows and the joint value for the bulk of the
     // scores) runs once that selection is out (step 5b).  The score-decay policy needs the joint value here.

@@ -101,11 +101,7 @@ def test_config2_stream_is_the_same_with_and_without_the_fetch_ahead(stream_128k
         return torch.cat(outs, dim=2), cm
 
     plain, cm0 = run(False)
-    monkeypatch.setenv("INFLLM_FETCH_OVERLAP", "0")               # one fetch at a time ...
-    serial, cm2 = run(True)
-    monkeypatch.delenv("INFLLM_FETCH_OVERLAP")                    # ... and the next one issued while the previous is in flight
     ahead, cm1 = run(True)
-    assert torch.equal(plain, serial) and cm0.stats == cm2.stats
     issued, confirmed = cm1.prefetch_stats()
     assert cm0.prefetch_stats() == (0, 0) and issued > 200 and issued // 2 < confirmed < issued
     assert cm1.staged_units() > 20       # wrong guesses are the blocks in which a just-carved unit is selected: those came from staging

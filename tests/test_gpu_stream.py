@@ -45,23 +45,6 @@ def test_local_stage_groups_of_other_sizes_follow_the_oracle(monkeypatch):
         assert cm.num_global_block > SMALL["topk"]
 
 
-def test_both_stages_in_one_launch_follow_the_oracle(monkeypatch):
-    """INFLLM_FUSED_STAGES=1 (with every block running its own local stage, call_tokens = 0): the local and the global
-    stage of every block as one launch over one list of tiles (infllm_attn_stages_fused) - same acceptance against the oracle, at the small and at the reference geometry, and
-    the same discrete trajectory as the two-launch order."""
-    from infllm_amd.attention import ContextManager
-    monkeypatch.delenv("INFLLM_CALL_TOKENS", raising=False)
-    monkeypatch.setattr(ContextManager, "call_tokens", 0)          # the one-launch form belongs to blocks that run on their own
-    monkeypatch.setenv("INFLLM_FUSED_STAGES", "1")
-    cm, _, _ = compare(1500, [700, 1, 1, 798], H=8, Hkv=2, base=1e4, seed=41, B=2, **SMALL)
-    assert cm.num_global_block > SMALL["topk"]
-    T = 4096 + 2048
-    cm1, _, _ = compare(T, [4096, 2048], H=32, Hkv=8, base=1e6, seed=42, **REFERENCE)
-    monkeypatch.delenv("INFLLM_FUSED_STAGES")
-    cm2, _, _ = compare(T, [4096, 2048], H=32, Hkv=8, base=1e6, seed=42, **REFERENCE)
-    assert [b["order"] for b in cm1.trace_blocks] == [b["order"] for b in cm2.trace_blocks] and cm1.stats == cm2.stats
-
-
 def test_page_table_in_the_launch_gives_the_bits_of_the_table_in_memory(monkeypatch):
     """The global stage reads its page table (selected units | init tokens | overflow rows of the ring) from the
     arguments of its own launch when the table has at most 64 entries; INFLLM_PAGE_TABLE_KERNEL=1 keeps the small
@@ -196,9 +179,8 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
         assert cm0.prefetch_stats() == (0, 0) and cm0.stats["misses"] > 0
         monkeypatch.setattr(ContextManager, "fetch_ahead", True)
         monkeypatch.setenv("INFLLM_FETCH_AHEAD_ALWAYS", "1")       # by default only the engines fetch ahead
-        for no_dma, overlap in (("0", "1"), ("0", "0"), ("1", "1")):
+        for no_dma in ("0", "1"):
             monkeypatch.setenv("INFLLM_NO_DMA_FETCH", no_dma)
-            monkeypatch.setenv("INFLLM_FETCH_OVERLAP", overlap)     # the next fetch issued while the previous one is in flight, or not
             ahead, cm1 = run_gpu(q, k, v, [1300, 1300], 1e4, **kw)
             issued, confirmed = cm1.prefetch_stats()
             assert issued > 0 and 0 <= confirmed <= issued
@@ -210,7 +192,6 @@ def test_fetch_ahead_of_the_selection_changes_nothing(monkeypatch):
                 assert cm0.policy[u].cached == cm1.policy[u].cached            # which slot a unit sits in may differ
                 assert sorted(cm1.policy[u].slot_of.values()) == sorted(set(cm1.policy[u].slot_of.values()))
         monkeypatch.delenv("INFLLM_NO_DMA_FETCH")
-        monkeypatch.delenv("INFLLM_FETCH_OVERLAP")
         monkeypatch.delenv("INFLLM_FETCH_AHEAD_ALWAYS")
     assert seen_confirmed > 0 and seen_refuted > 0          # both ways of settling a guess were exercised
 
