@@ -132,7 +132,7 @@ def hbm_leg(dev, n_units=8192, tables=8, launches=200):
                  "avg_launch_ms": us * 1e-3, "launches_timed": launches}
     us = _event_time_us(lambda i: ops.score_topk(reps[i % tables], n_units, qbar, 0, scores, None), launches, 2 * tables)
     scoring = _hbm_entry("unit_scores_rows_kernel<8, 2>", f"unit scores alone, {n_units} x {C} bf16, {tables} tables in rotation", nbytes, us,
-                         launches, traffic=counted_traffic("unit_scores__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"))
+                         launches, traffic=counted_traffic("retrieval__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"))
     return retrieval, scoring
 
 
@@ -289,7 +289,7 @@ def decode_workload(args, dev):
         "config": {"workload": f"config 3: {steps} single-token steps, {N} units x {bs} tokens, topk {topk}, n_local {n_local}, "
                                f"max_cached {KNOBS['max_cached_block']}"},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0,
-                     "traffic": counted_traffic("unit_scores__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"),
+                     "traffic": counted_traffic("retrieval__decode8192.hbm_bytes.txt", "unit_scores_traffic_bytes"),
                      "kernel": f"unit_scores_kernel ({N} x {H * D} bf16 representatives, {N * H * D * 2 / 2 ** 20:.1f} MiB per retrieval)",
                      "avg_launch_ms": ms},
         "cache": cm.stats}))
@@ -451,9 +451,9 @@ def main():
     ap.add_argument("--cpu-tokens", type=int, default=16384, help="tokens of config 1 the CPU baseline runs (0 disables it)")
     ap.add_argument("--no-hbm-leg", action="store_true", help="skip the HBM-bound kernels' measurements (roofline_hbm, kernels_hbm)")
     ap.add_argument("--no-extra-legs", action="store_true", help="skip the all-resident, decode (config 3) and 1M-token (config 5) legs")
-    ap.add_argument("--workload", choices=["prefill", "decode", "model"], default="prefill",
-                    help="prefill = the headline 128K-token stream (config 2); decode = config 3, model = config 4 "
-                         "(each with its own JSON line)")
+    ap.add_argument("--workload", choices=["prefill", "decode", "model", "hbm"], default="prefill",
+                    help="prefill = the headline 128K-token stream (config 2); decode = config 3, model = config 4, "
+                         "hbm = the HBM-bound kernels' legs alone (each with its own JSON line)")
     ap.add_argument("--model-layers", type=int, default=32)
     ap.add_argument("--model-tokens", type=int, default=131072)
     ap.add_argument("--model-decode-steps", type=int, default=128)
@@ -485,6 +485,10 @@ def main():
         return
     if args.workload == "model":
         model_workload(args, dev)
+        return
+    if args.workload == "hbm":
+        retrieval, scoring = hbm_leg(dev)
+        print(json.dumps({"roofline_hbm": retrieval, "kernels_hbm": [scoring] + kernels_hbm_leg(dev)}))
         return
     T = args.tokens
     q, k, v = make_stream(T, 0, dev, args.favour)
