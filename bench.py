@@ -157,7 +157,8 @@ def kernels_hbm_leg(dev):
     us = _event_time_us(lambda i: ops.ingest(q, k, v, 100000 + i * n, n_local - 1, inv_freq, 1.0, *rings, ring_score, q_loc, q_glb, qpart), 20, 3)
     per_token = (H + 2 * HKV) * D * 2 + 2 * H * D * 2 + 3 * HKV * D * 2
     out.append(_hbm_entry("ingest_kernel", f"prologue of an {n}-token append() call: reads q, k, v, writes both rotated q and three ring rows "
-                                           f"({per_token} B per token)", n * per_token, us, 20))
+                                           f"({per_token} B per token)", n * per_token, us, 20,
+                          traffic=counted_traffic("retrieval__decode8192.hbm_bytes.txt", "ingest_traffic_bytes")))
     del q, k, v, q_loc, q_glb, qpart
     # ---- representatives of the units a block carves (context_manager.py:268-277) and their rows out of the rings
     n_units = exc // bs
@@ -167,7 +168,7 @@ def kernels_hbm_leg(dev):
     per_unit = H * bs * 4 + H * KNOBS["repr_topk"] * D * 2 + H * D * 2
     out.append(_hbm_entry("repr_keys_kernel", f"representatives of the {n_units} units of a block: scores, {KNOBS['repr_topk']} gathered keys per head, "
                                               f"one row out ({per_unit} B per unit); a chain of dependent arg-max steps, latency-bound",
-                          n_units * per_unit, us, 200))
+                          n_units * per_unit, us, 200, traffic=counted_traffic("retrieval__decode8192.hbm_bytes.txt", "repr_keys_traffic_bytes")))
     stage = torch.empty((n_units, 1, 2, HKV, bs, D), **bf)
 
     def gather(i):
@@ -177,7 +178,9 @@ def kernels_hbm_leg(dev):
     unit_bytes = 2 * HKV * bs * D * 2
     us = _event_time_us(gather, 200, 10)
     out.append(_hbm_entry("gather_rows_kernel x2", f"K and V rows of a block's {n_units} carved units, ring -> staging ({unit_bytes} B per unit, "
-                                                   "read and written once)", n_units * unit_bytes, us, 200))
+                                                   "read and written once; two launches of 3 us whose event-timed mean is mostly launch gap; in the stream "
+                                                   "this copy rides in the repr_keys launch)", n_units * unit_bytes, us, 200,
+                          traffic=counted_traffic("retrieval__decode8192.hbm_bytes.txt", "gather_rows_traffic_bytes")))
     # ---- decode-shaped attention (config 3): one query per head over the window and the retrieved units, both stages + merge
     sets, n_glob = 12, topk * bs + n_init + 64
     ns_l, ns_g = 32, (n_glob // 64) // 2
@@ -208,7 +211,8 @@ def kernels_hbm_leg(dev):
     nbytes = (n_local + 1 + n_glob) * HKV * D * 2 * 2
     out.append(_hbm_entry("attn_stage_kernel<0> + <1> + attn_merge_wide_kernel", f"decode-shaped attention: 1 query x {H} heads over {n_local + 1} window keys "
                           f"({ns_l} key splits) and {n_glob} retrieved keys ({ns_g} splits), K and V read once, three launches; "
-                          f"{sets} K/V sets in rotation", nbytes, us, 200))
+                          f"{sets} K/V sets in rotation", nbytes, us, 200,
+                          traffic=counted_traffic("retrieval__decode8192.hbm_bytes.txt", "decode_attention_traffic_bytes")))
     return out
 
 
