@@ -507,6 +507,11 @@ typedef struct {
     int32_t *h_n_evicted, *h_n_miss;                  /* out, optional: [B] */
 } infllm_select_args;
 int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, void *copy_stream);
+/* The ids the last infllm_block_select worked on ([B, n_sel], the order it read them in), from the library's own
+ * copy: the pinned ids themselves are overwritten by the next selection as soon as infllm_block_back has been
+ * enqueued, so a caller that wants them afterwards (the lru-s scores of `selected_block`, context_manager.py:529-543;
+ * traces) reads them here.  Returns the number of ids written (<= capacity) or an error (< 0). */
+int infllm_layer_last_selection(void *layer, int32_t *ids, int32_t capacity);
 /* The fetch ahead of the selection.  infllm_block_front ranks the units that exist before its block for the NEXT
  * block already (the selection proper, late in infllm_block_back, only weighs these candidates against the units
  * carved in between) and publishes them to the host.  Called after infllm_block_back, this runs the residency

@@ -178,6 +178,7 @@ SYMBOLS = {
     "infllm_block_select": (c_i32, [c_vp, C.POINTER(SelectArgs), c_vp, c_vp]),
     "infllm_block_prefetch": (c_i32, [c_vp, C.POINTER(SelectArgs), c_vp, c_vp]),
     "infllm_layer_prefetch_stats": (c_i32, [c_vp, c_vp, c_vp]),
+    "infllm_layer_last_selection": (c_i32, [c_vp, c_vp, c_i32]),
     "infllm_layer_timing": (c_i32, [c_vp, c_i32, c_i32]),
     "infllm_layer_read_timing": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32]),
 }

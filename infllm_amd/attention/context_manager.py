@@ -497,8 +497,12 @@ class ContextManager:
             rc = lib.infllm_block_back(layer, self._ba_ref, self._main_raw, self._copy_raw)
             if rc:
                 check(rc, "infllm_block_back")
-            if selected is None:
-                selected = self.topk_idx_host.tolist()
+            if selected is None and (self.record_trace or self.cache_strategy == "lru-s"):
+                # from the library's copy: the pinned ids belong to the next selection once the second half is enqueued
+                got = lib.infllm_layer_last_selection(layer, self._sel_ids, len(self._sel_ids))
+                if got != B * n_sel:
+                    check(min(got, -1), "infllm_layer_last_selection")
+                selected = [self._sel_ids[u * n_sel:(u + 1) * n_sel] for u in range(B)]
             stats["evictions"] += sum(self._n_evicted[:B])
             for u in range(B):
                 if self.policy[u].evicted_log is not None:

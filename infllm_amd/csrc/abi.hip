@@ -77,14 +77,8 @@ __global__ __launch_bounds__(256) void unit_fetch_kernel(FetchList list, int n_u
     }
 }
 
-int env_int(const char *name, int fallback) {
-    const char *e = getenv(name);
-    const int v = e ? atoi(e) : 0;
-    return v > 0 ? v : fallback;
-}
-int fetch_workgroups() { static int n = env_int("INFLLM_FETCH_WGS", 128); return n; }
-int fetch_threads() { static int n = env_int("INFLLM_FETCH_THREADS", 64); return n == 128 || n == 256 ? n : 64; }
-int fetch_unroll() { static int n = env_int("INFLLM_FETCH_UNROLL", 1); return n == 2 || n == 4 ? n : 1; }
+// launch shape of the zero-copy fetch (see the kernel's comment)
+constexpr int kFetchWorkgroups = 128, kFetchThreads = 64;
 
 }  // namespace
 
@@ -102,12 +96,10 @@ extern "C" int infllm_fetch_units(const void *const *h_src, void *const *d_dst, 
             list.src[i] = (const uint4 *)h_src[first + i];
             list.dst[i] = (uint4 *)d_dst[first + i];
         }
-        const int threads = fetch_threads(), unroll = fetch_unroll();
-        const int64_t piece = (int64_t)threads * unroll * 16;
+        const int64_t piece = (int64_t)kFetchThreads * 16;
         const int64_t work = (int64_t)m * ((nbytes + piece - 1) / piece);
-        const int wgs = work < fetch_workgroups() ? (int)work : fetch_workgroups();
-        auto kern = unroll == 1 ? unit_fetch_kernel<1> : unroll == 2 ? unit_fetch_kernel<2> : unit_fetch_kernel<4>;
-        hipLaunchKernelGGL(kern, dim3(wgs), dim3(threads), 0, (hipStream_t)stream, list, m, nbytes);
+        const int wgs = work < kFetchWorkgroups ? (int)work : kFetchWorkgroups;
+        hipLaunchKernelGGL(unit_fetch_kernel<1>, dim3(wgs), dim3(kFetchThreads), 0, (hipStream_t)stream, list, m, nbytes);
         INFLLM_CHECK_LAUNCH("unit_fetch");
     }
     return 0;

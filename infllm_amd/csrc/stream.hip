@@ -1570,6 +1570,15 @@ extern "C" int infllm_layer_prefetch_stats(void *layer, int64_t *issued, int64_t
     return 0;
 }
 
+extern "C" int infllm_layer_last_selection(void *layer, int32_t *ids, int32_t capacity) {
+    INFLLM_REQUIRE(layer && (ids || capacity == 0) && capacity >= 0, "layer_last_selection: bad arguments");
+    Layer *L = (Layer *)layer;
+    const int64_t n = (int64_t)L->last_sel.size();
+    INFLLM_REQUIRE(n <= capacity, "layer_last_selection: %lld ids do not fit %d", (long long)n, capacity);
+    if (n) std::memcpy(ids, L->last_sel.data(), sizeof(int32_t) * n);
+    return (int)n;
+}
+
 extern "C" int infllm_block_select(void *layer, const infllm_select_args *a, void *stream, void *copy_stream) {
     INFLLM_REQUIRE(layer && a, "block_select: null argument");
     Layer *L = (Layer *)layer;
