@@ -387,6 +387,13 @@ typedef struct {
     int64_t unit_scores_sb;
     const void *d_q_next, *d_k_next, *d_v_next;       /* rows of the next block (same strides), or NULL */
     int32_t n_next, flags;                            /* INFLLM_NO_RETRIEVAL: the caller supplies the selection */
+    /* infllm_call_front only, optional: [ceil(n / exc), B, call_scores_cols] floats, call_scores_cols >= n_units + the
+     * units the call can carve.  Given, the k best of the units that exist now are chosen for every block of the call
+     * in one go (VectorTensor.get_topk, context_manager.py:159-163, once per call instead of once per block); a
+     * block's selection then only weighs its list against the units carved since the call began - the same ids in
+     * the same order.  The buffer is in use until the call's last infllm_block_back. */
+    float *d_call_scores;
+    int64_t call_scores_cols;
 } infllm_front_args;
 int infllm_block_front(void *layer, const infllm_front_args *a, void *stream);
 
@@ -401,7 +408,8 @@ int infllm_block_front(void *layer, const infllm_front_args *a, void *stream);
  *   infllm_call_front       a->d_q/d_k/d_v are the rows of the next a->n <= max_tokens tokens (a->b0 the first one's
  *                           position); runs the prologue for all of them (the rings must have room: ring_cap >=
  *                           a->b0 - cursor + a->n), every block's mean query, the first block's retrieval when
- *                           a->n_units > topk.  The blocks then go through infllm_block_front / select / back as
+ *                           a->n_units > topk (and, with a->d_call_scores, the lists of the other blocks'
+ *                           selections, see there).  The blocks then go through infllm_block_front / select / back as
  *                           ever, in order; block_front finds their prologue done (its d_q / d_k / d_v and
  *                           next-block pointers are not read, n_next still says whether a block of this call
  *                           follows) and launches the local stage for group_blocks blocks at a time, at the first
@@ -541,9 +549,11 @@ int64_t infllm_layer_staged_units(void *layer);
  * page tables of the global stage (get_global_hidden_and_mask, context_manager.py:386-451) carried in the stage's own
  * launch, [1] written to device memory by the table kernel, [2] uploaded from the host; [3] merges of a block's partial
  * outputs (torch_impl.py:15-36) carried by the block's local-score launch, [4] launched on their own in a block whose
- * order of launches allowed the carried form.  INFLLM_PAGE_TABLE_KERNEL=1 and INFLLM_SCORE_MERGE_APART=1, read by
- * infllm_layer_create, move blocks from [0] to [1] and from [3] to [4]. */
-int infllm_layer_path_counts(void *layer, int64_t *counts /* [5] */);
+ * order of launches allowed the carried form; [5] selections ranked from the lists of a prepared call
+ * (infllm_front_args.d_call_scores) instead of a pass over all units.  INFLLM_PAGE_TABLE_KERNEL=1,
+ * INFLLM_SCORE_MERGE_APART=1 and INFLLM_NO_CALL_LISTS=1, read by infllm_layer_create, move blocks from [0] to [1],
+ * from [3] to [4] and out of [5]. */
+int infllm_layer_path_counts(void *layer, int64_t *counts /* [6] */);
 /* Units moved from pinned host memory to the slab so far, whichever way (DMA engines or the fetch kernel): the misses
  * of the selections, the candidates a guess fetched that were not selected after all, and what a wrong guess's
  * repair brought back - the host-to-device traffic of MemoryUnit.load (context_manager.py:76-91) in units. */

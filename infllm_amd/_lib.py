@@ -88,6 +88,7 @@ class FrontArgs(C.Structure):
         ("d_reps", c_vp), ("rep_sb", c_i64), ("rep_su", c_i64),
         ("d_unit_scores", c_vp), ("unit_scores_sb", c_i64),
         ("d_q_next", c_vp), ("d_k_next", c_vp), ("d_v_next", c_vp), ("n_next", c_i32), ("flags", c_i32),
+        ("d_call_scores", c_vp), ("call_scores_cols", c_i64),
     ]
 
 

@@ -153,6 +153,7 @@ class ContextManager:
         self.load_count = 0
         self.record_trace = False
         self.trace_blocks, self.trace_units = [], []
+        self._call_scores = None      # [blocks of a call, B, units]: scores of every unit under every block's mean query
         self.stats = dict(blocks=0, hits=0, misses=0, evictions=0)
         self._layer = None
         self._timing_cap, self._timing_stride = 0, 1
@@ -398,10 +399,11 @@ class ContextManager:
 
     def path_counts(self):
         """Which interchangeable paths this layer's blocks took (infllm_layer_path_counts)."""
-        counts = (ctypes.c_int64 * 5)()
+        counts = (ctypes.c_int64 * 6)()
         if self._layer:
             check(self._lib.infllm_layer_path_counts(self._layer, counts), "infllm_layer_path_counts")
-        return dict(zip(("tables_inline", "tables_kernel", "tables_upload", "score_merged", "score_apart"), (int(c) for c in counts)))
+        return dict(zip(("tables_inline", "tables_kernel", "tables_upload", "score_merged", "score_apart", "call_ranked"),
+                        (int(c) for c in counts)))
 
     def fetched_units(self):
         """Units moved from pinned host memory to the device cache so far (wrongly guessed ones and repairs included)."""
@@ -667,6 +669,12 @@ class ContextManager:
                                               self._v_ptr + st * self._v_step)
                     fa.n, fa.n_units, fa.b0 = call_end - st, self.num_global_block, self.length + st
                     fa.flags = _lib.NO_RETRIEVAL if use_chunks else 0
+                    # room for every block's scores of the units there are and of those the call can carve
+                    blocks, cols = -(-self._call_tokens // exc), self.num_global_block + (call_end - st) // self.block_size + 2
+                    if self._call_scores is None or self._call_scores.shape[2] < cols or self._call_scores.shape[0] < blocks:
+                        cols = max(-(-cols // 256) * 256, 2 * (self._call_scores.shape[2] if self._call_scores is not None else 0))
+                        self._call_scores = torch.empty((blocks, self.num_units, cols), dtype=torch.float32, device=self.device)
+                    fa.d_call_scores, fa.call_scores_cols = self._call_scores.data_ptr(), self._call_scores.shape[2]
                     check(self._lib.infllm_call_front(self._layer, self._fa_ref, self._main_raw), "infllm_call_front")
             elif not self._call_tokens:
                 call_end = input_length

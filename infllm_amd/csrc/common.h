@@ -134,3 +134,27 @@ __device__ __forceinline__ void merge_piece(const MergeJob &mj, int64_t e) {
     *(u32x4 *)(mj.out + (int64_t)b * mj.o_sb + (int64_t)h * mj.o_sh + (int64_t)i * mj.o_sl + c * 8) = packed;
     if (c == 0 && mj.lse_out) mj.lse_out[row] = den > 0.f ? m + log2f(den) : -INFINITY;
 }
+
+
+// ---- a call's selections from lists made once per call (retrieve.hip: call_rank_kernel; stream.hip drives it)
+// For every later block of a prepared call the k best of the units that existed when the call began are known
+// (`base`), and so are those units' scores under the block's mean query (`scores`).  After a block has carved
+// n_new units, workgroup x of one launch scores them under the mean query of block j0 + x and, for the two blocks
+// that need a list now, ranks the base list against all the units carved since the call began.
+struct CallRankJob {
+    const bf16_t *reps;                // [B][units][C] representatives
+    int64_t rep_sb, rep_su;
+    const float *qbars;                // [blocks][B][C] mean queries of the call's blocks
+    float *scores;                     // [blocks][B][cols]
+    int64_t cols;
+    const int32_t *base;               // [blocks][B][k]
+    int32_t B, k;
+    int32_t n_base;                    // units that existed when the call began
+    int32_t first_new, n_new;          // the units carved just now: [first_new, first_new + n_new)
+    int32_t j0;                        // workgroup x works for block j0 + x
+    int32_t j_sel, j_cand;             // blocks whose selection / candidate list leaves now (-1: none)
+    int32_t *sel_out, *sel_flag;       // [B][k] ids, then the sequence number
+    int32_t sel_seq;
+    int32_t *cand_out, *cand_flag;
+    int32_t cand_seq;
+};

@@ -50,8 +50,10 @@ __global__ __launch_bounds__(256) void unit_scores_kernel(const bf16_t *reps, in
 // that all waves of the chip stream disjoint rows at once.
 template <int CPL, int ROWS>
 __global__ __launch_bounds__(256) void unit_scores_rows_kernel(const bf16_t *reps, int64_t rep_stride, int N,
-                                                                const float *qbar, float *scores) {
+                                                                const float *qbar, float *scores, int64_t qbar_ys, int64_t scores_ys) {
     extern __shared__ float qs[];
+    qbar += blockIdx.y * qbar_ys;                               // blockIdx.y: one of several queries over the same rows
+    scores += blockIdx.y * scores_ys;
     constexpr int C = CPL * 512;
     const int lane = threadIdx.x & 63;
     const int waves_per_wg = blockDim.x >> 6;
@@ -104,14 +106,16 @@ __global__ __launch_bounds__(256) void unit_scores_rows_kernel(const bf16_t *rep
 // At most 512 workgroups (two per CU, all resident at once: a second round of workgroups costs more than
 // it gains); long tables keep two rows per wave in flight.
 template <int CPL>
-void launch_unit_scores_rows(const bf16_t *reps, int64_t rep_stride, int N, const float *qbar, float *scores, hipStream_t st) {
+void launch_unit_scores_rows(const bf16_t *reps, int64_t rep_stride, int N, const float *qbar, float *scores, hipStream_t st,
+                             int n_queries = 1, int64_t qbar_ys = 0, int64_t scores_ys = 0) {
     constexpr int kRowsDeep = CPL <= 8 ? 2 : 1;
     const bool deep = kRowsDeep > 1 && N >= 4096;
     const int per_wg = 4 * (deep ? kRowsDeep : 1);
     int wgs = (N + per_wg - 1) / per_wg;
     if (wgs > 512) wgs = 512;
     auto kern = deep ? unit_scores_rows_kernel<CPL, kRowsDeep> : unit_scores_rows_kernel<CPL, 1>;
-    hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), (size_t)CPL * 512 * sizeof(float), st, reps, rep_stride, N, qbar, scores);
+    hipLaunchKernelGGL(kern, dim3(wgs, n_queries), dim3(256), (size_t)CPL * 512 * sizeof(float), st, reps, rep_stride, N, qbar, scores,
+                       qbar_ys, scores_ys);
 }
 
 // ---------------------------------------------------------------- top-k (radix select)
@@ -177,7 +181,10 @@ __device__ __forceinline__ void emit_descending(const int32_t *sel_id, const uin
 }
 
 __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *idx_out2,
-                                                           int32_t *flag, int32_t flag_value) {
+                                                           int32_t *flag, int32_t flag_value, int64_t scores_xs, int64_t idx_xs) {
+    scores += blockIdx.x * scores_xs;                           // blockIdx.x: one of several tables
+    idx_out += blockIdx.x * idx_xs;
+    if (idx_out2) idx_out2 += blockIdx.x * idx_xs;
     __shared__ int hist[256];
     __shared__ int wave_tot[kSelThreads / 64];
     __shared__ int32_t sel_id[kSelThreads];
@@ -238,7 +245,10 @@ __global__ __launch_bounds__(kSelThreads) void topk_kernel(const float *scores, 
 // Output contract as above: lowest indices among keys equal to the k-th; ids leave in descending score.
 template <int R>
 __global__ __launch_bounds__(kSelThreads) void topk_regs_kernel(const float *scores, int N, int k, int32_t *idx_out, int32_t *idx_out2,
-                                                                int32_t *flag, int32_t flag_value) {
+                                                                int32_t *flag, int32_t flag_value, int64_t scores_xs, int64_t idx_xs) {
+    scores += blockIdx.x * scores_xs;                           // blockIdx.x: one of several tables
+    idx_out += blockIdx.x * idx_xs;
+    if (idx_out2) idx_out2 += blockIdx.x * idx_xs;
     __shared__ __align__(16) int hist[4096];
     __shared__ int wave_tot[kSelThreads / 64];
     __shared__ uint32_t sh_prefix;
@@ -717,14 +727,14 @@ int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_
     return infllm_topk_publish_pair(d_scores, N, k, d_idx, nullptr, d_flag, flag_value, stream);
 }
 
-// ... with a second copy of the ids in d_idx2 (may be NULL)
-int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag,
-                             int32_t flag_value, void *stream) {
+// the selection over `tables` tables of N scores each (scores_xs apart), table t's ids to d_idx + t * idx_xs
+static int launch_topk(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag, int32_t flag_value,
+                       int tables, int64_t scores_xs, int64_t idx_xs, void *stream) {
     INFLLM_REQUIRE(d_scores && d_idx, "topk: null pointer");
-    INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && k <= 1024, "topk: k=%d with N=%d", k, N);
+    INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && k <= 1024 && tables >= 1, "topk: k=%d with N=%d, %d tables", k, N, tables);
     const hipStream_t st = (hipStream_t)stream;
     switch (N <= 16384 ? (N + kSelThreads - 1) / kSelThreads : 0) {       // keys per thread
-#define REGS_CASE(r) hipLaunchKernelGGL(topk_regs_kernel<r>, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_idx2, d_flag, flag_value); break
+#define REGS_CASE(r) hipLaunchKernelGGL(topk_regs_kernel<r>, dim3(tables), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_idx2, d_flag, flag_value, scores_xs, idx_xs); break
     case 1: REGS_CASE(1);
     case 2: REGS_CASE(2);
     case 3: REGS_CASE(3);
@@ -735,10 +745,16 @@ int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_
     case 11: case 12: REGS_CASE(12);
     case 13: case 14: case 15: case 16: REGS_CASE(16);
 #undef REGS_CASE
-    default: hipLaunchKernelGGL(topk_kernel, dim3(1), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_idx2, d_flag, flag_value);
+    default: hipLaunchKernelGGL(topk_kernel, dim3(tables), dim3(kSelThreads), 0, st, d_scores, N, k, d_idx, d_idx2, d_flag, flag_value, scores_xs, idx_xs);
     }
     INFLLM_CHECK_LAUNCH("topk");
     return 0;
+}
+
+// ... with a second copy of the ids in d_idx2 (may be NULL)
+int infllm_topk_publish_pair(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag,
+                             int32_t flag_value, void *stream) {
+    return launch_topk(d_scores, N, k, d_idx, d_idx2, d_flag, flag_value, 1, 0, 0, stream);
 }
 
 // internal: see topk_merge_kernel
@@ -781,6 +797,123 @@ extern "C" int infllm_score_new_topk(const void *d_reps, int64_t rep_stride, int
     return rc == 1 ? infllm_fail(-1, "score_new_topk: rows of %d elements (supported: 512, 1024, 2048, 4096)", C) : rc;
 }
 
+
+// ---------------------------------------------------------------- a call's selections from lists made once per call
+// (see CallRankJob in common.h).  Scoring is unit_scores_rows_kernel's arithmetic, term by term; the ranking orders
+// base list and new units by (score, lower id first) as every selection here does, so the list that leaves is the
+// one a selection over all units would give: a unit of the overall top-k that existed when the call began is among
+// the k best of the units of that time.
+constexpr int kCallRankEntries = 256;      // base list + units carved since the call began
+constexpr int kCallRankNew = 64;           // units carved by one block
+
+template <int CPL>
+__global__ __launch_bounds__(256) void call_rank_kernel(CallRankJob jb) {
+    __shared__ float fresh[kCallRankNew];
+    __shared__ uint32_t e_key[kCallRankEntries];
+    __shared__ int32_t e_id[kCallRankEntries];
+    constexpr int C = CPL * 512;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = jb.j0 + (int)blockIdx.x;
+    const bool is_sel = j == jb.j_sel, is_cand = j == jb.j_cand;
+    for (int u = 0; u < jb.B; ++u) {
+        const float *qbar = jb.qbars + ((int64_t)j * jb.B + u) * C;
+        float *scores = jb.scores + ((int64_t)j * jb.B + u) * jb.cols;
+        if (jb.n_new > 0) {
+            float q[CPL][8];
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) {
+                const f32x4 lo = *(const f32x4 *)(qbar + c * 512 + lane * 8), hi = *(const f32x4 *)(qbar + c * 512 + lane * 8 + 4);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) q[c][i] = lo[i], q[c][4 + i] = hi[i];
+            }
+            for (int r = wave; r < jb.n_new; r += 4) {
+                const bf16_t *row = jb.reps + (int64_t)u * jb.rep_sb + (int64_t)(jb.first_new + r) * jb.rep_su + lane * 8;
+                u32x4 w[CPL];
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) w[c] = *(const u32x4 *)(row + c * 512);
+                float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc0 += bf16_bits_to_f32(w[c][i] & 0xffffu) * q[c][2 * i];
+                        acc1 += bf16_bits_to_f32(w[c][i] >> 16) * q[c][2 * i + 1];
+                    }
+                }
+                const float acc = wave_sum(acc0 + acc1);
+                if (lane == 0) {
+                    scores[jb.first_new + r] = acc;
+                    fresh[r] = acc;
+                }
+            }
+        }
+        if (!is_sel && !is_cand) continue;                       // workgroup-uniform
+        __syncthreads();
+        const int n_late = jb.first_new + jb.n_new - jb.n_base;  // units carved since the call began
+        const int n = jb.k + n_late;
+        if (tid < n) {
+            const int id = tid < jb.k ? jb.base[((int64_t)j * jb.B + u) * jb.k + tid] : jb.n_base + (tid - jb.k);
+            e_id[tid] = id;
+            e_key[tid] = order_key(id >= jb.first_new ? fresh[id - jb.first_new] : scores[id]);
+        }
+        __syncthreads();
+        if (tid < n) {
+            const uint32_t key = e_key[tid];
+            const int id = e_id[tid];
+            int rank = 0;
+            for (int e = 0; e < n; ++e) {
+                const uint32_t ke = e_key[e];
+                const int ide = e_id[e];
+                rank += (ke > key || (ke == key && ide < id)) ? 1 : 0;
+            }
+            if (rank < jb.k) (is_sel ? jb.sel_out : jb.cand_out)[(int64_t)u * jb.k + rank] = id;
+        }
+        __syncthreads();                                         // fresh / e_key / e_id are rewritten for the next row
+    }
+    if (is_sel) publish(jb.sel_flag, jb.sel_seq);
+    else if (is_cand) publish(jb.cand_flag, jb.cand_seq);
+}
+
+// library-internal: launches call_rank_kernel for n_wgs blocks of the call from job->j0 on.  Returns 1, with nothing
+// launched, where the kernel does not apply (row lengths other than 512 * {1, 2, 4, 8}, lists that do not fit).
+int infllm_call_rank(const CallRankJob *job, int32_t C, int32_t n_wgs, void *stream) {
+    INFLLM_REQUIRE(job && job->reps && job->qbars && job->scores && job->base, "call_rank: null pointer");
+    INFLLM_REQUIRE(n_wgs >= 1 && job->B >= 1 && job->k >= 1 && job->n_new >= 0 && job->n_base >= job->k && job->first_new >= job->n_base,
+                   "call_rank: bad job");
+    INFLLM_REQUIRE(job->first_new + job->n_new <= job->cols, "call_rank: %d units do not fit score rows of %lld", job->first_new + job->n_new,
+                   (long long)job->cols);
+    INFLLM_REQUIRE(job->j_sel < 0 || job->sel_out, "call_rank: no place for the selection");
+    INFLLM_REQUIRE(job->j_cand < 0 || job->cand_out, "call_rank: no place for the candidates");
+    if (job->n_new > kCallRankNew || job->k + (job->first_new + job->n_new - job->n_base) > kCallRankEntries) return 1;
+    switch (C % 512 == 0 ? C / 512 : 0) {
+#define CALL_RANK_CASE(n) case n: hipLaunchKernelGGL(call_rank_kernel<n>, dim3(n_wgs), dim3(256), 0, (hipStream_t)stream, *job); break
+        CALL_RANK_CASE(1); CALL_RANK_CASE(2); CALL_RANK_CASE(4); CALL_RANK_CASE(8);
+#undef CALL_RANK_CASE
+    default: return 1;
+    }
+    INFLLM_CHECK_LAUNCH("call_rank");
+    return 0;
+}
+int infllm_call_rank_room() { return kCallRankEntries; }
+
+// library-internal: the k best of the same N units under each of n_queries queries (context_manager.py:159-163 for
+// several blocks of a call at once): query q's scores go to d_scores + q * scores_qs, its ids to d_idx + q * idx_qs.
+// Returns 1, with nothing launched, for row lengths other than 512 * {1, 2, 4, 8}.
+int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbars, int64_t qbar_qs,
+                              int32_t n_queries, int32_t k, float *d_scores, int64_t scores_qs, int32_t *d_idx, int64_t idx_qs, void *stream) {
+    INFLLM_REQUIRE(d_reps && d_qbars && d_scores && d_idx, "score_topk_queries: null pointer");
+    INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && n_queries >= 1 && n_queries <= 65535, "score_topk_queries: k=%d N=%d queries=%d", k, N, n_queries);
+    INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "score_topk_queries: row stride %lld", (long long)rep_stride);
+    const bf16_t *rows = (const bf16_t *)d_reps;
+    switch (C % 512 == 0 ? C / 512 : 0) {
+#define QUERIES_CASE(n) case n: launch_unit_scores_rows<n>(rows, rep_stride, N, d_qbars, d_scores, (hipStream_t)stream, n_queries, qbar_qs, scores_qs); break
+        QUERIES_CASE(1); QUERIES_CASE(2); QUERIES_CASE(4); QUERIES_CASE(8);
+#undef QUERIES_CASE
+    default: return 1;
+    }
+    INFLLM_CHECK_LAUNCH("score_topk_queries");
+    return launch_topk(d_scores, N, k, d_idx, nullptr, nullptr, 0, n_queries, scores_qs, idx_qs, stream);
+}
 
 // library-internal: unit scores of all N units and the k best of them in ONE launch (retrieve_fused_kernel), the ids
 // leaving as infllm_topk_publish_pair leaves them.  Returns 1, with nothing launched, where that kernel does not apply

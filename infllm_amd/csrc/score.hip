@@ -22,11 +22,13 @@ constexpr int kQPad = kD + 8;              // LDS row of Q (bf16 elements): 272 
 // launch is a chain of stages that each wait for one global load (there is next to no arithmetic to hide it behind),
 // so it takes stages of 128 queries and half as many of them.
 //
-// MERGE: the launch also carries the merge of the block's partial attention outputs, as extra workgroups behind the
-// scoring ones (blockIdx.y >= score_tiles; one thread per (row, 8 dims), merge_piece of common.h).  The two kinds of
-// work do not depend on each other - the scoring workgroups join the partial log-sum-exps themselves, by the merge's
-// own arithmetic - and the merge is a stream of loads that runs beside the matrix work: one launch instead of two
-// on the chain from one block's selection to the next.
+// MERGE: the launch also carries the merge of the block's partial attention outputs: every scoring workgroup merges
+// two (row, 8 dims) pieces per thread (merge_issue / merge_finish of common.h) while it waits for its keys.  The two
+// kinds of work do not depend on each other - the scoring workgroups join the partial log-sum-exps themselves, by
+// the merge's own arithmetic - and the merge is a handful of loads per thread that are in flight during a wait the
+// workgroup has anyway: one launch instead of two on the chain from one block's selection to the next, and no
+// workgroups of its own that would queue for the scoring workgroups' places.  In this form the joined log-sum-exps of
+// ALL the launch's queries are put into LDS once, in the same wait, instead of stage by stage.
 struct ScoreMerge {
     MergeJob job;
     int32_t score_tiles;               // blockIdx.y below this scores, from there on merges
@@ -49,6 +51,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     extern __shared__ __attribute__((aligned(16))) char score_lds[];
     bf16_t(*Qs)[kQStage][kQPad] = (bf16_t(*)[kQStage][kQPad])score_lds;                               // [2][QS][kQPad]
     float(*Ls)[kQStage] = (float(*)[kQStage])(score_lds + 2 * kQStage * kQPad * sizeof(bf16_t));      // [2][QS]
+    [[maybe_unused]] float *Lall = (float *)Ls;                                                        // MERGE: [Lq rounded up to QS]
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, grp = lane >> 5;
@@ -117,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
             const int qi = i0 + ld_row + 16 * i;
             qbuf[i] = qi < a.Lq ? *(const u32x4 *)(qbase + (int64_t)qi * a.q_sl + ld_chunk * 8) : u32x4{0, 0, 0, 0};
         }
-        if (tid < kQStage) {
+        if (!MERGE && tid < kQStage) {
             if (i0 + tid >= a.Lq) {
                 lbuf = INFINITY;                                                  // +inf => probability 0
             } else if (a.n_parts <= 0) {
@@ -145,12 +148,29 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
     auto store_stage = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < kQStage / 16; ++i) *(u32x4 *)&Qs[buf][ld_row + 16 * i][ld_chunk * 8] = qbuf[i];
-        if (tid < kQStage) Ls[buf][tid] = lbuf;
+        if (!MERGE && tid < kQStage) Ls[buf][tid] = lbuf;
     };
 
     float colsum[KS] = {};
+    if (st_hi > st_lo) load_stage(st_lo);
+    if constexpr (MERGE) {
+        // joined log-sum-exps of every query of the launch (the per-stage join above for one group of 8 partials)
+        const int64_t rows = (int64_t)a.B * a.H * a.Lq;
+        const int lq_pad = (a.Lq + kQStage - 1) / kQStage * kQStage;
+        for (int i = tid; i < lq_pad; i += 256) {
+            float l8[8], m8 = -INFINITY, den = 0.f;
+#pragma unroll
+            for (int p = 0; p < 8; ++p) l8[p] = i < a.Lq && p < a.n_parts ? lse[lps.l(p, rows) + i] : -INFINITY;
+#pragma unroll
+            for (int p = 0; p < 8; ++p) m8 = fmaxf(m8, l8[p]);
+            if (m8 != -INFINITY) {
+#pragma unroll
+                for (int p = 0; p < 8; ++p) den += __builtin_amdgcn_exp2f(l8[p] - m8);
+            }
+            Lall[i] = den > 0.f ? m8 + log2f(den) : INFINITY;              // +inf => probability 0
+        }
+    }
     if (st_hi > st_lo) {
-        load_stage(st_lo);
         store_stage(0);
         if (st_lo + 1 < st_hi) load_stage(st_lo + 1);
     }
@@ -176,7 +196,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
 #pragma unroll
                 for (int kk = 0; kk < kD / 16; ++kk) qa[kk] = *(const bf16x8 *)(qrow + kk * 16);
 #pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) l4[pb][q4] = *(const f32x4 *)&Ls[cur][qs * 32 + 8 * q4 + 4 * grp];
+                for (int q4 = 0; q4 < 4; ++q4) l4[pb][q4] = *(const f32x4 *)(MERGE ? &Lall[i0 + qs * 32 + 8 * q4 + 4 * grp] : &Ls[cur][qs * 32 + 8 * q4 + 4 * grp]);
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
@@ -222,7 +242,7 @@ __global__ __launch_bounds__(256, 2) void local_score_kernel(infllm_score_args a
                 for (int kk = 0; kk < kD / 16; ++kk) qa[kk] = *(const bf16x8 *)(qrow + kk * 16);
                 f32x4 l4[4];                                     // lse of rows 8*(r>>2) + 4*grp + (r&3)
 #pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) l4[q4] = *(const f32x4 *)&Ls[cur][qs * 32 + 8 * q4 + 4 * grp];
+                for (int q4 = 0; q4 < 4; ++q4) l4[q4] = *(const f32x4 *)(MERGE ? &Lall[i0 + qs * 32 + 8 * q4 + 4 * grp] : &Ls[cur][qs * 32 + 8 * q4 + 4 * grp]);
                 // both key halves at once: two independent accumulator chains keep the matrix pipe busy
                 f32x16 sacc2[KS];
 #pragma unroll
@@ -304,6 +324,8 @@ int check_score_args(const infllm_score_args *a) {
 }
 
 size_t score_lds_bytes(int qs) { return (size_t)(2 * qs * kQPad * sizeof(bf16_t) + 2 * qs * sizeof(float)); }
+constexpr int kMergedMaxLq = 2048;                     // MERGE: 4 bytes of LDS per query of the launch
+size_t score_lds_bytes_merged(int qs, int lq) { return (size_t)(2 * qs * kQPad * sizeof(bf16_t) + (size_t)((lq + qs - 1) / qs * qs) * sizeof(float)); }
 
 int score_lds_setup() {
     static bool lds_set = false;                       // dynamic LDS above 64 KiB must be enabled once per kernel
@@ -315,7 +337,7 @@ int score_lds_setup() {
                                     (int)score_lds_bytes(128));
         if (e == hipSuccess)
             e = hipFuncSetAttribute((const void *)local_score_kernel<2, 128, true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)score_lds_bytes(128));
+                                    (int)score_lds_bytes_merged(128, kMergedMaxLq));
         if (e != hipSuccess) return infllm_fail(-2, "local_score: %s", hipGetErrorString(e));
         lds_set = true;
     }
@@ -355,7 +377,7 @@ int infllm_local_score_merged(const infllm_score_args *a, const MergeJob *job, v
     sc.n_parts = job->P;
     int rc = check_score_args(&sc);
     if (rc) return rc;
-    if (sc.j_hi - sc.j_lo <= 1024) return 1;
+    if (sc.j_hi - sc.j_lo <= 1024 || sc.Lq > kMergedMaxLq) return 1;
     rc = score_lds_setup();
     if (rc) return rc;
     const int64_t tiles = (sc.j_hi - 1) / 64 - sc.j_lo / 64 + 1;
@@ -363,8 +385,8 @@ int infllm_local_score_merged(const infllm_score_args *a, const MergeJob *job, v
     const int64_t merge_wgs = ((int64_t)job->B * job->H * job->Lq * 16 + 255) / 256;
     const int gx = sc.B * sc.H;
     const int merge_slots = (int)((merge_wgs + gx - 1) / gx);
-    hipLaunchKernelGGL((local_score_kernel<2, 128, true>), dim3(gx, (unsigned)(score_tiles + merge_slots)), dim3(256), score_lds_bytes(128),
-                       (hipStream_t)stream, sc, ScoreMerge{*job, score_tiles});
+    hipLaunchKernelGGL((local_score_kernel<2, 128, true>), dim3(gx, (unsigned)(score_tiles + merge_slots)), dim3(256),
+                       score_lds_bytes_merged(128, sc.Lq), (hipStream_t)stream, sc, ScoreMerge{*job, score_tiles});
     INFLLM_CHECK_LAUNCH("local_score_merged");
     return 0;
 }

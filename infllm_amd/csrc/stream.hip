@@ -76,9 +76,14 @@ struct Layer {
     bool guessing = false;                             // the last selection settled a fetch made ahead of it
     // The fetch ahead of the selection (see infllm_block_prefetch): the candidates' host copy with the sequence number
     // the kernel publishes behind them, the selection whose global stage may still be running, and the guess in flight.
-    int32_t *h_cand = nullptr;                         // pinned [B*topk + 1]
+    int32_t *h_cand = nullptr;                         // pinned 2 x [B*topk + 1]: two lists may be on their way at a time
     int32_t cand_seq = 0;
-    int cand_for_units = -1;                           // unit count the published candidates were chosen from, -1: none
+    struct CandPub {
+        int64_t b0 = -1;                               // first position of the block the list is for, -1: none
+        int32_t seq = 0;                               // what the kernel stores behind the list
+    } cand_pub[2];
+    int cand_next = 0;                                 // the buffer the next list goes to
+    int64_t next_b0 = -1;                              // first position after the block whose second half was enqueued last
     std::vector<int32_t> last_sel;                     // [B, last_n_sel]
     int last_n_sel = 0;
     struct Ahead {
@@ -116,6 +121,16 @@ struct Layer {
     // device ids (this handle's own allocation) and the unit count they were chosen from (-1: none)
     int32_t *d_cand = nullptr;
     int cand_units = -1;
+    // Lists made once per prepared call (infllm_front_args.d_call_scores): for every block of the call the k best of
+    // the units that existed when the call began (d_base: [kMaxCallBlocks, B, topk], this handle's allocation) and
+    // those units' scores under the block's mean query (the caller's buffer).  While call_lists is set, a block's
+    // selection and the next block's candidates are ranked from them (run_call_rank).
+    int32_t *d_base = nullptr;
+    bool call_lists = false, no_call_lists = false;    // INFLLM_NO_CALL_LISTS=1 turns them off
+    int call_n0 = 0, call_blocks = 0;
+    float *call_scores = nullptr;
+    int64_t call_cols = 0;
+    int64_t n_call_ranked = 0;
     bool has_global = false;
     bool global_unmarked = false;         // the last global stage ran without recording global_done (see block_back)
     hipEvent_t idle_main = nullptr, idle_copy = nullptr;      // recorded by layer_flush: this layer's work up to there
@@ -180,6 +195,11 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
+int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbars, int64_t qbar_qs,
+                              int32_t n_queries, int32_t k, float *d_scores, int64_t scores_qs, int32_t *d_idx, int64_t idx_qs, void *stream);
+int infllm_call_rank(const CallRankJob *job, int32_t C, int32_t n_wgs, void *stream);
+int infllm_call_rank_room();
+constexpr int kMaxCallBlocks = 16;
 int infllm_retrieve_fused(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbar, int32_t k, float *d_scores,
                           int32_t *d_idx, int32_t *d_idx2, int32_t *d_flag, int32_t flag_value, void *stream);
 int infllm_inline_page_limit();
@@ -863,12 +883,18 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         L->page_table_kernel = pk && pk[0] && pk[0] != '0';
         const char *ma = getenv("INFLLM_SCORE_MERGE_APART");
         L->score_merge_apart = ma && ma[0] && ma[0] != '0';
+        const char *nl = getenv("INFLLM_NO_CALL_LISTS");
+        L->no_call_lists = nl && nl[0] && nl[0] != '0';
     }
-    if (hipHostMalloc((void **)&L->h_cand, ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
+    if (hipHostMalloc((void **)&L->h_cand, 2 * ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
         (void)hipGetLastError();
         L->h_cand = nullptr;                        // no fetch ahead of the selection then
     } else
-        std::memset(L->h_cand, 0, ((size_t)d.B * d.topk + 1) * sizeof(int32_t));
+        std::memset(L->h_cand, 0, 2 * ((size_t)d.B * d.topk + 1) * sizeof(int32_t));
+    if (d.topk > 0 && hipMalloc((void **)&L->d_base, sizeof(int32_t) * kMaxCallBlocks * d.B * d.topk) != hipSuccess) {
+        (void)hipGetLastError();
+        L->d_base = nullptr;                        // not fatal: every block's selection then runs over all units
+    }
     return L;
 }
 
@@ -902,6 +928,7 @@ extern "C" int infllm_layer_destroy(void *layer) {
         for (hipEvent_t e : t.ev)
             if (e) (void)hipEventDestroy(e);
     if (L->d_cand) (void)hipFree(L->d_cand);
+    if (L->d_base) (void)hipFree(L->d_base);
     if (L->h_cand) (void)hipHostFree(L->h_cand);
     for (void *c : L->ahead.shadow)
         if (c) (void)infllm_cache_destroy(c);
@@ -1120,6 +1147,60 @@ int run_score_new_rank(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_s
     return 0;
 }
 
+int32_t *cand_buffer(Layer *L, int buf) { return L->h_cand + (int64_t)buf * ((int64_t)L->d.B * L->d.topk + 1); }
+
+// where the next candidate list goes: the buffer, and the note by which infllm_block_prefetch finds it
+int cand_publication(Layer *L, int64_t for_b0) {
+    const int buf = L->cand_next;
+    L->cand_next ^= 1;
+    ++L->cand_seq;
+    L->cand_pub[buf].b0 = for_b0;
+    L->cand_pub[buf].seq = L->cand_seq;
+    return buf;
+}
+
+bool call_rank_fits(const Layer *L, int first_new, int n_new) {
+    return n_new <= 64 && L->d.topk + (first_new + n_new - L->call_n0) <= infllm_call_rank_room();
+}
+
+// From the lists of the prepared call (Layer::call_lists): the n_new units from first_new on were carved just now;
+// their scores under the mean queries of the call's later blocks, the selection of block j_sel and the candidates of
+// block j_cand (block numbers within the call, -1: none) in one launch.  The caller has checked call_rank_fits.
+int run_call_rank(Layer *L, const void *reps, int64_t rep_sb, int64_t rep_su, int first_new, int n_new, int j_sel, int j_cand, void *stream) {
+    const infllm_layer_desc &d = L->d;
+    hipStream_t st = (hipStream_t)stream;
+    if (j_cand >= 0 && !L->h_cand) j_cand = -1;
+    const int j0 = j_sel >= 0 ? j_sel : j_cand;
+    if (j0 < 0) return 0;                                   // (new units are only ever carved with a block to follow)
+    CallRankJob jb{};
+    jb.reps = (const bf16_t *)reps; jb.rep_sb = rep_sb; jb.rep_su = rep_su;
+    jb.qbars = L->bd.d_qbar; jb.scores = L->call_scores; jb.cols = L->call_cols; jb.base = L->d_base;
+    jb.B = d.B; jb.k = d.topk; jb.n_base = L->call_n0; jb.first_new = first_new; jb.n_new = n_new;
+    jb.j0 = j0; jb.j_sel = j_sel; jb.j_cand = j_cand;
+    const bool poll = d.d_topk_flag && d.h_topk_flag && !d.h_topk_idx;
+    if (j_sel >= 0) {
+        if (poll) ++L->topk_seq;
+        jb.sel_out = d.d_topk_idx; jb.sel_flag = poll ? d.d_topk_flag : nullptr; jb.sel_seq = L->topk_seq;
+    }
+    if (j_cand >= 0) {
+        const int buf = cand_publication(L, L->batch_b0 + (int64_t)j_cand * d.exc);
+        jb.cand_out = cand_buffer(L, buf); jb.cand_flag = jb.cand_out + (int64_t)d.B * d.topk; jb.cand_seq = L->cand_seq;
+    }
+    const int last = j_cand >= 0 ? j_cand : j_sel;
+    const int n_wgs = n_new > 0 ? L->call_blocks - j0 : last - j0 + 1;
+    int rc = infllm_call_rank(&jb, d.H * kD, n_wgs, stream);
+    if (rc) return rc < 0 ? rc : infllm_fail(-2, "call_rank: no kernel after the checks");
+    if (j_sel >= 0) {
+        if (d.h_topk_idx)
+            HIP_OK(hipMemcpyAsync(d.h_topk_idx, d.d_topk_idx, sizeof(int32_t) * d.B * d.topk, hipMemcpyDeviceToHost, st), "index copy");
+        if (!poll) HIP_OK(hipEventRecord(L->topk_done, st), "event");
+        L->topk_stream = st;
+        L->topk_pending = true;
+        ++L->n_call_ranked;
+    }
+    return 0;
+}
+
 // n_parts > 0: the stages' partial log-sum-exps are joined inside the launch (d_lse is not ready yet)
 infllm_score_args local_score_args(Layer *L, int n, int64_t b0, const Layer::QView &qv, int64_t j_lo, int64_t j_hi, int n_parts) {
     const infllm_layer_desc &d = L->d;
@@ -1263,6 +1344,30 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
     L->fresh = batch_view(L, a->b0);
 
     L->batch_retrieved = retrieve;
+
+    // ---- the lists of the call's other blocks: the k best of the units that exist now under each block's mean query,
+    //      in two launches for the whole call; the candidates of the second block are its list as it stands
+    L->call_lists = false;
+    const int max_new = (a->n + d.block_size - 1) / d.block_size + 1;
+    const int cpl = C % 512 == 0 ? C / 512 : 0;
+    if (retrieve && n_blocks > 1 && n_blocks <= kMaxCallBlocks && a->d_call_scores && L->d_base && !L->no_call_lists && d.topk <= 64 &&
+        (cpl == 1 || cpl == 2 || cpl == 4 || cpl == 8) && a->call_scores_cols >= (int64_t)a->n_units + max_new) {
+        const int64_t cols = a->call_scores_cols;
+        for (int u = 0; u < d.B; ++u) {
+            rc = infllm_score_topk_queries((const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb, a->rep_su, a->n_units, C,
+                                           L->bd.d_qbar + ((int64_t)d.B + u) * C, (int64_t)d.B * C, n_blocks - 1, d.topk,
+                                           a->d_call_scores + ((int64_t)d.B + u) * cols, (int64_t)d.B * cols,
+                                           L->d_base + ((int64_t)d.B + u) * d.topk, (int64_t)d.B * d.topk, stream);
+            if (rc) return rc < 0 ? rc : infllm_fail(-2, "call_front: no scoring kernel after the geometry check");
+        }
+        L->call_lists = true;
+        L->call_n0 = a->n_units;
+        L->call_blocks = n_blocks;
+        L->call_scores = a->d_call_scores;
+        L->call_cols = cols;
+        rc = run_call_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->n_units, 0, -1, 1, stream);
+        if (rc) return rc;
+    }
     return 0;
 }
 
@@ -1302,7 +1407,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     L->prepared = false;
     L->cur = L->fresh;
     L->cur_n = a->n;
-    L->cand_for_units = -1;
+    if (!batched) L->call_lists = false;
 
     const int64_t b1 = a->b0 + a->n;
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
@@ -1319,21 +1424,24 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
             rc = run_ingest(L, a, a->d_q_next, a->d_k_next, a->d_v_next, a->n_next, b1, L->slot, true, stream);
             if (rc) return rc;
         }
-        if (a->n_units > 0 && !(a->flags & INFLLM_NO_RETRIEVAL)) {
+        // (with the lists of a prepared call the next block's candidates were ranked when the previous block had
+        //  carved its units, or by infllm_call_front: nothing to do here)
+        if (a->n_units > 0 && !(a->flags & INFLLM_NO_RETRIEVAL) && !(L->call_lists && next_batched)) {
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
             // The scores of the existing units and their k best now, while the fetch is in flight: the selection after the
             // block then only has to weigh these against the few units carved in between, instead of running over every
             // unit on the chain.  One launch per batch row where the geometry has the kernel for it, else two.
             L->cand_units = -1;
             const bool want_cand = L->d_cand && a->n_units > d.topk;
-            if (want_cand && L->h_cand) ++L->cand_seq;       // the host gets a copy, with a sequence number behind the last row's: it may fetch them ahead
+            // the host gets a copy, with a sequence number behind the last row's: it may fetch them ahead
+            const int buf = want_cand && L->h_cand ? cand_publication(L, b1) : -1;
             const int C = d.H * kD;
             for (int u = 0; u < d.B; ++u) {
                 const bf16_t *reps_u = (const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb;
                 float *scores_u = a->d_unit_scores + (int64_t)u * a->unit_scores_sb;
                 const float *qbar_u = L->fresh.qbar + (int64_t)u * C;
-                int32_t *cand_host = L->h_cand ? L->h_cand + (int64_t)u * d.topk : nullptr;
-                int32_t *cand_flag = L->h_cand && u == d.B - 1 ? L->h_cand + (int64_t)d.B * d.topk : nullptr;
+                int32_t *cand_host = buf >= 0 ? cand_buffer(L, buf) + (int64_t)u * d.topk : nullptr;
+                int32_t *cand_flag = buf >= 0 && u == d.B - 1 ? cand_buffer(L, buf) + (int64_t)d.B * d.topk : nullptr;
                 rc = want_cand ? infllm_retrieve_fused(reps_u, a->rep_su, a->n_units, C, qbar_u, d.topk, scores_u, L->d_cand + (int64_t)u * d.topk,
                                                        cand_host, cand_flag, L->cand_seq, stream)
                                : 1;
@@ -1348,10 +1456,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
                     }
                 }
             }
-            if (want_cand) {
-                L->cand_units = a->n_units;
-                L->cand_for_units = L->h_cand ? a->n_units : -1;
-            }
+            if (want_cand) L->cand_units = a->n_units;
         }
         L->prepared = true;
         L->prepared_b0 = b1;
@@ -1472,23 +1577,29 @@ extern "C" int infllm_block_prefetch(void *layer, const infllm_select_args *a, v
     Layer::Ahead &g = L->ahead;
     INFLLM_REQUIRE(!g.active, "block_prefetch: the previous guess has not been settled by infllm_block_select");
     const int k = d.topk, B = d.B;
-    if (L->cand_for_units < 0 || !L->h_cand || k > 64) return 0;
-    L->cand_for_units = -1;
+    if (!L->h_cand || k > 64 || L->next_b0 < 0) return 0;
+    int buf = -1;                                        // the list that was chosen for the block that comes next
+    for (int i = 0; i < 2; ++i)
+        if (L->cand_pub[i].b0 == L->next_b0) buf = i;
+    if (buf < 0) return 0;
+    const int32_t cand_seq = L->cand_pub[buf].seq;
+    L->cand_pub[buf].b0 = -1;
+    const int32_t *h_cand = cand_buffer(L, buf);
     // Beside the block's own kernels the fetch kernel slows them down by more than the shorter chain gains (measured):
     // without the DMA engines the fetch stays behind the selection, unless INFLLM_FETCH_AHEAD_ALWAYS=1 asks for it.
     if (!L->efetch_ok && !L->ahead_any_path) return 0;
     INFLLM_REQUIRE(a->caches && a->h_chunk_base && a->units_per_chunk > 0 && a->n_chunks >= 0 && a->unit_bytes > 0 && a->row_bytes > 0,
                    "block_prefetch: bad cache list / host arena description");
-    // the candidates were chosen right after the local stage of the block in flight
-    const volatile int32_t *flag = L->h_cand + (int64_t)B * k;
+    // (the list was launched ahead of the local stage of the block in flight, or behind the block before it)
+    const volatile int32_t *flag = h_cand + (int64_t)B * k;
     const auto t0 = std::chrono::steady_clock::now();
-    for (uint32_t spins = 0; *flag != L->cand_seq; ++spins) {
+    for (uint32_t spins = 0; *flag != cand_seq; ++spins) {
         if ((spins & 1023u) == 1023u && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) return 0;
         __builtin_ia32_pause();
     }
     std::atomic_thread_fence(std::memory_order_acquire);
     g.n_sel = k;
-    g.cand.assign(L->h_cand, L->h_cand + (int64_t)B * k);
+    g.cand.assign(h_cand, h_cand + (int64_t)B * k);
     g.sel_slots.resize((size_t)B * k);
     g.evicted.resize((size_t)B * k);
     g.n_evicted.assign(B, 0);
@@ -1554,6 +1665,7 @@ extern "C" int infllm_layer_path_counts(void *layer, int64_t *counts) {
     counts[2] = L->n_tables_upload;
     counts[3] = L->n_score_merged;
     counts[4] = L->n_score_apart;
+    counts[5] = L->n_call_ranked;
     return 0;
 }
 
@@ -1726,6 +1838,7 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
                    "block_back: bad output / carve arguments");
     INFLLM_REQUIRE(a->n_units >= 0, "block_back: negative unit count");
     const int64_t b1 = a->b0 + a->n;
+    L->next_b0 = b1;
     const int64_t unit_elems = (int64_t)d.Hkv * bs * kD;          // K (or V) of one unit
     const int64_t slot_elems = 2 * unit_elems;
     const Layer::QView &cur = L->cur;
@@ -2013,11 +2126,23 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     const int n_units_next = a->n_units + a->n_carve;
     if (L->prepared && n_units_next > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL)) {
         INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_back: null representative / score buffer");
-        const bool merge = L->cand_units == a->n_units && d.topk + a->n_carve <= 64;
-        rc = merge ? run_score_new_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, stream)
-                   : 1;
+        // with the lists of a prepared call: the new units' scores for the call's later blocks, the next block's
+        // selection and the candidates of the block after it, one launch
+        const int j_next = L->call_lists && batched ? (int)((b1 - L->batch_b0) / d.exc) : -1;
+        if (j_next >= 1 && j_next < L->call_blocks && block_in_batch(L, b1, L->prepared_n) && call_rank_fits(L, a->n_units, a->n_carve)) {
+            rc = run_call_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->n_units, a->n_carve, j_next, j_next + 1 < L->call_blocks ? j_next + 1 : -1,
+                               stream);
+            if (rc) return rc;
+            rc = 0;
+        } else {
+            L->call_lists = false;      // (lists that no longer fit their kernel: the rest of the call selects over all units)
+            const bool merge = L->cand_units == a->n_units && d.topk + a->n_carve <= 64;
+            rc = merge ? run_score_new_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, stream)
+                       : 1;
+        }
         if (rc < 0) return rc;
         if (rc == 1) {                  // the two steps on their own
+            const bool merge = L->cand_units == a->n_units && d.topk + a->n_carve <= 64;
             rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->fresh.qbar,
                                  stream);
             if (rc) return rc;

@@ -67,6 +67,30 @@ def test_page_table_in_the_launch_gives_the_bits_of_the_table_in_memory(monkeypa
         assert b[2]["tables_inline"] == 0 and b[2]["tables_kernel"] == a[2]["tables_inline"], (a[2], b[2])
 
 
+def test_selections_from_the_lists_of_a_call_are_the_selections_over_all_units(monkeypatch):
+    """A prepared call chooses, once, the k best of the units that exist when it begins for every one of its blocks; a
+    block's selection (and the candidates its fetch is started from) then weighs that list against the units carved since
+    the call began.  INFLLM_NO_CALL_LISTS=1 keeps a pass over all units per block.  The same ids in the same order either
+    way, so outputs, selections, residency counters and representatives are equal bit for bit: small geometry with two
+    batch rows (calls of 16 blocks, 2 units carved per block) and the reference geometry."""
+    def run(no_lists, T, calls, H, Hkv, base, seed, B, kw):
+        if no_lists:
+            monkeypatch.setenv("INFLLM_NO_CALL_LISTS", "1")
+        else:
+            monkeypatch.delenv("INFLLM_NO_CALL_LISTS", raising=False)
+        q, k, v = make_stream(T, H, Hkv, seed, B=B)
+        out, cm = run_gpu(q, k, v, calls, base, **kw)
+        return out, [b["order"] for b in cm.trace_blocks], cm.stats, cm.prefetch_stats(), cm.path_counts(), cm.trace_repr_indices()
+
+    for args in ((3000, [1500, 1, 1499], 8, 2, 1e4, 47, 2, SMALL), (8192 + 8192 + 1000, [8192, 8192, 1000], 32, 8, 1e6, 48, 1, REFERENCE)):
+        a, b = run(False, *args), run(True, *args)
+        assert torch.equal(a[0], b[0]) and a[1] == b[1] and a[2] == b[2] and a[3] == b[3] and len(a[1]) > 20
+        assert a[5].keys() == b[5].keys() and all(torch.equal(a[5][u], b[5][u]) for u in a[5])
+        # the switch is read when a layer is created: the first run ranked from the lists, the second never did
+        assert a[4]["call_ranked"] > 10 and b[4]["call_ranked"] == 0, (a[4], b[4])
+        assert a[3][0] > 10                                          # fetches were started ahead from the lists' candidates
+
+
 def test_score_decay_policy_follows_oracle():
     """cache_strategy lru-s: evictions are decided by the decayed attention mass each cached unit received
     (context_manager.py:454-470), which the device computes and the host reads back once per block."""
