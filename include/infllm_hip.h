@@ -232,6 +232,15 @@ int infllm_score_topk(const void *d_reps, int64_t rep_stride, int32_t N, int32_t
 int infllm_score_new_topk(const void *d_reps, int64_t rep_stride, int32_t C, const float *d_qbar, float *d_scores,
                           const int32_t *d_cand, int32_t n_cand, int32_t first_new, int32_t n_new, int32_t k, int32_t *d_idx,
                           void *stream);
+/* infllm_score_topk for several mean queries over the same N units, every representative read once per 8 queries
+ * (the selections of all execution blocks of a chunk or call against the units that exist at its start:
+ * get_batched_topk, context_manager.py:548-612; the stream uses it once per prepared call).  Query q's scores go to
+ * d_scores + q * scores_qs (the same bits as infllm_unit_scores gives), its ids to d_idx + q * idx_qs, its mean query
+ * is at d_qbars + q * qbar_qs.  Rows of 512, 1024, 2048 or 4096 elements; returns 1, with nothing launched, for other
+ * row lengths. */
+int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbars, int64_t qbar_qs,
+                              int32_t n_queries, int32_t k, float *d_scores, int64_t scores_qs, int32_t *d_idx, int64_t idx_qs,
+                              void *stream);
 /* The two halves of infllm_score_topk: scores of rows [first, first+count) into d_scores[first..], and the
  * selection over d_scores[0..N).  Scoring the units that exist early and only the newly carved ones late keeps
  * the retrieval of the next block short. */

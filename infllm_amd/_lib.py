@@ -146,6 +146,7 @@ SYMBOLS = {
     "infllm_unit_scores": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp]),
     "infllm_topk": (c_i32, [c_vp, c_i32, c_i32, c_vp, c_vp]),
     "infllm_score_topk": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_vp, c_i32, c_vp, c_vp, c_vp]),
+    "infllm_score_topk_queries": (c_i32, [c_vp, c_i64, c_i32, c_i32, c_vp, c_i64, c_i32, c_i32, c_vp, c_i64, c_vp, c_i64, c_vp]),
     "infllm_score_new_topk": (c_i32, [c_vp, c_i64, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "infllm_repr_keys": (c_i32, [c_vp, c_vp, c_i64, c_i32, c_i32, c_i32, c_i64, c_i32, c_i32, c_i32,
                                  c_vp, c_i64, c_i64, c_vp, c_vp]),

@@ -896,23 +896,105 @@ int infllm_call_rank(const CallRankJob *job, int32_t C, int32_t n_wgs, void *str
 }
 int infllm_call_rank_room() { return kCallRankEntries; }
 
-// library-internal: the k best of the same N units under each of n_queries queries (context_manager.py:159-163 for
-// several blocks of a call at once): query q's scores go to d_scores + q * scores_qs, its ids to d_idx + q * idx_qs.
-// Returns 1, with nothing launched, for row lengths other than 512 * {1, 2, 4, 8}.
-int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbars, int64_t qbar_qs,
+// select_topk_block over several tables, one workgroup each (table t at scores + t * scores_xs, its ids to
+// idx_out + t * idx_xs)
+template <int NB>
+__global__ __launch_bounds__(kRetrThreads) void select_rows_kernel(const float *scores, int N, int k, int32_t *idx_out, int64_t scores_xs,
+                                                                   int64_t idx_xs) {
+    select_topk_block<NB>(scores + blockIdx.x * scores_xs, N, k, idx_out + blockIdx.x * idx_xs, nullptr);
+}
+
+// Scores of the same N rows under several queries, every row read once per group of QG queries: the group's queries
+// sit in LDS (QG x C floats), a wave keeps two rows in registers and walks the group's queries over them.  The sums
+// are unit_scores_rows_kernel's, term by term.
+constexpr int kQueryGroup = 8;
+template <int CPL>
+__global__ __launch_bounds__(512) void unit_scores_queries_kernel(const bf16_t *reps, int64_t rep_stride, int N, const float *qbars,
+                                                                   int64_t qbar_qs, int n_queries, float *scores, int64_t scores_qs) {
+    extern __shared__ float qs[];                               // [kQueryGroup][C]
+    constexpr int C = CPL * 512;
+    const int lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * 8;
+    const int q0 = blockIdx.y * kQueryGroup;
+    const int nq = min(kQueryGroup, n_queries - q0);
+    int n = blockIdx.x * 8 + (threadIdx.x >> 6);                // rows n, n + n_waves, ... belong to this wave
+    u32x4 w[2][CPL];
+    auto load_rows = [&](int first) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+            if (first + r * n_waves < N) {
+                const bf16_t *row = reps + (int64_t)(first + r * n_waves) * rep_stride + lane * 8;
+#pragma unroll
+                for (int j = 0; j < CPL; ++j) w[r][j] = *(const u32x4 *)(row + j * 512);
+            }
+    };
+    load_rows(n);
+    for (int e = threadIdx.x * 4; e < nq * C; e += 512 * 4)
+        *(f32x4 *)(qs + e) = *(const f32x4 *)(qbars + (int64_t)(q0 + e / C) * qbar_qs + e % C);
+    __syncthreads();
+    while (n < N) {
+        const bool two = n + n_waves < N;
+        float res[2][kQueryGroup];
+        for (int q = 0; q < nq; ++q) {
+            const float *qq = qs + q * C;
+            float a00 = 0.f, a01 = 0.f, a10 = 0.f, a11 = 0.f;
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+                const f32x4 lo = *(const f32x4 *)(qq + j * 512 + lane * 8), hi = *(const f32x4 *)(qq + j * 512 + lane * 8 + 4);
+                const float qv[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    a00 += bf16_bits_to_f32(w[0][j][i] & 0xffffu) * qv[2 * i];
+                    a01 += bf16_bits_to_f32(w[0][j][i] >> 16) * qv[2 * i + 1];
+                    a10 += bf16_bits_to_f32(w[1][j][i] & 0xffffu) * qv[2 * i];
+                    a11 += bf16_bits_to_f32(w[1][j][i] >> 16) * qv[2 * i + 1];
+                }
+            }
+            res[0][q] = wave_sum(a00 + a01);
+            res[1][q] = wave_sum(a10 + a11);
+        }
+        if (lane == 0) {
+            for (int q = 0; q < nq; ++q) {
+                scores[(int64_t)(q0 + q) * scores_qs + n] = res[0][q];
+                if (two) scores[(int64_t)(q0 + q) * scores_qs + n + n_waves] = res[1][q];
+            }
+        }
+        n += 2 * n_waves;
+        load_rows(n);
+    }
+}
+
+extern "C" int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbars, int64_t qbar_qs,
                               int32_t n_queries, int32_t k, float *d_scores, int64_t scores_qs, int32_t *d_idx, int64_t idx_qs, void *stream) {
     INFLLM_REQUIRE(d_reps && d_qbars && d_scores && d_idx, "score_topk_queries: null pointer");
     INFLLM_REQUIRE(N > 0 && k > 0 && k <= N && n_queries >= 1 && n_queries <= 65535, "score_topk_queries: k=%d N=%d queries=%d", k, N, n_queries);
     INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "score_topk_queries: row stride %lld", (long long)rep_stride);
     const bf16_t *rows = (const bf16_t *)d_reps;
+    const int groups = (n_queries + kQueryGroup - 1) / kQueryGroup;
+    int wgs = (N + 15) / 16;                               // two rows per wave and trip
+    if (wgs > 256) wgs = 256;                              // one workgroup per CU: the queries take most of its LDS
+    static bool lds_set = false;                           // dynamic LDS above 64 KiB must be enabled once per kernel
+    if (!lds_set) {
+        hipError_t e = hipFuncSetAttribute((const void *)unit_scores_queries_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kQueryGroup * 4096 * (int)sizeof(float));
+        if (e != hipSuccess) return infllm_fail(-2, "score_topk_queries: %s", hipGetErrorString(e));
+        lds_set = true;
+    }
     switch (C % 512 == 0 ? C / 512 : 0) {
-#define QUERIES_CASE(n) case n: launch_unit_scores_rows<n>(rows, rep_stride, N, d_qbars, d_scores, (hipStream_t)stream, n_queries, qbar_qs, scores_qs); break
+#define QUERIES_CASE(n) case n: hipLaunchKernelGGL(unit_scores_queries_kernel<n>, dim3(wgs, groups), dim3(512), (size_t)kQueryGroup * n * 512 * sizeof(float), \
+                                                    (hipStream_t)stream, rows, rep_stride, N, d_qbars, qbar_qs, n_queries, d_scores, scores_qs); break
         QUERIES_CASE(1); QUERIES_CASE(2); QUERIES_CASE(4); QUERIES_CASE(8);
 #undef QUERIES_CASE
     default: return 1;
     }
     INFLLM_CHECK_LAUNCH("score_topk_queries");
-    return launch_topk(d_scores, N, k, d_idx, nullptr, nullptr, 0, n_queries, scores_qs, idx_qs, stream);
+    if (N > 32 * kRetrThreads || k > 64) return launch_topk(d_scores, N, k, d_idx, nullptr, nullptr, 0, n_queries, scores_qs, idx_qs, stream);
+    if (N <= 16 * kRetrThreads)
+        hipLaunchKernelGGL(select_rows_kernel<1>, dim3(n_queries), dim3(kRetrThreads), 0, (hipStream_t)stream, d_scores, N, k, d_idx, scores_qs, idx_qs);
+    else
+        hipLaunchKernelGGL(select_rows_kernel<2>, dim3(n_queries), dim3(kRetrThreads), 0, (hipStream_t)stream, d_scores, N, k, d_idx, scores_qs, idx_qs);
+    INFLLM_CHECK_LAUNCH("score_topk_queries (selection)");
+    return 0;
 }
 
 // library-internal: unit scores of all N units and the k best of them in ONE launch (retrieve_fused_kernel), the ids

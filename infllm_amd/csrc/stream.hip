@@ -127,6 +127,7 @@ struct Layer {
     // selection and the next block's candidates are ranked from them (run_call_rank).
     int32_t *d_base = nullptr;
     bool call_lists = false, no_call_lists = false;    // INFLLM_NO_CALL_LISTS=1 turns them off
+    bool call_lists_pending = false;                   // the call in flight wants them: its first block's second half makes them
     int call_n0 = 0, call_blocks = 0;
     float *call_scores = nullptr;
     int64_t call_cols = 0;
@@ -195,8 +196,6 @@ __global__ __launch_bounds__(256) void unit_mass_kernel(const float *scratch, in
 
 }  // namespace
 int infllm_topk_publish(const float *d_scores, int32_t N, int32_t k, int32_t *d_idx, int32_t *d_flag, int32_t flag_value, void *stream);
-int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride, int32_t N, int32_t C, const float *d_qbars, int64_t qbar_qs,
-                              int32_t n_queries, int32_t k, float *d_scores, int64_t scores_qs, int32_t *d_idx, int64_t idx_qs, void *stream);
 int infllm_call_rank(const CallRankJob *job, int32_t C, int32_t n_wgs, void *stream);
 int infllm_call_rank_room();
 constexpr int kMaxCallBlocks = 16;
@@ -1345,28 +1344,20 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
 
     L->batch_retrieved = retrieve;
 
-    // ---- the lists of the call's other blocks: the k best of the units that exist now under each block's mean query,
-    //      in two launches for the whole call; the candidates of the second block are its list as it stands
+    // ---- the lists of the call's other blocks (the k best of the units that exist now under each block's mean query)
+    //      are made behind the first block's global stage (block_back): here they would sit between the first
+    //      selection and the first global stage, a stretch in which the stream only waits for the first fetch
     L->call_lists = false;
+    L->call_lists_pending = false;
     const int max_new = (a->n + d.block_size - 1) / d.block_size + 1;
     const int cpl = C % 512 == 0 ? C / 512 : 0;
     if (retrieve && n_blocks > 1 && n_blocks <= kMaxCallBlocks && a->d_call_scores && L->d_base && !L->no_call_lists && d.topk <= 64 &&
         (cpl == 1 || cpl == 2 || cpl == 4 || cpl == 8) && a->call_scores_cols >= (int64_t)a->n_units + max_new) {
-        const int64_t cols = a->call_scores_cols;
-        for (int u = 0; u < d.B; ++u) {
-            rc = infllm_score_topk_queries((const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb, a->rep_su, a->n_units, C,
-                                           L->bd.d_qbar + ((int64_t)d.B + u) * C, (int64_t)d.B * C, n_blocks - 1, d.topk,
-                                           a->d_call_scores + ((int64_t)d.B + u) * cols, (int64_t)d.B * cols,
-                                           L->d_base + ((int64_t)d.B + u) * d.topk, (int64_t)d.B * d.topk, stream);
-            if (rc) return rc < 0 ? rc : infllm_fail(-2, "call_front: no scoring kernel after the geometry check");
-        }
-        L->call_lists = true;
+        L->call_lists_pending = true;
         L->call_n0 = a->n_units;
         L->call_blocks = n_blocks;
         L->call_scores = a->d_call_scores;
-        L->call_cols = cols;
-        rc = run_call_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->n_units, 0, -1, 1, stream);
-        if (rc) return rc;
+        L->call_cols = a->call_scores_cols;
     }
     return 0;
 }
@@ -1407,7 +1398,7 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
     L->prepared = false;
     L->cur = L->fresh;
     L->cur_n = a->n;
-    if (!batched) L->call_lists = false;
+    if (!batched) L->call_lists = L->call_lists_pending = false;
 
     const int64_t b1 = a->b0 + a->n;
     const int64_t lo = a->b0 > d.n_local ? a->b0 - d.n_local : 0;
@@ -2128,6 +2119,19 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_back: null representative / score buffer");
         // with the lists of a prepared call: the new units' scores for the call's later blocks, the next block's
         // selection and the candidates of the block after it, one launch
+        if (L->call_lists_pending && batched && a->b0 == L->batch_b0) {
+            // the first block of a prepared call: the lists of its other blocks, two launches for the whole call
+            L->call_lists_pending = false;
+            const int C = d.H * kD;
+            for (int u = 0; u < d.B && a->n_units == L->call_n0; ++u) {
+                rc = infllm_score_topk_queries((const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb, a->rep_su, L->call_n0, C,
+                                               L->bd.d_qbar + ((int64_t)d.B + u) * C, (int64_t)d.B * C, L->call_blocks - 1, d.topk,
+                                               L->call_scores + ((int64_t)d.B + u) * L->call_cols, (int64_t)d.B * L->call_cols,
+                                               L->d_base + ((int64_t)d.B + u) * d.topk, (int64_t)d.B * d.topk, stream);
+                if (rc) return rc < 0 ? rc : infllm_fail(-2, "block_back: no scoring kernel after the geometry check");
+                L->call_lists = u == d.B - 1;
+            }
+        }
         const int j_next = L->call_lists && batched ? (int)((b1 - L->batch_b0) / d.exc) : -1;
         if (j_next >= 1 && j_next < L->call_blocks && block_in_batch(L, b1, L->prepared_n) && call_rank_fits(L, a->n_units, a->n_carve)) {
             rc = run_call_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->n_units, a->n_carve, j_next, j_next + 1 < L->call_blocks ? j_next + 1 : -1,

@@ -206,6 +206,23 @@ def score_topk(reps, n, qbar, k, scores, idx):
           "infllm_score_topk")
 
 
+def unit_scores(reps, first, count, qbar, scores):
+    """scores[first:first+count] = reps[first:first+count] @ qbar."""
+    check(_lib.load().infllm_unit_scores(reps.data_ptr(), reps.stride(0), first, count, reps.shape[1], qbar.data_ptr(),
+                                         scores.data_ptr(), _stream()), "infllm_unit_scores")
+
+
+def score_topk_queries(reps, n, qbars, k, scores, idx):
+    """scores[q, :n] = reps[:n] @ qbars[q] and idx[q, :k] = indices of the k largest, descending score, for every query q
+    in one pass over the representatives."""
+    rc = _lib.load().infllm_score_topk_queries(reps.data_ptr(), reps.stride(0), n, reps.shape[1], qbars.data_ptr(), qbars.stride(0),
+                                               qbars.shape[0], k, scores.data_ptr(), scores.stride(0), idx.data_ptr(), idx.stride(0),
+                                               _stream())
+    if rc == 1:
+        raise ValueError(f"score_topk_queries: rows of {reps.shape[1]} elements (supported: 512, 1024, 2048, 4096)")
+    check(rc, "infllm_score_topk_queries")
+
+
 def score_new_topk(reps, qbar, scores, cand, first_new, n_new, k, idx):
     """scores[first_new:first_new+n_new] = reps[those rows] @ qbar, then idx[:k] = the top-k over all first_new + n_new
     scores, given cand = the top-k of the first first_new."""

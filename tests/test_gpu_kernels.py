@@ -379,6 +379,29 @@ def test_score_topk_matches_bruteforce(N, k):
         assert abs(want[i] - kth) <= 1e-3 * abs(kth)
 
 
+@pytest.mark.parametrize("N,k,heads,Q", [(991, 16, 32, 15), (17, 16, 32, 1), (8159, 16, 32, 9), (300, 4, 8, 16), (5000, 64, 4, 3),
+                                         (20000, 16, 16, 2)])
+def test_several_queries_in_one_pass_give_the_scores_and_ids_of_one_query_at_a_time(N, k, heads, Q):
+    """infllm_score_topk_queries against infllm_unit_scores + infllm_topk query by query: the scores bit for bit (a unit's
+    score must not depend on which kernel computed it: selections ranked from a call's lists are compared with
+    selections over all units), the same ids in the same order."""
+    ops = _ops()
+    C = heads * D
+    reps = _rand((N + 3, C), 60 + N)[:N].cuda()
+    qbars = torch.randn((Q, C), generator=torch.Generator().manual_seed(61)).cuda()
+    scores = torch.full((Q, N + 5), -7.0, dtype=torch.float32, device="cuda")
+    idx = torch.full((Q, k + 2), -1, dtype=torch.int32, device="cuda")
+    ops.score_topk_queries(reps, N, qbars, k, scores, idx)
+    for q in range(Q):
+        one = torch.empty((N,), dtype=torch.float32, device="cuda")
+        one_idx = torch.empty((k,), dtype=torch.int32, device="cuda")
+        ops.unit_scores(reps, 0, N, qbars[q], one)
+        ops.topk(one, N, k, one_idx)
+        assert torch.equal(scores[q, :N], one), q
+        assert torch.equal(idx[q, :k], one_idx), q
+    assert bool((scores[:, N:] == -7.0).all()) and bool((idx[:, k:] == -1).all())      # nothing beyond what was asked for
+
+
 @pytest.mark.parametrize("n_old,n_new,k,heads", [(991, 4, 16, 32), (40, 1, 16, 32), (16, 16, 16, 8), (300, 7, 4, 16), (5000, 48, 16, 4),
                                                  (64, 3, 1, 32)])
 def test_new_units_scored_and_ranked_in_one_launch_equal_the_two_steps(n_old, n_new, k, heads):
