@@ -571,13 +571,20 @@ class ContextManager:
                                           self.unit_size, c1 - c0, exc, self.inv_freq.data_ptr(),
                                           float(self.position_embedding.distance_scale), self.n_local - 1,
                                           qbar.data_ptr(), self._main_raw), "infllm_chunk_qbar")
-        scores = torch.empty((N,), dtype=torch.float32, device=self.device)
+        # every block's mean query over the same units: the representatives are read once per eight blocks
+        scores = torch.empty((n_blocks, N), dtype=torch.float32, device=self.device)
         idx = torch.empty((n_blocks, B, topk), dtype=torch.int32, device=self.device)
-        for j in range(n_blocks):
-            for u in range(B):
-                check(self._lib.infllm_score_topk(self.reps[u].data_ptr(), self.reps.stride(1), N, C, qbar[u, j].data_ptr(),
-                                                  topk, scores.data_ptr(), idx[j, u].data_ptr(), self._main_raw),
-                      "infllm_score_topk")
+        for u in range(B):
+            rc = self._lib.infllm_score_topk_queries(self.reps[u].data_ptr(), self.reps.stride(1), N, C, qbar[u].data_ptr(), qbar.stride(1),
+                                                     n_blocks, topk, scores.data_ptr(), scores.stride(0), idx[:, u].data_ptr(),
+                                                     idx.stride(0), self._main_raw)
+            if rc == 1:                                      # row lengths without that kernel: one block at a time
+                for j in range(n_blocks):
+                    check(self._lib.infllm_score_topk(self.reps[u].data_ptr(), self.reps.stride(1), N, C, qbar[u, j].data_ptr(),
+                                                      topk, scores.data_ptr(), idx[j, u].data_ptr(), self._main_raw),
+                          "infllm_score_topk")
+            else:
+                check(rc, "infllm_score_topk_queries")
         return idx.cpu().tolist()
 
     def _grow_reps(self, need):
