@@ -818,6 +818,16 @@ __global__ __launch_bounds__(256) void call_rank_kernel(CallRankJob jb) {
     for (int u = 0; u < jb.B; ++u) {
         const float *qbar = jb.qbars + ((int64_t)j * jb.B + u) * C;
         float *scores = jb.scores + ((int64_t)j * jb.B + u) * jb.cols;
+        // a ranking thread's entry, asked for ahead of the scoring: the base list's units and the units carved earlier
+        // in the call have had their scores since then, so these loads travel beside those of the new units' rows
+        const int n_late = jb.first_new + jb.n_new - jb.n_base;  // units carved since the call began
+        const int n = jb.k + n_late;
+        int my_id = -1;
+        float my_score = 0.f;
+        if ((is_sel || is_cand) && tid < n) {
+            my_id = tid < jb.k ? jb.base[((int64_t)j * jb.B + u) * jb.k + tid] : jb.n_base + (tid - jb.k);
+            if (my_id < jb.first_new) my_score = scores[my_id];
+        }
         if (jb.n_new > 0) {
             float q[CPL][8];
 #pragma unroll
@@ -849,12 +859,9 @@ __global__ __launch_bounds__(256) void call_rank_kernel(CallRankJob jb) {
         }
         if (!is_sel && !is_cand) continue;                       // workgroup-uniform
         __syncthreads();
-        const int n_late = jb.first_new + jb.n_new - jb.n_base;  // units carved since the call began
-        const int n = jb.k + n_late;
         if (tid < n) {
-            const int id = tid < jb.k ? jb.base[((int64_t)j * jb.B + u) * jb.k + tid] : jb.n_base + (tid - jb.k);
-            e_id[tid] = id;
-            e_key[tid] = order_key(id >= jb.first_new ? fresh[id - jb.first_new] : scores[id]);
+            e_id[tid] = my_id;
+            e_key[tid] = order_key(my_id >= jb.first_new ? fresh[my_id - jb.first_new] : my_score);
         }
         __syncthreads();
         if (tid < n) {

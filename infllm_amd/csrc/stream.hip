@@ -121,6 +121,7 @@ struct Layer {
     // device ids (this handle's own allocation) and the unit count they were chosen from (-1: none)
     int32_t *d_cand = nullptr;
     int cand_units = -1;
+    int scored_units = -1;                // block_front scored units [0, scored_units) under the next block's mean query (-1: none)
     // Lists made once per prepared call (infllm_front_args.d_call_scores): for every block of the call the k best of
     // the units that existed when the call began (d_base: [kMaxCallBlocks, B, topk], this handle's allocation) and
     // those units' scores under the block's mean query (the caller's buffer).  While call_lists is set, a block's
@@ -128,6 +129,8 @@ struct Layer {
     int32_t *d_base = nullptr;
     bool call_lists = false, no_call_lists = false;    // INFLLM_NO_CALL_LISTS=1 turns them off
     bool call_lists_pending = false;                   // the call in flight wants them: its first block's second half makes them
+    int call_room = 0;                                 // entries a ranking takes (INFLLM_CALL_LISTS_ROOM lowers it: the rest of
+                                                       // such a call goes back to selections over all units)
     int call_n0 = 0, call_blocks = 0;
     float *call_scores = nullptr;
     int64_t call_cols = 0;
@@ -884,6 +887,9 @@ extern "C" void *infllm_layer_create(const infllm_layer_desc *desc) {
         L->score_merge_apart = ma && ma[0] && ma[0] != '0';
         const char *nl = getenv("INFLLM_NO_CALL_LISTS");
         L->no_call_lists = nl && nl[0] && nl[0] != '0';
+        const char *room = getenv("INFLLM_CALL_LISTS_ROOM");
+        L->call_room = infllm_call_rank_room();
+        if (room && atoi(room) > 0 && atoi(room) < L->call_room) L->call_room = atoi(room);
     }
     if (hipHostMalloc((void **)&L->h_cand, 2 * ((size_t)d.B * d.topk + 1) * sizeof(int32_t)) != hipSuccess) {
         (void)hipGetLastError();
@@ -1159,7 +1165,7 @@ int cand_publication(Layer *L, int64_t for_b0) {
 }
 
 bool call_rank_fits(const Layer *L, int first_new, int n_new) {
-    return n_new <= 64 && L->d.topk + (first_new + n_new - L->call_n0) <= infllm_call_rank_room();
+    return n_new <= 64 && L->d.topk + (first_new + n_new - L->call_n0) <= L->call_room;
 }
 
 // From the lists of the prepared call (Layer::call_lists): the n_new units from first_new on were carved just now;
@@ -1352,7 +1358,8 @@ extern "C" int infllm_call_front(void *layer, const infllm_front_args *a, void *
     const int max_new = (a->n + d.block_size - 1) / d.block_size + 1;
     const int cpl = C % 512 == 0 ? C / 512 : 0;
     if (retrieve && n_blocks > 1 && n_blocks <= kMaxCallBlocks && a->d_call_scores && L->d_base && !L->no_call_lists && d.topk <= 64 &&
-        (cpl == 1 || cpl == 2 || cpl == 4 || cpl == 8) && a->call_scores_cols >= (int64_t)a->n_units + max_new) {
+        (cpl == 1 || cpl == 2 || cpl == 4 || cpl == 8) && a->call_scores_cols >= (int64_t)a->n_units + max_new &&
+        d.topk + max_new <= infllm_call_rank_room() && d.max_carve <= 64) {
         L->call_lists_pending = true;
         L->call_n0 = a->n_units;
         L->call_blocks = n_blocks;
@@ -1416,8 +1423,10 @@ extern "C" int infllm_block_front(void *layer, const infllm_front_args *a, void 
             if (rc) return rc;
         }
         // (with the lists of a prepared call the next block's candidates were ranked when the previous block had
-        //  carved its units, or by infllm_call_front: nothing to do here)
+        //  carved its units: nothing to do here)
+        L->scored_units = -1;
         if (a->n_units > 0 && !(a->flags & INFLLM_NO_RETRIEVAL) && !(L->call_lists && next_batched)) {
+            L->scored_units = a->n_units;
             INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_front: null representative / score buffer");
             // The scores of the existing units and their k best now, while the fetch is in flight: the selection after the
             // block then only has to weigh these against the few units carved in between, instead of running over every
@@ -2147,7 +2156,9 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
         if (rc < 0) return rc;
         if (rc == 1) {                  // the two steps on their own
             const bool merge = L->cand_units == a->n_units && d.topk + a->n_carve <= 64;
-            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, a->n_units, a->n_carve, L->fresh.qbar,
+            // (the older units were scored by block_front, unless the call's lists stood in for that)
+            const int first = L->scored_units == a->n_units ? a->n_units : 0;
+            rc = run_unit_scores(L, a->d_reps, a->rep_sb, a->rep_su, a->d_unit_scores, a->unit_scores_sb, first, n_units_next - first, L->fresh.qbar,
                                  stream);
             if (rc) return rc;
             if (merge)

@@ -89,6 +89,15 @@ def test_selections_from_the_lists_of_a_call_are_the_selections_over_all_units(m
         # the switch is read when a layer is created: the first run ranked from the lists, the second never did
         assert a[4]["call_ranked"] > 10 and b[4]["call_ranked"] == 0, (a[4], b[4])
         assert a[3][0] > 10                                          # fetches were started ahead from the lists' candidates
+    # a call whose lists outgrow the ranking kernel half way (forced here: room for the 4 best + 8 units) goes on with
+    # selections over all units, to the same results
+    args = (3000, [1500, 1, 1499], 8, 2, 1e4, 47, 2, SMALL)
+    monkeypatch.setenv("INFLLM_CALL_LISTS_ROOM", "12")
+    c = run(False, *args)
+    monkeypatch.delenv("INFLLM_CALL_LISTS_ROOM")
+    a = run(False, *args)
+    assert torch.equal(a[0], c[0]) and a[1] == c[1] and a[2] == c[2]
+    assert 0 < c[4]["call_ranked"] < a[4]["call_ranked"], (a[4], c[4])
 
 
 def test_score_decay_policy_follows_oracle():
