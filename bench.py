@@ -136,6 +136,24 @@ def hbm_leg(dev, n_units=8192, tables=8, launches=200):
     return retrieval, scoring
 
 
+def call_lists_entry(dev, n_units=8192, tables=8, queries=15, launches=40):
+    """The lists of a prepared call (infllm_score_topk_queries): the scores of n_units representatives under the mean queries
+    of a call's other 15 blocks and the 16 best per query, the representatives read once per eight queries.  Algorithmic
+    bytes: the representatives once (N*H*D*2) plus the queries' score rows written and read by the selection."""
+    from infllm_amd import ops
+    C, k = H * D, KNOBS["topk"]
+    reps = torch.randn((tables, n_units, C), device=dev, dtype=torch.bfloat16)
+    qbars = torch.randn((queries, C), device=dev)
+    scores = torch.empty((queries, n_units), dtype=torch.float32, device=dev)
+    idx = torch.empty((queries, k), dtype=torch.int32, device=dev)
+    us = _event_time_us(lambda i: ops.score_topk_queries(reps[i % tables], n_units, qbars, k, scores, idx), launches, 2 * tables)
+    nbytes = n_units * C * 2 + 2 * queries * n_units * 4
+    return _hbm_entry("unit_scores_queries_kernel<8> + select_rows_kernel<1>",
+                      f"lists of a call: {queries} mean queries over {n_units} x {C} bf16 representatives, top-{k} each, two launches "
+                      f"({tables} tables in rotation; the same by one retrieval per block: {queries} x {n_units * C * 2 / 2 ** 20:.0f} MiB)",
+                      nbytes, us, launches)
+
+
 def kernels_hbm_leg(dev):
     """The other HBM-bound kernels of the path at the shapes the benchmark configurations give them, each timed in this
     run with events over repeated launches; algorithmic bytes as the scope table counts them.  Inputs of more than a
@@ -492,7 +510,7 @@ def main():
         return
     if args.workload == "hbm":
         retrieval, scoring = hbm_leg(dev)
-        print(json.dumps({"roofline_hbm": retrieval, "kernels_hbm": [scoring] + kernels_hbm_leg(dev)}))
+        print(json.dumps({"roofline_hbm": retrieval, "kernels_hbm": [scoring, call_lists_entry(dev)] + kernels_hbm_leg(dev)}))
         return
     T = args.tokens
     q, k, v = make_stream(T, 0, dev, args.favour)
@@ -579,7 +597,7 @@ def main():
         res.update(extra_legs(args, dev))
     if not args.no_hbm_leg:
         res["roofline_hbm"], scoring = hbm_leg(dev)
-        res["kernels_hbm"] = [scoring] + kernels_hbm_leg(dev)
+        res["kernels_hbm"] = [scoring, call_lists_entry(dev)] + kernels_hbm_leg(dev)
     if args.cpu_tokens > 0:
         res["cpu_baseline"] = cpu_baseline(min(args.cpu_tokens, 16384), min(os.cpu_count() or 1, 16))
     print(json.dumps(res))
