@@ -921,53 +921,75 @@ __global__ __launch_bounds__(512) void unit_scores_queries_kernel(const bf16_t *
     extern __shared__ float qs[];                               // [kQueryGroup][C]
     constexpr int C = CPL * 512;
     const int lane = threadIdx.x & 63;
-    const int n_waves = gridDim.x * 8;
-    const int q0 = blockIdx.y * kQueryGroup;
+    // Workgroups go to the 8 XCDs round-robin by their id.  The workgroups that walk the same rows for different
+    // groups of queries get ids 8 apart: they run on the same XCD at about the same time, and all but the first of
+    // them find the rows in that XCD's L2.
+    const int groups = (n_queries + kQueryGroup - 1) / kQueryGroup;
+    const int wgs = gridDim.x / groups;                         // workgroups per group of queries (a multiple of 8)
+    const int slot = blockIdx.x / 8, xcd = blockIdx.x % 8;
+    const int wg = (slot / groups) * 8 + xcd;
+    const int n_waves = wgs * 8;
+    const int q0 = (slot % groups) * kQueryGroup;
     const int nq = min(kQueryGroup, n_queries - q0);
-    int n = blockIdx.x * 8 + (threadIdx.x >> 6);                // rows n, n + n_waves, ... belong to this wave
-    u32x4 w[2][CPL];
-    auto load_rows = [&](int first) {
+    int n = wg * 8 + (threadIdx.x >> 6);                        // rows n, n + n_waves, ... belong to this wave
+    u32x4 w[2][CPL], w_next[2][CPL];
+    auto load_rows = [&](u32x4 (&dst)[2][CPL], int first) {
 #pragma unroll
         for (int r = 0; r < 2; ++r)
             if (first + r * n_waves < N) {
                 const bf16_t *row = reps + (int64_t)(first + r * n_waves) * rep_stride + lane * 8;
 #pragma unroll
-                for (int j = 0; j < CPL; ++j) w[r][j] = *(const u32x4 *)(row + j * 512);
+                for (int j = 0; j < CPL; ++j) dst[r][j] = *(const u32x4 *)(row + j * 512);
             }
     };
-    load_rows(n);
+    load_rows(w, n);
     for (int e = threadIdx.x * 4; e < nq * C; e += 512 * 4)
         *(f32x4 *)(qs + e) = *(const f32x4 *)(qbars + (int64_t)(q0 + e / C) * qbar_qs + e % C);
     __syncthreads();
     while (n < N) {
         const bool two = n + n_waves < N;
-        float res[2][kQueryGroup];
-        for (int q = 0; q < nq; ++q) {
-            const float *qq = qs + q * C;
-            float a00 = 0.f, a01 = 0.f, a10 = 0.f, a11 = 0.f;
+        load_rows(w_next, n + 2 * n_waves);                     // the next two rows travel while these are multiplied
+        // a row's elements are unpacked once and meet every query of the group; per (row, query) the two running sums
+        // take their terms in unit_scores_rows_kernel's order (chunk by chunk, element by element)
+        float acc[2][kQueryGroup][2];
 #pragma unroll
-            for (int j = 0; j < CPL; ++j) {
-                const f32x4 lo = *(const f32x4 *)(qq + j * 512 + lane * 8), hi = *(const f32x4 *)(qq + j * 512 + lane * 8 + 4);
-                const float qv[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        for (int q = 0; q < kQueryGroup; ++q) acc[0][q][0] = acc[0][q][1] = acc[1][q][0] = acc[1][q][1] = 0.f;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    a00 += bf16_bits_to_f32(w[0][j][i] & 0xffffu) * qv[2 * i];
-                    a01 += bf16_bits_to_f32(w[0][j][i] >> 16) * qv[2 * i + 1];
-                    a10 += bf16_bits_to_f32(w[1][j][i] & 0xffffu) * qv[2 * i];
-                    a11 += bf16_bits_to_f32(w[1][j][i] >> 16) * qv[2 * i + 1];
-                }
+        for (int j = 0; j < CPL; ++j) {
+            float lo[2][4], hi[2][4];
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) lo[r][i] = bf16_bits_to_f32(w[r][j][i] & 0xffffu), hi[r][i] = bf16_bits_to_f32(w[r][j][i] >> 16);
+#pragma unroll
+            for (int q = 0; q < kQueryGroup; ++q) {
+                if (q >= nq) break;
+                const float *qq = qs + q * C + j * 512 + lane * 8;
+                const f32x4 q_lo = *(const f32x4 *)qq, q_hi = *(const f32x4 *)(qq + 4);
+                const float qv[8] = {q_lo[0], q_lo[1], q_lo[2], q_lo[3], q_hi[0], q_hi[1], q_hi[2], q_hi[3]};
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[r][q][0] += lo[r][i] * qv[2 * i];
+                        acc[r][q][1] += hi[r][i] * qv[2 * i + 1];
+                    }
             }
-            res[0][q] = wave_sum(a00 + a01);
-            res[1][q] = wave_sum(a10 + a11);
         }
-        if (lane == 0) {
-            for (int q = 0; q < nq; ++q) {
-                scores[(int64_t)(q0 + q) * scores_qs + n] = res[0][q];
-                if (two) scores[(int64_t)(q0 + q) * scores_qs + n + n_waves] = res[1][q];
+#pragma unroll
+        for (int q = 0; q < kQueryGroup; ++q) {
+            if (q >= nq) break;
+            const float s0 = wave_sum(acc[0][q][0] + acc[0][q][1]), s1 = wave_sum(acc[1][q][0] + acc[1][q][1]);
+            if (lane == 0) {
+                scores[(int64_t)(q0 + q) * scores_qs + n] = s0;
+                if (two) scores[(int64_t)(q0 + q) * scores_qs + n + n_waves] = s1;
             }
         }
         n += 2 * n_waves;
-        load_rows(n);
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) w[r][j] = w_next[r][j];
     }
 }
 
@@ -978,7 +1000,7 @@ extern "C" int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride,
     INFLLM_REQUIRE(rep_stride >= C && rep_stride % 8 == 0, "score_topk_queries: row stride %lld", (long long)rep_stride);
     const bf16_t *rows = (const bf16_t *)d_reps;
     const int groups = (n_queries + kQueryGroup - 1) / kQueryGroup;
-    int wgs = (N + 15) / 16;                               // two rows per wave and trip
+    int wgs = ((N + 15) / 16 + 7) / 8 * 8;                 // two rows per wave and trip; a multiple of the 8 XCDs
     if (wgs > 256) wgs = 256;                              // one workgroup per CU: the queries take most of its LDS
     static bool lds_set = false;                           // dynamic LDS above 64 KiB must be enabled once per kernel
     if (!lds_set) {
@@ -988,7 +1010,7 @@ extern "C" int infllm_score_topk_queries(const void *d_reps, int64_t rep_stride,
         lds_set = true;
     }
     switch (C % 512 == 0 ? C / 512 : 0) {
-#define QUERIES_CASE(n) case n: hipLaunchKernelGGL(unit_scores_queries_kernel<n>, dim3(wgs, groups), dim3(512), (size_t)kQueryGroup * n * 512 * sizeof(float), \
+#define QUERIES_CASE(n) case n: hipLaunchKernelGGL(unit_scores_queries_kernel<n>, dim3(wgs * groups), dim3(512), (size_t)kQueryGroup * n * 512 * sizeof(float), \
                                                     (hipStream_t)stream, rows, rep_stride, N, d_qbars, qbar_qs, n_queries, d_scores, scores_qs); break
         QUERIES_CASE(1); QUERIES_CASE(2); QUERIES_CASE(4); QUERIES_CASE(8);
 #undef QUERIES_CASE
