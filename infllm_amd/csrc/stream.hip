@@ -2127,20 +2127,12 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     if (L->prepared && n_units_next > d.topk && !(a->flags & INFLLM_NO_RETRIEVAL)) {
         INFLLM_REQUIRE(a->d_reps && a->d_unit_scores, "block_back: null representative / score buffer");
         // with the lists of a prepared call: the new units' scores for the call's later blocks, the next block's
-        // selection and the candidates of the block after it, one launch
-        if (L->call_lists_pending && batched && a->b0 == L->batch_b0) {
-            // the first block of a prepared call: the lists of its other blocks, two launches for the whole call
-            L->call_lists_pending = false;
-            const int C = d.H * kD;
-            for (int u = 0; u < d.B && a->n_units == L->call_n0; ++u) {
-                rc = infllm_score_topk_queries((const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb, a->rep_su, L->call_n0, C,
-                                               L->bd.d_qbar + ((int64_t)d.B + u) * C, (int64_t)d.B * C, L->call_blocks - 1, d.topk,
-                                               L->call_scores + ((int64_t)d.B + u) * L->call_cols, (int64_t)d.B * L->call_cols,
-                                               L->d_base + ((int64_t)d.B + u) * d.topk, (int64_t)d.B * d.topk, stream);
-                if (rc) return rc < 0 ? rc : infllm_fail(-2, "block_back: no scoring kernel after the geometry check");
-                L->call_lists = u == d.B - 1;
-            }
-        }
+        // selection and the candidates of the block after it, one launch.  (The first block of such a call selects
+        // for the second as a block on its own would, from the candidates block_front chose, and makes the lists
+        // behind that selection: see below.)
+        const bool make_lists = L->call_lists_pending && batched && a->b0 == L->batch_b0 && a->n_units == L->call_n0 &&
+                                call_rank_fits(L, a->n_units, a->n_carve);
+        if (batched && a->b0 == L->batch_b0) L->call_lists_pending = false;
         const int j_next = L->call_lists && batched ? (int)((b1 - L->batch_b0) / d.exc) : -1;
         if (j_next >= 1 && j_next < L->call_blocks && block_in_batch(L, b1, L->prepared_n) && call_rank_fits(L, a->n_units, a->n_carve)) {
             rc = run_call_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->n_units, a->n_carve, j_next, j_next + 1 < L->call_blocks ? j_next + 1 : -1,
@@ -2166,6 +2158,25 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
             else
                 rc = run_topk(L, a->d_unit_scores, a->unit_scores_sb, n_units_next, stream);
             if (rc) return rc;
+        }
+        if (make_lists) {
+            // The lists of the call's other blocks, two launches for the whole call, BEHIND the second block's selection:
+            // the host is busy with that selection and the stream with the wait for its fetch while they are made.
+            // Then the first ranking from them: the units just carved under the later blocks' mean queries, and the
+            // third block's candidates.
+            const int C = d.H * kD;
+            for (int u = 0; u < d.B; ++u) {
+                rc = infllm_score_topk_queries((const bf16_t *)a->d_reps + (int64_t)u * a->rep_sb, a->rep_su, L->call_n0, C,
+                                               L->bd.d_qbar + ((int64_t)d.B + u) * C, (int64_t)d.B * C, L->call_blocks - 1, d.topk,
+                                               L->call_scores + ((int64_t)d.B + u) * L->call_cols, (int64_t)d.B * L->call_cols,
+                                               L->d_base + ((int64_t)d.B + u) * d.topk, (int64_t)d.B * d.topk, stream);
+                if (rc) return rc < 0 ? rc : infllm_fail(-2, "block_back: no scoring kernel after the geometry check");
+            }
+            L->call_lists = true;
+            if (L->call_blocks > 2) {
+                rc = run_call_rank(L, a->d_reps, a->rep_sb, a->rep_su, a->n_units, a->n_carve, -1, 2, stream);
+                if (rc) return rc;
+            }
         }
     }
     L->cand_units = -1;
