@@ -31,7 +31,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 def make_stream(T, seed, device, favour=0):
     """q, v ~ N(0,1); keys from a 64-component Gaussian mixture per kv head (means N(0,1), std 0.3).
-    favour > 0 (BASELINE config 5): the queries of an execution block lean towards `favour` mixture components
+    favour > 0 (benchmark configuration 5): the queries of an execution block lean towards `favour` mixture components
     drawn per block (q = that component's mean + N(0,1)), so consecutive blocks retrieve different units."""
     g = torch.Generator(device=device).manual_seed(seed)
     means = torch.randn((HKV, 64, D), generator=g, device=device)
@@ -111,7 +111,7 @@ def _hbm_entry(kernel, what, nbytes, us, launches, **extra):
 
 def hbm_leg(dev, n_units=8192, tables=8, launches=200):
     """The HBM half of the metric, measured in this run: a RETRIEVAL (context_manager.py:159-163: unit scores, then
-    their top-k) over n_units representatives of H*D bf16 each, the shape of BASELINE config 3, as ONE launch -
+    their top-k) over n_units representatives of H*D bf16 each, the shape of benchmark configuration 3, as ONE launch -
     N*H*D*2 algorithmic bytes (64 MiB), read once (the selection re-reads the N fp32 scores: 32 KiB).  The launches
     rotate over `tables` distinct tables (512 MiB together, more than the 256 MB of last-level cache), so every launch
     reads from HBM; the figure is the MEAN over all launches, timed with events on the stream the kernel runs on.
@@ -235,7 +235,7 @@ def kernels_hbm_leg(dev):
 
 
 def make_decode_state(dev, n_units, seed=3):
-    """A prepared memory for the decode shape (BASELINE config 3): n_units units of mixture keys with representatives
+    """A prepared memory for the decode shape (benchmark configuration 3): n_units units of mixture keys with representatives
     (the mean of each unit's first repr_topk keys), a full local window and the init tokens.  Returns the state
     ContextManager.load_state takes, and a function drawing further (q, k, v) tokens from the same generator."""
     bs, n_local, n_init = KNOBS["block_size"], KNOBS["n_local"], KNOBS["n_init"]
@@ -269,7 +269,7 @@ def make_decode_state(dev, n_units, seed=3):
 
 
 def decode_workload(args, dev):
-    """BASELINE config 3: 256 single-token steps over a prepared memory of 8192 units (1,048,576 past tokens)
+    """benchmark configuration 3: 256 single-token steps over a prepared memory of 8192 units (1,048,576 past tokens)
     with precomputed representatives.  Prints its own JSON line; not the headline metric."""
     from infllm_amd import ops
     from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
@@ -318,7 +318,7 @@ def decode_workload(args, dev):
 
 
 def model_workload(args, dev):
-    """BASELINE config 4: a 32-layer decoder with the Llama-3-8B architecture and random weights, every attention
+    """benchmark configuration 4: a 32-layer decoder with the Llama-3-8B architecture and random weights, every attention
     routed through the "inf-llm" type; chunked prefill (all but the last token in pieces of 8192, then the last
     token) followed by greedy decode steps, driven by GreedySearch.  Prints its own JSON line; not the headline."""
     import transformers
@@ -375,8 +375,8 @@ def model_workload(args, dev):
 
 def extra_legs(args, dev):
     """The other single-layer configurations, timed in this run so that their figures come with the headline:
-    the same 131,072-token stream with every unit resident (nothing crosses PCIe: the kernels' own time), BASELINE
-    config 3 (single-token steps over 8,192 prepared units) and config 5 (one 1,048,576-token stream whose queries
+    the same 131,072-token stream with every unit resident (nothing crosses PCIe: the kernels' own time), benchmark
+    configuration 3 (single-token steps over 8,192 prepared units) and config 5 (one 1,048,576-token stream whose queries
     favour two mixture components per block)."""
     from infllm_amd.attention import ContextManager, RotaryEmbeddingESM
     legs = {}
@@ -443,7 +443,7 @@ def extra_legs(args, dev):
 
 
 def cpu_baseline(tokens, threads, seed=1):
-    """BASELINE config 1: the reference's torch path restated (the fp32 oracle; the reference's own files hard-code
+    """benchmark configuration 1: the reference's torch path restated (the fp32 oracle; the reference's own files hard-code
     "cuda") on the host cores - q, k, v i.i.d. N(0,1) from `seed`, fp32, the first `tokens` tokens of the
     16,384-token stream (all of it by default)."""
     from oracle.rope import RopeOracle

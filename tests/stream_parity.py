@@ -15,7 +15,7 @@ Acceptance rules (written here once, used by every stream test):
   N(0,1) and mixture keys) plus the 2,880 picks of the two-layer Llama-3-8B-shaped model 1.5 % of the picks differ at
   all, 15 of them by more than 1e-3, the largest gaps being 1.19e-3 (mixture keys), 1.40e-3 (N(0,1) keys), 2.05e-3
   (small geometry) and 2.09e-3 (model activations); such streams are held to UNFAVOURED_GAP = 4e-3, twice the
-  largest.  BASELINE config 5 is the wide one: its queries lean towards two mixture components per block, so a token's
+  largest.  benchmark configuration 5 is the wide one: its queries lean towards two mixture components per block, so a token's
   mass comes from a handful of near-one probabilities - 19 of 2,560 picks differ, 14 by more than 1e-3, five beyond
   4e-3, the largest 6.29e-3 (the same with the score kernel of either form, bit for bit); it is held to the full 1e-2.
   How often a pick differs at all, and by more than 1e-3, is counted (Follower.stats), bounded for every stream by

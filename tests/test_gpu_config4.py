@@ -1,4 +1,4 @@
-"""BASELINE config 4 at its own geometry: a decoder with the Llama-3-8B architecture (hidden 4096, 32 query / 8 kv
+"""benchmark configuration 4 at its own geometry: a decoder with the Llama-3-8B architecture (hidden 4096, 32 query / 8 kv
 heads, head_dim 128, FFN 14336 SwiGLU, RoPE base 500000, vocabulary 128,256, random weights, bf16), every attention
 routed through the "inf-llm" type with the reference's knobs, driven by GreedySearch with chunk_size 8192
 (inf_llm/utils/greedy_search.py:52-70).

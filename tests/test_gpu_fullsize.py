@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their full sizes on the GPU.
+"""The five benchmark configurations at their full sizes on the GPU.
 
 A whole 131,072-token (let alone 1,048,576-token) stream is too long for the CPU oracle, so the long streams are
 checked through (i) the closed forms of the state machine, (ii) byte-exact host copies of carved units, and (iii) the
@@ -50,7 +50,7 @@ def stream_128k():
 
 
 def test_config2_last_twenty_blocks_resume_in_the_oracle(stream_128k):
-    """BASELINE config 2 (131,072 tokens, bf16, mixture keys): closed forms of the state at the snapshot and at the
+    """benchmark configuration 2 (131,072 tokens, bf16, mixture keys): closed forms of the state at the snapshot and at the
     end, then the last 20 execution blocks on both sides from the exported state."""
     q, k, v, qd, kd, vd = stream_128k
     T, base = 131072, 1e6
@@ -115,7 +115,7 @@ def test_config2_stream_is_the_same_with_and_without_the_fetch_ahead(stream_128k
 
 
 def test_config1_literal_stream_follows_the_oracle():
-    """BASELINE config 1's workload on the HIP path: 16,384 tokens, q / k / v i.i.d. N(0,1) (rounded to bf16 once, the
+    """benchmark configuration 1's workload on the HIP path: 16,384 tokens, q / k / v i.i.d. N(0,1) (rounded to bf16 once, the
     oracle consumes the same values in fp32), the whole stream on both sides.  With unstructured keys the unit scores
     crowd together, which is where the selection tie rule is exercised hardest."""
     T = 16384
@@ -126,7 +126,7 @@ def test_config1_literal_stream_follows_the_oracle():
 
 
 def test_config3_decode_steps_over_8192_units_follow_the_oracle():
-    """BASELINE config 3: a prepared memory of 8,192 units (1,048,576 past tokens) with representatives, then
+    """benchmark configuration 3: a prepared memory of 8,192 units (1,048,576 past tokens) with representatives, then
     single-token steps.  Six steps are recomputed by the oracle from the same state: top-16 by brute force over all
     8,192 representatives, the fetch of the chosen units from pinned host memory, and the attention of one query."""
     import bench
@@ -156,7 +156,7 @@ def test_config3_decode_steps_over_8192_units_follow_the_oracle():
 
 
 def test_config5_million_token_stream_with_favoured_queries():
-    """BASELINE config 5: a 1,048,576-token stream whose queries lean towards 2 mixture components per execution
+    """benchmark configuration 5: a 1,048,576-token stream whose queries lean towards 2 mixture components per execution
     block, max_cached_block 32, lru; evicted units live in pinned host memory and come back through the DMA engines.
     Closed forms (8,159 units), sampled host units byte for byte, hits and misses both present, and the last 20
     blocks - at positions around 10^6 - on both sides from the exported state."""
