@@ -475,6 +475,13 @@ int infllm_block_fetch(void *layer, int32_t n_miss, const int32_t *h_miss_row, c
 int infllm_block_back(void *layer, const infllm_back_args *a, void *stream, void *copy_stream);
 
 int infllm_layer_flush(void *layer, void *copy_stream);
+/* The end of an append() call without the wait: what infllm_layer_flush does, except that the copy of the units the
+ * last blocks carved to their pinned home (MemoryUnit.cpu_data, context_manager.py:39-45) is left to go on in the
+ * background, as it does between the blocks of a call - the next call's blocks, or a later infllm_layer_flush, see
+ * it through (a unit that is selected before its copy has landed is served from its staging slot as ever).  For a
+ * caller that does not read the pinned copies between calls: the host then goes straight on to the next call instead
+ * of waiting 50-120 us for the copy engine.  infllm_layer_flush before reading pinned units or freeing them. */
+int infllm_layer_end_call(void *layer, void *copy_stream);
 
 /* ---- residency policy of the device unit cache, one object per batch row (context_manager.py:246-265 for the
  * values, 495-515 for the eviction): lru = clock of the last use, fifo = clock of the first load, lru-s = decayed

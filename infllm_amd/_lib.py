@@ -168,6 +168,7 @@ SYMBOLS = {
     "infllm_block_fetch": (c_i32, [c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]),
     "infllm_block_back": (c_i32, [c_vp, C.POINTER(BackArgs), c_vp, c_vp]),
     "infllm_layer_flush": (c_i32, [c_vp, c_vp]),
+    "infllm_layer_end_call": (c_i32, [c_vp, c_vp]),
     "infllm_cache_create": (c_vp, [c_i32, c_i32, c_f64]),
     "infllm_cache_destroy": (c_i32, [c_vp]),
     "infllm_cache_touch": (c_i32, [c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp]),

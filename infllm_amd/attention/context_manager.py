@@ -154,6 +154,7 @@ class ContextManager:
         self.record_trace = False
         self.trace_blocks, self.trace_units = [], []
         self._call_scores = None      # [blocks of a call, B, units]: scores of every unit under every block's mean query
+        self._host_copies_open = False
         self.stats = dict(blocks=0, hits=0, misses=0, evictions=0)
         self._layer = None
         self._timing_cap, self._timing_stride = 0, 1
@@ -368,9 +369,17 @@ class ContextManager:
         chunk, idx = divmod(unit, _HOST_CHUNK_UNITS)
         return self.host_chunks[chunk][idx]
 
+    def _finish_host_copies(self):
+        """append() leaves the copy of the units it carved last to their pinned home in flight; this sees it through."""
+        if self._host_copies_open and self._layer:
+            check(self._lib.infllm_layer_flush(self._layer, self._copy_raw), "infllm_layer_flush")
+            torch.cuda.synchronize(self.device)            # (the copy-stream form of that copy is only ordered by its stream)
+            self._host_copies_open = False
+
     def host_unit(self, unit):
         """Pinned host tensor [B, 2, Hkv, bs, D] of a carved unit (K at index 0, V at 1); for heads narrower than 128 a
         copy with the real dimensions picked out."""
+        self._finish_host_copies()
         return _narrow(self._host_unit_rows(unit), self.dim_head)
 
     def rep_rows(self, row, lo, hi):
@@ -694,7 +703,9 @@ class ContextManager:
                 plan_pos += 1
             self._block(st, n, out_ptr + st * out_step, min(exc, call_end - st - n), chosen)
         self.length += input_length
-        check(self._lib.infllm_layer_flush(self._layer, self._copy_raw), "infllm_layer_flush")
+        # (the last carved units go on to their pinned home in the background: _finish_host_copies before reading them)
+        check(self._lib.infllm_layer_end_call(self._layer, self._copy_raw), "infllm_layer_end_call")
+        self._host_copies_open = True
         out = _narrow(out, self.dim_head)
         if self.perhead:
             out = out.view(batch_size, heads, input_length, -1)
@@ -706,6 +717,7 @@ class ContextManager:
     def export_state(self, with_units=True):
         """Snapshot after an append(): everything a fresh ContextManager needs to continue the stream.
         with_units=False leaves the units out (4 GiB at a million tokens): host_unit(u) still reads them in place."""
+        self._finish_host_copies()
         torch.cuda.synchronize()
         T, cur, cap = self.length, self.cursor, self.ring_cap
         rows = torch.arange(cur, T, device=self.device) % cap

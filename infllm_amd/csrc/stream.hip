@@ -2224,9 +2224,22 @@ extern "C" int infllm_block_back(void *layer, const infllm_back_args *a, void *s
     return 0;
 }
 
+namespace {
+int end_of_call(Layer *L, void *copy_stream, bool finish_copies);
+}
+
 extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
     INFLLM_REQUIRE(layer, "layer_flush: null layer");
-    Layer *L = (Layer *)layer;
+    return end_of_call((Layer *)layer, copy_stream, true);
+}
+
+extern "C" int infllm_layer_end_call(void *layer, void *copy_stream) {
+    INFLLM_REQUIRE(layer, "layer_end_call: null layer");
+    return end_of_call((Layer *)layer, copy_stream, false);
+}
+
+namespace {
+int end_of_call(Layer *L, void *copy_stream, bool finish_copies) {
     if (L->ahead.active) {                      // a guess nobody settled: put back what it overwrote
         L->ahead.active = false;
         hipStream_t cs = (hipStream_t)copy_stream;
@@ -2240,7 +2253,7 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
         HIP_OK(hipStreamSynchronize(cs), "layer_flush: repair");
         L->fetch_wait = L->efetch_wait = false;
     }
-    if (L->off.pending) {
+    if (L->off.pending && finish_copies) {
         int drc = issue_offload_dma(L);
         if (drc < 0) return drc;
         if (drc == 0) {
@@ -2248,7 +2261,7 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
             if (drc) return drc;
         }
     }
-    for (size_t s = 0; s < L->dma_busy.size(); ++s) {       // engine copies are not ordered by any stream: finish them here
+    for (size_t s = 0; s < L->dma_busy.size() && finish_copies; ++s) {       // engine copies are not ordered by any stream: finish them here
         const int wrc = dma_wait_slot(L, (int)s, "layer_flush");
         if (wrc) return wrc;
     }
@@ -2261,3 +2274,4 @@ extern "C" int infllm_layer_flush(void *layer, void *copy_stream) {
     }
     return 0;
 }
+}  // namespace
