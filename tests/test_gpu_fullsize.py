@@ -81,7 +81,8 @@ def test_config2_stream_is_the_same_with_and_without_the_fetch_ahead(stream_128k
     """Config 2 at full size with 32 slots for 16 selected units of 512 KiB each: the stream with the fetch ahead of the
     selection (DMA engines, most guesses confirmed, the others repaired) against the stream without it - outputs bit for
     bit, hit / miss / eviction counts, the eviction sequence, the final residency, and the units' pinned host copies
-    against the input."""
+    against the input.  Then against the stream whose selections run over all units instead of being ranked from the
+    lists of their call: the same again, guesses included."""
     from infllm_amd.attention import ContextManager
     q, k, v, qd, kd, vd = stream_128k
     T = 131072
@@ -89,8 +90,12 @@ def test_config2_stream_is_the_same_with_and_without_the_fetch_ahead(stream_128k
     monkeypatch.delenv("INFLLM_NO_STAGING_COPY", raising=False)
     monkeypatch.setenv("INFLLM_FETCH_AHEAD_ALWAYS", "1")          # ... and guesses also where it cannot
 
-    def run(ahead):
+    def run(ahead, lists=True):
         monkeypatch.setattr(ContextManager, "fetch_ahead", ahead)
+        if lists:
+            monkeypatch.delenv("INFLLM_NO_CALL_LISTS", raising=False)
+        else:
+            monkeypatch.setenv("INFLLM_NO_CALL_LISTS", "1")
         cm = new_manager(1e6, async_global_stream=True, **REFERENCE)
         outs = []
         for i, st in enumerate(range(0, T, 8192)):
@@ -112,6 +117,11 @@ def test_config2_stream_is_the_same_with_and_without_the_fetch_ahead(stream_128k
     for u in range(0, cm1.num_global_block, 41):
         lo, hu = N_INIT + u * BS, cm1.host_unit(u)
         assert torch.equal(hu[0, 0], k[0, :, lo:lo + BS]) and torch.equal(hu[0, 1], v[0, :, lo:lo + BS]), u
+    # ... and the same stream with every block's selection over all units instead of ranked from its call's lists
+    every, cm2 = run(True, lists=False)
+    assert cm1.path_counts()["call_ranked"] > 200 and cm2.path_counts()["call_ranked"] == 0
+    assert torch.equal(every, ahead) and cm2.stats == cm1.stats and cm2.prefetch_stats() == cm1.prefetch_stats()
+    assert cm2.policy[0].evicted_log == cm1.policy[0].evicted_log and cm2.policy[0].cached == cm1.policy[0].cached
 
 
 def test_config1_literal_stream_follows_the_oracle():
