@@ -422,7 +422,7 @@ int infllm_block_front(void *layer, const infllm_front_args *a, void *stream);
  *                           ever, in order; block_front finds their prologue done (its d_q / d_k / d_v and
  *                           next-block pointers are not read, n_next still says whether a block of this call
  *                           follows) and launches the local stage for group_blocks blocks at a time, at the first
- *                           block of each group.  infllm_layer_flush ends the call.
+ *                           block of each group.  infllm_layer_end_call (or infllm_layer_flush) ends the call.
  * Without these two calls every block runs its own prologue and local stage (block_front). */
 typedef struct {
     void *d_q_loc, *d_q_glb;          /* [B, H, max_tokens, 128] bf16 each */
